@@ -1,0 +1,210 @@
+"""Writes the golden fixtures in this directory from the reference implementation.
+
+Run once, in the build container only (the reference never leaves it):
+
+    python tests/golden/make_golden.py [/root/reference]
+
+The reference imports ``opt_einsum_fx`` at module scope; that package only re-orders
+einsum contractions (no arithmetic of its own) and is not installed here, so an
+in-memory module with identity ``jitable`` / ``optimize_einsums_full`` is registered
+before the import.  Everything is evaluated in float64.  The fixtures hold inputs and
+expected outputs only:
+
+* w3j.npz          wigner_3j(l1, l2, l3) for every valid triple with l <= 4
+* sh.npz           spherical_harmonics on 24 fixed points, l <= 8, all option combinations
+* tp_cases.json    instruction tables (path weights, shapes, weight_numel, sorted output
+                   irreps, output_mask) incl. the five benchmark configurations
+* tp_cases.npz     seeded inputs and outputs of small TensorProducts and of
+                   gather -> TensorProduct -> scatter
+"""
+import json
+import os
+import sys
+import types
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def import_reference(path):
+    stub = types.ModuleType("opt_einsum_fx")
+    stub.jitable = lambda m: m
+    stub.optimize_einsums_full = lambda m, example_inputs: m
+    sys.modules["opt_einsum_fx"] = stub
+    sys.path.insert(0, path)
+    torch.set_default_dtype(torch.float64)
+    import e3nn  # noqa: F401
+    from e3nn import o3
+
+    return o3
+
+
+def conv_builder(o3, irreps_in, irreps_edge, keep):
+    # call-site instruction builder, as the reference model code does it
+    irreps_in, irreps_edge = o3.Irreps(irreps_in), o3.Irreps(irreps_edge)
+    keep = [o3.Irrep(k) for k in keep]
+    mid, ins = [], []
+    for i, (mul, ir_in) in enumerate(irreps_in):
+        for j, (_, ir_edge) in enumerate(irreps_edge):
+            for ir_out in ir_in * ir_edge:
+                if ir_out in keep:
+                    ins.append((i, j, len(mid), "uvu", True))
+                    mid.append((mul, ir_out))
+    mid = o3.Irreps(mid)
+    mid, p, _ = mid.sort()
+    return mid, [(a, b, p[c], m, t) for a, b, c, m, t in ins]
+
+
+def merged_uvu(o3, irreps_in, irreps_edge, irreps_out):
+    irreps_in, irreps_edge, irreps_out = o3.Irreps(irreps_in), o3.Irreps(irreps_edge), o3.Irreps(irreps_out)
+    return [
+        (i, j, k, "uvu", True)
+        for i, (_, a) in enumerate(irreps_in)
+        for j, (_, b) in enumerate(irreps_edge)
+        for k, (_, c) in enumerate(irreps_out)
+        if c in a * b
+    ]
+
+
+def describe(tp):
+    return {
+        "irreps_in1": str(tp.irreps_in1),
+        "irreps_in2": str(tp.irreps_in2),
+        "irreps_out": str(tp.irreps_out),
+        "instructions": [
+            [t.i_in1, t.i_in2, t.i_out, t.connection_mode, bool(t.has_weight), float(t.path_weight), list(t.path_shape)]
+            for t in tp.instructions
+        ],
+        "weight_numel": int(tp.weight_numel),
+        "shared_weights": bool(tp.shared_weights),
+        "internal_weights": bool(tp.internal_weights),
+        # one flag per output irrep block (the mask is constant inside a block)
+        "output_mask_blocks": [int(tp.output_mask[s.start]) if s.stop > s.start else -1 for s in tp.irreps_out.slices()],
+    }
+
+
+def main():
+    ref = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+    o3 = import_reference(ref)
+    g = torch.Generator().manual_seed(0)
+
+    # ---- wigner 3j ---------------------------------------------------------------
+    w3j = {}
+    for l1 in range(5):
+        for l2 in range(5):
+            for l3 in range(abs(l1 - l2), min(4, l1 + l2) + 1):
+                w3j[f"{l1}_{l2}_{l3}"] = o3.wigner_3j(l1, l2, l3).numpy()
+    np.savez_compressed(os.path.join(HERE, "w3j.npz"), **w3j)
+
+    # ---- spherical harmonics -----------------------------------------------------
+    pts = torch.randn(20, 3, generator=g)
+    pts = torch.cat([pts, torch.zeros(1, 3), torch.tensor([[0.0, 1.0, 0.0], [1e-20, 0.0, 0.0], [3.0, -4.0, 12.0]])])
+    sh = {"points": pts.numpy()}
+    for normalize in (True, False):
+        for normalization in ("integral", "component", "norm"):
+            out = o3.spherical_harmonics(list(range(9)), pts, normalize, normalization)
+            sh[f"lmax8_{int(normalize)}_{normalization}"] = out.numpy()
+    sh["ls_2_0_3_1_component"] = o3.spherical_harmonics([2, 0, 3], pts, True, "component").numpy()
+    np.savez_compressed(os.path.join(HERE, "sh.npz"), **sh)
+
+    # ---- tensor products ---------------------------------------------------------
+    meta, arrays = {}, {}
+
+    def add_case(name, tp, Z, extra=None, run=True):
+        d = describe(tp)
+        if extra:
+            d.update(extra)
+        meta[name] = d
+        if not run:
+            return
+        x1 = torch.randn(Z, tp.irreps_in1.dim, generator=g)
+        x2 = torch.randn(Z, tp.irreps_in2.dim, generator=g)
+        if tp.weight_numel and not tp.internal_weights:
+            w = torch.randn(*(() if tp.shared_weights else (Z,)), tp.weight_numel, generator=g)
+            out = tp(x1, x2, w)
+        elif tp.weight_numel:
+            w = tp.weight.detach().clone()
+            out = tp(x1, x2)
+        else:
+            w = torch.zeros(0)
+            out = tp(x1, x2)
+        arrays[name + "/x1"], arrays[name + "/x2"] = x1.numpy(), x2.numpy()
+        arrays[name + "/w"], arrays[name + "/out"] = w.numpy(), out.detach().numpy()
+
+    # configuration 1 (rows of it), and the structure of configuration 5
+    tp = o3.FullyConnectedTensorProduct("16x0e+16x1o", "0e+1o+2e", "16x0e+16x1o+16x2e")
+    add_case("fctp_cfg1", tp, 16)
+    tp = o3.FullyConnectedTensorProduct("128x0e+128x1o+128x2e", "128x0e+128x1o+128x2e", "128x0e+128x1o+128x2e")
+    add_case("fctp_cfg5_structure", tp, 0, run=False)
+    tp = o3.FullyConnectedTensorProduct("3x0e+3x1o+3x2e", "3x0e+3x1o+3x2e", "3x0e+3x1o+3x2e")
+    add_case("fctp_small_cfg5_like", tp, 5)
+    tp = o3.FullyConnectedTensorProduct("2x0e+3x1o", "2x0e+1x1o+1x1e", "2x0e+2x1o+3x1e+1x2e", shared_weights=False)
+    add_case("fctp_per_sample_weights", tp, 6)
+    tp = o3.FullyConnectedTensorProduct("4x0e+2x1o+1x2e", "0e+1o", "3x0e+5x1o", irrep_normalization="norm", path_normalization="path")
+    add_case("fctp_norm_path", tp, 4)
+
+    # configuration 3: merged outputs, and the call-site builder with sorted per-path blocks
+    sh2, sh3 = str(o3.Irreps.spherical_harmonics(2)), str(o3.Irreps.spherical_harmonics(3))
+    for mul, tag, run in ((32, "cfg3_structure", False), (4, "cfg3_like_mul4", True)):
+        feats = f"{mul}x0e+{mul}x1o+{mul}x2e"
+        tp = o3.TensorProduct(feats, sh2, feats, merged_uvu(o3, feats, sh2, feats), internal_weights=False, shared_weights=False)
+        add_case("uvu_merged_" + tag, tp, 7, run=run)
+        mid, ins = conv_builder(o3, feats, sh2, ["0e", "1o", "2e"])
+        tp = o3.TensorProduct(feats, sh2, mid, ins, internal_weights=False, shared_weights=False)
+        add_case("uvu_builder_" + tag, tp, 7, run=run)
+    # configuration 4: MACE-scale, targets 0e 1o 2e 3o (A) and every l <= 3 of both parities (B)
+    for mul, tag, run in ((128, "cfg4_structure", False), (2, "cfg4_like_mul2", True)):
+        feats = f"{mul}x0e+{mul}x1o+{mul}x2e+{mul}x3o"
+        mid, ins = conv_builder(o3, feats, sh3, ["0e", "1o", "2e", "3o"])
+        tp = o3.TensorProduct(feats, sh3, mid, ins, internal_weights=False, shared_weights=False)
+        add_case("uvu_builderA_" + tag, tp, 5, run=run)
+        mid, ins = conv_builder(o3, feats, sh3, ["0e", "0o", "1e", "1o", "2e", "2o", "3e", "3o"])
+        tp = o3.TensorProduct(feats, sh3, mid, ins, internal_weights=False, shared_weights=False)
+        add_case("uvu_builderB_" + tag, tp, 5, run=run)
+
+    # uvu with in2 multiplicity > 1 and shared weights; unweighted uvu
+    tp = o3.TensorProduct("3x0e+3x1o", "2x0e+2x1o", "3x0e+3x1o", [(0, 0, 0, "uvu", True), (0, 1, 1, "uvu", True), (1, 0, 1, "uvu", True), (1, 1, 0, "uvu", True)])
+    add_case("uvu_shared_v2", tp, 5)
+    tp = o3.TensorProduct("3x1o", "2x1o", "3x1e+3x2e", [(0, 0, 0, "uvu", False), (0, 0, 1, "uvu", True, 2.5)], internal_weights=False, shared_weights=True)
+    add_case("uvu_mixed_weightless", tp, 5, extra={"user_path_weights": [1.0, 2.5]})
+    # the other connection modes
+    tp = o3.TensorProduct("3x1o+3x2e", "3x1o+3x0e", "3x1e+3x2e+9x1o+2x2o+3x1o", [
+        (0, 0, 0, "uuu", True), (1, 1, 1, "uuu", False), (0, 1, 2, "uvuv", True), (1, 0, 3, "uuw", True), (0, 1, 4, "uvv", True)])
+    add_case("modes_uuu_uvuv_uuw_uvv", tp, 4)
+    tp = o3.TensorProduct("4x1o", "4x1o", "6x1e+3x2e", [(0, 0, 0, "uvu<v", True), (0, 0, 1, "u<vw", True)])
+    add_case("modes_triangular", tp, 4)
+    tp = o3.TensorProduct("2x0e+0x1o", "1o", "2x1o+3x2e", [(0, 0, 0, "uvu", True), (1, 0, 1, "uvw", True)])
+    add_case("empty_path_and_missing_output", tp, 3)
+
+    # gather -> TP -> scatter, with the reference's scatter()
+    feats = "4x0e+4x1o+4x2e"
+    mid, ins = conv_builder(o3, feats, sh2, ["0e", "1o", "2e"])
+    tp = o3.TensorProduct(feats, sh2, mid, ins, internal_weights=False, shared_weights=False)
+    N, E = 6, 17
+    node_x = torch.randn(N, tp.irreps_in1.dim, generator=g)
+    vec = torch.randn(E, 3, generator=g)
+    attr = o3.spherical_harmonics(list(range(3)), vec, True, "component")
+    w = torch.randn(E, tp.weight_numel, generator=g)
+    src = torch.randint(0, N, (E,), generator=g)
+    dst = torch.randint(0, N - 1, (E,), generator=g)  # node N-1 receives nothing
+    msg = tp(node_x[src], attr, w)
+    out = msg.new_zeros(N, msg.shape[1]).scatter_add_(0, dst.reshape(-1, 1).expand_as(msg), msg)
+    meta["conv_small"] = describe(tp)
+    for k, v in dict(node_x=node_x, vec=vec, attr=attr, w=w, src=src, dst=dst, out=out).items():
+        arrays["conv_small/" + k] = v.numpy()
+
+    meta["sort"] = {}
+    for s in ("2o+1e+0e+1e", "1e+0e+1e", "4x0e+4x1o+4x2e+4x1o+4x0e+4x2o+1x0o"):
+        r = o3.Irreps(s).sort()
+        meta["sort"][s] = {"irreps": str(r.irreps), "p": list(r.p), "inv": list(r.inv)}
+
+    np.savez_compressed(os.path.join(HERE, "tp_cases.npz"), **arrays)
+    with open(os.path.join(HERE, "tp_cases.json"), "w") as f:
+        json.dump(meta, f, separators=(",", ":"))
+    print("wrote", sorted(os.listdir(HERE)))
+
+
+if __name__ == "__main__":
+    main()
