@@ -1,0 +1,196 @@
+// Edge-list preprocessing for the fused scatter (gfx950): range checks of the edge
+// indices and a stable sort of edge ids by destination, giving CSR row pointers.
+//
+// The reference adds messages with scatter_add_ (e3nn/nn/models/v2106/points_convolution.py:13-17);
+// grouping the edges of one destination lets one wavefront sum them in registers and
+// write each output row exactly once.  The sort is integer-only and stable, so the
+// permutation (and therefore the summation order) is unique for a given edge list.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include <rocprim/rocprim.hpp>
+
+#include "e3x_internal.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+
+__device__ int d_flag[4];  // range-check result of e3x_index_check (one copy per device)
+
+template <typename IdxT>
+__global__ __launch_bounds__(kBlock) void keys_kernel(const IdxT* __restrict__ dst, long long E, long long N,
+                                                      unsigned* __restrict__ keys, int* __restrict__ ids,
+                                                      int* __restrict__ flags) {
+  bool bad = false;
+  for (long long e = (long long)blockIdx.x * kBlock + threadIdx.x; e < E; e += (long long)gridDim.x * kBlock) {
+    const long long d = (long long)dst[e];
+    if (d < 0 || d >= N) bad = true;
+    keys[e] = (unsigned)d;
+    ids[e] = (int)e;
+  }
+  if (bad) atomicOr(&flags[0], 1);
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(kBlock) void range_kernel(const IdxT* __restrict__ idx, long long E, long long N,
+                                                       int* __restrict__ flags) {
+  bool bad = false;
+  for (long long e = (long long)blockIdx.x * kBlock + threadIdx.x; e < E; e += (long long)gridDim.x * kBlock) {
+    const long long d = (long long)idx[e];
+    if (d < -N || d >= N) bad = true;
+  }
+  if (bad) atomicOr(&flags[0], 1);
+}
+
+// rowptr[n] = first position k with sorted_key[k] >= n   (n = 0..N)
+__global__ __launch_bounds__(kBlock) void rowptr_kernel(const unsigned* __restrict__ sorted, long long E,
+                                                        long long N, int* __restrict__ rowptr) {
+  for (long long n = (long long)blockIdx.x * kBlock + threadIdx.x; n <= N; n += (long long)gridDim.x * kBlock) {
+    long long lo = 0, hi = E;
+    while (lo < hi) {
+      const long long mid = (lo + hi) >> 1;
+      if ((long long)sorted[mid] < n) lo = mid + 1; else hi = mid;
+    }
+    rowptr[n] = (int)lo;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void fill_zero_kernel(int* p, int n) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+__global__ __launch_bounds__(kBlock) void copy16_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                        size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += (size_t)gridDim.x * kBlock) dst[i] = src[i];
+}
+
+__global__ __launch_bounds__(kBlock) void fill_zero_bytes_kernel(unsigned char* p, size_t n) {
+  // 16-byte stores over the aligned middle, byte stores at the ragged ends
+  const size_t head = (16 - ((uintptr_t)p & 15)) & 15;
+  const size_t h = head < n ? head : n;
+  const size_t n16 = (n - h) / 16;
+  const size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x, stride = (size_t)gridDim.x * kBlock;
+  uint4* mid = reinterpret_cast<uint4*>(p + h);
+  for (size_t i = tid; i < n16; i += stride) mid[i] = make_uint4(0, 0, 0, 0);
+  if (tid < h) p[tid] = 0;
+  const size_t tail0 = h + n16 * 16;
+  if (tid < n - tail0) p[tail0 + tid] = 0;
+}
+
+unsigned grid_for(long long n, int per_block) {
+  long long b = (n + per_block - 1) / per_block;
+  if (b < 1) b = 1;
+  if (b > 256 * 16) b = 256 * 16;
+  return (unsigned)b;
+}
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+int key_bits(long long N) {
+  int b = 1;
+  while ((1LL << b) < N) ++b;
+  return b;
+}
+
+size_t sort_temp_bytes(long long E, long long N) {
+  size_t temp = 0;
+  (void)rocprim::radix_sort_pairs(nullptr, temp, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr, (int*)nullptr,
+                            (size_t)E, 0, key_bits(N), (hipStream_t)0);
+  return temp;
+}
+
+}  // namespace
+
+int e3x::fill_zero_bytes(void* p, size_t n_bytes, void* stream) {
+  if (n_bytes == 0) return E3X_OK;
+  hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(grid_for((long long)(n_bytes / 16 + 1), kBlock)), dim3(kBlock), 0,
+                     (hipStream_t)stream, (unsigned char*)p, n_bytes);
+  return hipGetLastError() == hipSuccess ? E3X_OK : e3x::fail(E3X_ERR_HIP, "zero-fill launch failed");
+}
+
+extern "C" size_t e3x_csr_workspace_bytes(int64_t E, int64_t num_nodes) {
+  if (E < 0 || num_nodes < 0) return 0;
+  const size_t e4 = align_up((size_t)E * 4, 256);
+  // flags | keys_in | keys_out | ids_in | rocPRIM temp
+  return 256 + 3 * e4 + align_up(sort_temp_bytes(E > 0 ? E : 1, num_nodes > 1 ? num_nodes : 2), 256);
+}
+
+extern "C" int e3x_csr_build(const void* dst, int idx_bits, int64_t E, int64_t num_nodes, int32_t* rowptr,
+                             int32_t* perm, void* workspace, size_t workspace_bytes, void* stream) {
+  if (E < 0 || num_nodes < 0 || E >= (1LL << 31) || num_nodes >= (1LL << 31))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_csr_build: E and num_nodes must fit in int32");
+  if (idx_bits != 32 && idx_bits != 64) return e3x::fail(E3X_ERR_INVALID, "e3x_csr_build: idx_bits must be 32 or 64");
+  if (!rowptr || (E > 0 && (!dst || !perm || !workspace)))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_csr_build: null pointer");
+  if (workspace_bytes < e3x_csr_workspace_bytes(E, num_nodes))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_csr_build: workspace smaller than e3x_csr_workspace_bytes()");
+  hipStream_t st = (hipStream_t)stream;
+  if (E == 0) {
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(num_nodes + 1, kBlock)), dim3(kBlock), 0, st, rowptr,
+                       (int)(num_nodes + 1));
+    return hipGetLastError() == hipSuccess ? E3X_OK : e3x::fail(E3X_ERR_HIP, "e3x_csr_build: launch failed");
+  }
+  const size_t e4 = align_up((size_t)E * 4, 256);
+  char* ws = (char*)workspace;
+  int* flags = (int*)ws;
+  unsigned* keys_in = (unsigned*)(ws + 256);
+  unsigned* keys_out = (unsigned*)(ws + 256 + e4);
+  int* ids_in = (int*)(ws + 256 + 2 * e4);
+  void* temp = ws + 256 + 3 * e4;
+  size_t temp_bytes = sort_temp_bytes(E, num_nodes > 1 ? num_nodes : 2);
+
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(kBlock), 0, st, flags, 2);
+  if (idx_bits == 64)
+    hipLaunchKernelGGL((keys_kernel<long long>), dim3(grid_for(E, kBlock)), dim3(kBlock), 0, st,
+                       (const long long*)dst, (long long)E, (long long)num_nodes, keys_in, ids_in, flags);
+  else
+    hipLaunchKernelGGL((keys_kernel<int>), dim3(grid_for(E, kBlock)), dim3(kBlock), 0, st, (const int*)dst,
+                       (long long)E, (long long)num_nodes, keys_in, ids_in, flags);
+  // stable LSD radix sort of (dst, edge id) over the significant key bits only
+  hipError_t err = rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, ids_in, perm, (size_t)E, 0,
+                                             key_bits(num_nodes > 1 ? num_nodes : 2), st);
+  if (err != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_csr_build: radix sort failed");
+  hipLaunchKernelGGL(rowptr_kernel, dim3(grid_for(num_nodes + 1, kBlock)), dim3(kBlock), 0, st, keys_out, (long long)E,
+                     (long long)num_nodes, rowptr);
+  int h_flags[2] = {0, 0};
+  if (hipMemcpyAsync(h_flags, flags, sizeof(h_flags), hipMemcpyDeviceToHost, st) != hipSuccess ||
+      hipStreamSynchronize(st) != hipSuccess)
+    return e3x::fail(E3X_ERR_HIP, "e3x_csr_build: reading back the range flags failed");
+  if (h_flags[0]) return e3x::fail(E3X_ERR_INDEX, "index out of range in scatter destination");
+  return E3X_OK;
+}
+
+extern "C" int e3x_index_check(const void* idx, int idx_bits, int64_t E, int64_t num_nodes, void* stream) {
+  if (idx_bits != 32 && idx_bits != 64) return e3x::fail(E3X_ERR_INVALID, "e3x_index_check: idx_bits must be 32 or 64");
+  if (E == 0) return E3X_OK;
+  if (!idx) return e3x::fail(E3X_ERR_INVALID, "e3x_index_check: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  int* flag = nullptr;
+  if (hipGetSymbolAddress((void**)&flag, HIP_SYMBOL(d_flag)) != hipSuccess)
+    return e3x::fail(E3X_ERR_HIP, "e3x_index_check: hipGetSymbolAddress failed");
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(kBlock), 0, st, flag, 1);
+  if (idx_bits == 64)
+    hipLaunchKernelGGL((range_kernel<long long>), dim3(grid_for(E, kBlock)), dim3(kBlock), 0, st,
+                       (const long long*)idx, (long long)E, (long long)num_nodes, flag);
+  else
+    hipLaunchKernelGGL((range_kernel<int>), dim3(grid_for(E, kBlock)), dim3(kBlock), 0, st, (const int*)idx,
+                       (long long)E, (long long)num_nodes, flag);
+  int h = 0;
+  if (hipMemcpyAsync(&h, flag, sizeof(int), hipMemcpyDeviceToHost, st) != hipSuccess ||
+      hipStreamSynchronize(st) != hipSuccess)
+    return e3x::fail(E3X_ERR_HIP, "e3x_index_check: reading back the range flag failed");
+  if (h) return e3x::fail(E3X_ERR_INDEX, "index out of range in gather source");
+  return E3X_OK;
+}
+
+extern "C" int e3x_copy_bytes(const void* src, void* dst, size_t n_bytes, void* stream) {
+  if (n_bytes % 16 || ((uintptr_t)src % 16) || ((uintptr_t)dst % 16))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_copy_bytes: size and pointers must be multiples of 16");
+  if (n_bytes == 0) return E3X_OK;
+  hipLaunchKernelGGL(copy16_kernel, dim3(grid_for((long long)(n_bytes / 16), kBlock * 4)), dim3(kBlock), 0,
+                     (hipStream_t)stream, (const uint4*)src, (uint4*)dst, n_bytes / 16);
+  return hipGetLastError() == hipSuccess ? E3X_OK : e3x::fail(E3X_ERR_HIP, "e3x_copy_bytes: launch failed");
+}

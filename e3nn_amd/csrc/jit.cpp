@@ -1,0 +1,125 @@
+// Kernel specialisation: source assembly, on-disk code-object cache, compiler driver.
+//
+// A specialised kernel = generated constexpr tables (one instruction set) + a fixed
+// hand-written device template.  The code object is compiled once with the system HIP
+// compiler and kept under the cache directory, keyed by a hash of the full source text
+// and the compiler flags, so identical instruction sets never compile twice.
+#include <dlfcn.h>
+#include <fcntl.h>
+#include <spawn.h>
+#include <sys/stat.h>
+#include <sys/wait.h>
+#include <unistd.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+
+#include "e3x_internal.h"
+#include "jit.h"
+
+extern char** environ;
+
+namespace e3x {
+
+static const char* kFlags[] = {"--genco", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+                               "-Xclang", "-packed-fp32-ops", "-ffp-contract=fast", "-Wno-unused-value"};
+
+static uint64_t fnv1a(const std::string& s, uint64_t h = 1469598103934665603ULL) {
+  for (unsigned char c : s) {
+    h ^= c;
+    h *= 1099511628211ULL;
+  }
+  return h;
+}
+
+static bool file_exists(const std::string& p) {
+  struct stat st;
+  return ::stat(p.c_str(), &st) == 0 && st.st_size > 0;
+}
+
+std::string cache_dir() {
+  if (const char* env = std::getenv("E3X_KERNEL_CACHE")) return env;
+  Dl_info info;
+  if (dladdr((void*)&cache_dir, &info) && info.dli_fname) {
+    std::string lib = info.dli_fname;
+    size_t s = lib.rfind('/');
+    std::string dir = s == std::string::npos ? "." : lib.substr(0, s);
+    return dir + "/../kernel_cache";
+  }
+  return "./kernel_cache";
+}
+
+static std::string find_compiler() {
+  if (const char* env = std::getenv("E3X_HIPCC")) return env;
+  if (file_exists("/opt/rocm/bin/hipcc")) return "/opt/rocm/bin/hipcc";
+  return "hipcc";
+}
+
+int get_code_object(const std::string& family, const std::string& source, std::string* key_out,
+                    std::string* path_out) {
+  std::string flags;
+  for (const char* f : kFlags) flags += std::string(f) + " ";
+  const uint64_t h1 = fnv1a(source), h2 = fnv1a(flags + source, 0x9e3779b97f4a7c15ULL);
+  char key[64];
+  std::snprintf(key, sizeof(key), "%s_%016llx%08llx", family.c_str(), (unsigned long long)h1,
+                (unsigned long long)(h2 & 0xffffffffULL));
+  const std::string dir = cache_dir();
+  const std::string base = dir + "/" + key;
+  *key_out = key;
+  *path_out = base + ".hsaco";
+  if (file_exists(*path_out)) return E3X_OK;
+
+  if (const char* nojit = std::getenv("E3X_NO_JIT"))
+    if (nojit[0] == '1')
+      return fail(E3X_ERR_COMPILE, "kernel " + std::string(key) + " is not in the cache (" + dir +
+                                       ") and E3X_NO_JIT=1 forbids compiling it");
+  ::mkdir(dir.c_str(), 0755);
+  const std::string src_path = base + ".hip", log_path = base + ".log";
+  char tmp_name[64];
+  std::snprintf(tmp_name, sizeof(tmp_name), ".tmp%d.hsaco", (int)getpid());
+  const std::string tmp_path = base + tmp_name;
+  {
+    std::ofstream f(src_path);
+    if (!f) return fail(E3X_ERR_COMPILE, "cannot write " + src_path);
+    f << source;
+  }
+  const std::string cc = find_compiler();
+  std::vector<std::string> args = {cc};
+  for (const char* f : kFlags) args.push_back(f);
+  args.push_back("-o");
+  args.push_back(tmp_path);
+  args.push_back(src_path);
+  std::vector<char*> argv;
+  for (auto& a : args) argv.push_back(const_cast<char*>(a.c_str()));
+  argv.push_back(nullptr);
+
+  posix_spawn_file_actions_t fa;
+  posix_spawn_file_actions_init(&fa);
+  posix_spawn_file_actions_addopen(&fa, 1, log_path.c_str(), O_WRONLY | O_CREAT | O_TRUNC, 0644);
+  posix_spawn_file_actions_adddup2(&fa, 1, 2);
+  pid_t pid = 0;
+  int rc = posix_spawnp(&pid, cc.c_str(), &fa, nullptr, argv.data(), environ);
+  posix_spawn_file_actions_destroy(&fa);
+  if (rc != 0) return fail(E3X_ERR_COMPILE, "cannot start the HIP compiler '" + cc + "': " + std::strerror(rc));
+  int status = 0;
+  while (waitpid(pid, &status, 0) < 0) {
+    if (errno != EINTR) return fail(E3X_ERR_COMPILE, "waitpid on the HIP compiler failed");
+  }
+  if (!WIFEXITED(status) || WEXITSTATUS(status) != 0 || !file_exists(tmp_path)) {
+    std::ifstream lf(log_path);
+    std::stringstream ss;
+    ss << lf.rdbuf();
+    std::string log = ss.str();
+    if (log.size() > 2000) log = log.substr(0, 2000) + "...";
+    return fail(E3X_ERR_COMPILE, "compiling " + src_path + " failed:\n" + log);
+  }
+  if (std::rename(tmp_path.c_str(), path_out->c_str()) != 0)
+    return fail(E3X_ERR_COMPILE, "cannot move the code object into the cache");
+  std::remove(log_path.c_str());
+  return E3X_OK;
+}
+
+}  // namespace e3x

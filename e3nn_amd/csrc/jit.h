@@ -1,0 +1,19 @@
+// Kernel specialisation helpers (see jit.cpp).
+#pragma once
+#include <string>
+
+namespace e3x {
+
+// Device template sources, embedded at library build time from templates/*.inc.
+extern const char* const kTplCommon;
+extern const char* const kTplUvu;
+extern const char* const kTplUvwSmall;
+extern const char* const kTplUvwMfma;
+
+std::string cache_dir();
+
+// Returns the path of the code object for `source`, compiling it on a cache miss.
+int get_code_object(const std::string& family, const std::string& source, std::string* key_out,
+                    std::string* path_out);
+
+}  // namespace e3x

@@ -1,0 +1,324 @@
+// Spherical harmonics kernels (gfx950).
+//
+// Fast path, l = 0..LMAX with LMAX <= 3: closed-form polynomials
+// (reference e3nn/o3/_spherical_harmonics.py:194-226).  One wavefront owns a tile of 64
+// vectors: the 768-byte input tile is fetched with 48 dwordx4 loads and redistributed
+// through LDS, every lane evaluates one vector, and the 64 x NC output tile goes back
+// through LDS so that each store instruction writes 1 KiB of consecutive addresses.
+// The kernel is pure streaming: 12 B in + 4 NC B out per vector.
+//
+// Generic path, any list of l <= 12: the recurrence the reference's generator used
+// (e3nn/o3/_spherical_harmonics_generator.py:57-65), driven by a sparse table of
+// wigner_3j(l+1, 1, l) in constant memory; per-lane values live in LDS columns.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <mutex>
+#include <vector>
+
+#include "e3x_internal.h"
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kWavesPerBlock = 4;
+
+// Orders this wavefront's LDS writes before its later LDS reads (no other wave shares
+// the buffer, so no workgroup barrier is needed and loop trip counts may differ per wave).
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int LMAX>
+__device__ __forceinline__ void sh_poly(float x, float y, float z, float (&o)[(LMAX + 1) * (LMAX + 1)],
+                                        const float (&scale)[4]) {
+  o[0] = scale[0];
+  if constexpr (LMAX >= 1) {
+    const float c = 1.7320508075688772f * scale[1];
+    o[1] = c * x;
+    o[2] = c * y;
+    o[3] = c * z;
+  }
+  if constexpr (LMAX >= 2) {
+    const float r15 = 3.872983346207417f, r5 = 2.23606797749979f;
+    const float y2 = y * y, s = x * x + z * z;
+    const float a20 = r15 * x * z;
+    const float a24 = 0.5f * r15 * (z * z - x * x);
+    o[4] = scale[2] * a20;
+    o[5] = scale[2] * (r15 * x * y);
+    o[6] = scale[2] * (r5 * (y2 - 0.5f * s));
+    o[7] = scale[2] * (r15 * y * z);
+    o[8] = scale[2] * a24;
+    if constexpr (LMAX >= 3) {
+      const float r7 = 2.6457513110645907f;
+      const float c0 = 1.0801234497346435f;  // sqrt(42)/6
+      const float c2 = 1.6201851746019651f;  // sqrt(168)/8
+      const float t = 4.0f * y2 - s;
+      o[9] = scale[3] * (c0 * (a20 * z + a24 * x));
+      o[10] = scale[3] * (r7 * a20 * y);
+      o[11] = scale[3] * (c2 * t * x);
+      o[12] = scale[3] * (0.5f * r7 * y * (2.0f * y2 - 3.0f * s));
+      o[13] = scale[3] * (c2 * z * t);
+      o[14] = scale[3] * (r7 * a24 * y);
+      o[15] = scale[3] * (c0 * (a24 * z - a20 * x));
+    }
+  }
+}
+
+struct Scale4 {
+  float s[4];
+};
+
+template <int LMAX, bool NORMALIZE>
+__global__ __launch_bounds__(kWave* kWavesPerBlock) void sh_tile_kernel(const float* __restrict__ xyz,
+                                                                       float* __restrict__ out, long long n,
+                                                                       Scale4 sc) {
+  constexpr int NC = (LMAX + 1) * (LMAX + 1);
+  constexpr int LD = NC | 1;  // odd LDS row stride: conflict-free column access
+  __shared__ float s_in[kWavesPerBlock][kWave * 3];
+  __shared__ float s_out[kWavesPerBlock][kWave * LD];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = threadIdx.x / kWave;
+  const long long n_tiles = (n + kWave - 1) / kWave;
+  const float scale[4] = {sc.s[0], sc.s[1], sc.s[2], sc.s[3]};
+
+  for (long long tile = (long long)blockIdx.x * kWavesPerBlock + wv; tile < n_tiles;
+       tile += (long long)gridDim.x * kWavesPerBlock) {
+    const long long v0 = tile * kWave;
+    const int nv = (int)min((long long)kWave, n - v0);
+    float x, y, z;
+    if (nv == kWave) {
+      if (lane < 48) {
+        const float4 q = reinterpret_cast<const float4*>(xyz + v0 * 3)[lane];
+        reinterpret_cast<float4*>(s_in[wv])[lane] = q;
+      }
+      wave_lds_sync();
+      x = s_in[wv][lane * 3 + 0];
+      y = s_in[wv][lane * 3 + 1];
+      z = s_in[wv][lane * 3 + 2];
+    } else {
+      x = y = z = 0.0f;
+      if (lane < nv) {
+        x = xyz[(v0 + lane) * 3 + 0];
+        y = xyz[(v0 + lane) * 3 + 1];
+        z = xyz[(v0 + lane) * 3 + 2];
+      }
+    }
+    if constexpr (NORMALIZE) {
+      // x / max(|x|, 1e-12): torch.nn.functional.normalize (reference :96)
+      const float nrm = sqrtf(x * x + y * y + z * z);
+      const float inv = 1.0f / fmaxf(nrm, 1e-12f);
+      x *= inv;
+      y *= inv;
+      z *= inv;
+    }
+    float o[NC];
+    sh_poly<LMAX>(x, y, z, o, scale);
+#pragma unroll
+    for (int c = 0; c < NC; ++c) s_out[wv][lane * LD + c] = o[c];
+    wave_lds_sync();
+    float* dst = out + v0 * NC;
+    if (nv == kWave) {
+      constexpr int NQ = kWave * NC / 4;  // float4 per tile
+#pragma unroll
+      for (int q0 = 0; q0 < NQ; q0 += kWave) {
+        const int q = q0 + lane;
+        if (NQ % kWave == 0 || q < NQ) {
+          float4 v;
+          float* pv = reinterpret_cast<float*>(&v);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int e = q * 4 + t;
+            pv[t] = s_out[wv][(e / NC) * LD + (e % NC)];
+          }
+          reinterpret_cast<float4*>(dst)[q] = v;
+        }
+      }
+    } else {
+      for (int e = lane; e < nv * NC; e += kWave) dst[e] = s_out[wv][(e / NC) * LD + (e % NC)];
+    }
+    wave_lds_sync();
+  }
+}
+
+// ---------------------------------------------------------------- generic path
+constexpr int kMaxL = 12;
+constexpr int kMaxCols = (kMaxL + 1) * (kMaxL + 1);
+constexpr int kMaxEntries = 2048;
+
+struct RecEntry {
+  unsigned short out_col;  // absolute column of Y^{l+1}_i
+  unsigned short in_col;   // absolute column of Y^l_j
+  int axis;                // k: 0 x, 1 y, 2 z
+  float coef;              // c_l * w3j(l+1, 1, l)[i, k, j]
+};
+
+__constant__ RecEntry c_rec[kMaxEntries];
+__constant__ int c_rec_end[kMaxL + 1];  // entries for levels < l end at c_rec_end[l]
+
+struct ColMap {
+  unsigned char src[kMaxCols];  // output column -> polynomial column
+  float scale[kMaxCols];
+};
+
+__global__ __launch_bounds__(kWave) void sh_generic_kernel(const float* __restrict__ xyz, float* __restrict__ out,
+                                                           long long n, int lmax, int n_out, int normalize,
+                                                           const ColMap cmap) {
+  extern __shared__ float s_y[];  // [(lmax+1)^2][64]
+  const int lane = threadIdx.x;
+  for (long long v = (long long)blockIdx.x * kWave + lane; v - lane < n; v += (long long)gridDim.x * kWave) {
+    const bool live = v < n;
+    float x = 0.f, y = 0.f, z = 0.f;
+    if (live) {
+      x = xyz[v * 3 + 0];
+      y = xyz[v * 3 + 1];
+      z = xyz[v * 3 + 2];
+    }
+    if (normalize) {
+      const float inv = 1.0f / fmaxf(sqrtf(x * x + y * y + z * z), 1e-12f);
+      x *= inv;
+      y *= inv;
+      z *= inv;
+    }
+    s_y[lane] = 1.0f;
+    const int n_ent = c_rec_end[lmax];
+    int cur = -1;
+    float acc = 0.f;
+    for (int e = 0; e < n_ent; ++e) {
+      const RecEntry r = c_rec[e];
+      if ((int)r.out_col != cur) {
+        if (cur >= 0) s_y[cur * kWave + lane] = acc;
+        cur = r.out_col;
+        acc = 0.f;
+      }
+      const float a = r.axis == 0 ? x : (r.axis == 1 ? y : z);
+      acc = fmaf(r.coef * a, s_y[r.in_col * kWave + lane], acc);
+    }
+    if (cur >= 0) s_y[cur * kWave + lane] = acc;
+    if (live) {
+      for (int c = 0; c < n_out; ++c) out[v * n_out + c] = cmap.scale[c] * s_y[cmap.src[c] * kWave + lane];
+    }
+  }
+}
+
+std::mutex g_mu;
+bool g_tables_ready[64] = {false};
+
+int upload_tables(int dev) {
+  if (g_tables_ready[dev]) return E3X_OK;
+  std::vector<RecEntry> ent;
+  int ends[kMaxL + 1];
+  ends[0] = 0;
+  // Y^{l+1}_i = c_l sum_{k,j} w3j(l+1,1,l)[i,k,j] x_k Y^l_j ; c_l > 0 from |Y^{l+1}(0,1,0)|^2 = 2l+3
+  std::vector<double> pole(1, 1.0);
+  for (int l = 0; l < kMaxL; ++l) {
+    const auto& C = e3x::wigner_3j(l + 1, 1, l);
+    const int d_out = 2 * l + 3, d_in = 2 * l + 1;
+    std::vector<double> raw(d_out, 0.0);
+    double nrm = 0;
+    for (int i = 0; i < d_out; ++i) {
+      for (int j = 0; j < d_in; ++j) raw[i] += C[(i * 3 + 1) * d_in + j] * pole[j];
+      nrm += raw[i] * raw[i];
+    }
+    const double cl = std::sqrt((2.0 * l + 3.0) / nrm);
+    for (auto& v : raw) v *= cl;
+    pole = raw;
+    for (int i = 0; i < d_out; ++i)
+      for (int k = 0; k < 3; ++k)
+        for (int j = 0; j < d_in; ++j) {
+          const double c = C[(i * 3 + k) * d_in + j];
+          if (c != 0.0) {
+            RecEntry r;
+            r.out_col = (unsigned short)((l + 1) * (l + 1) + i);
+            r.in_col = (unsigned short)(l * l + j);
+            r.axis = k;
+            r.coef = (float)(cl * c);
+            ent.push_back(r);
+          }
+        }
+    ends[l + 1] = (int)ent.size();
+  }
+  if ((int)ent.size() > kMaxEntries) return e3x::fail(E3X_ERR_INVALID, "sh: recurrence table overflow");
+  if (hipMemcpyToSymbol(HIP_SYMBOL(c_rec), ent.data(), ent.size() * sizeof(RecEntry)) != hipSuccess ||
+      hipMemcpyToSymbol(HIP_SYMBOL(c_rec_end), ends, sizeof(ends)) != hipSuccess)
+    return e3x::fail(E3X_ERR_HIP, "sh: uploading the recurrence table failed");
+  g_tables_ready[dev] = true;
+  return E3X_OK;
+}
+
+template <int LMAX>
+void launch_tile(bool normalize, const float* xyz, float* out, long long n, Scale4 sc, hipStream_t st) {
+  const long long tiles = (n + kWave - 1) / kWave;
+  long long blocks = (tiles + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (blocks > 256 * 32) blocks = 256 * 32;  // grid-stride beyond 32 blocks per CU
+  if (normalize)
+    hipLaunchKernelGGL((sh_tile_kernel<LMAX, true>), dim3((unsigned)blocks), dim3(kWave * kWavesPerBlock), 0, st, xyz,
+                       out, n, sc);
+  else
+    hipLaunchKernelGGL((sh_tile_kernel<LMAX, false>), dim3((unsigned)blocks), dim3(kWave * kWavesPerBlock), 0, st,
+                       xyz, out, n, sc);
+}
+
+}  // namespace
+
+extern "C" int e3x_sh_forward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization,
+                              const void* xyz, void* out, int64_t n, int32_t dtype, void* stream) {
+  if (!ls || n_ls <= 0 || n < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_forward: empty l list or negative n");
+  if (dtype != E3X_F32) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_forward: only fp32 storage is implemented");
+  if (normalization < 0 || normalization > 2)
+    return e3x::fail(E3X_ERR_INVALID, "e3x_sh_forward: normalization must be integral, component or norm");
+  int lmax = 0, n_out = 0;
+  bool is_range = true;
+  for (int i = 0; i < n_ls; ++i) {
+    if (ls[i] < 0 || ls[i] > kMaxL)
+      return e3x::fail(E3X_ERR_INVALID, "spherical_harmonics maximum l implemented is 12");
+    lmax = ls[i] > lmax ? ls[i] : lmax;
+    is_range = is_range && ls[i] == i;
+    n_out += 2 * ls[i] + 1;
+  }
+  if (n_out > kMaxCols) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_forward: more than 169 output columns");
+  if (n == 0) return E3X_OK;
+  if (!xyz || !out) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_forward: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  auto lscale = [&](int l) -> float {
+    if (normalization == E3X_NORM_INTEGRAL) return (float)(1.0 / std::sqrt(4.0 * M_PI));
+    if (normalization == E3X_NORM_NORM) return (float)(1.0 / std::sqrt(2.0 * l + 1.0));
+    return 1.0f;
+  };
+  const bool aligned = ((uintptr_t)xyz % 16 == 0) && ((uintptr_t)out % 16 == 0);
+  if (is_range && lmax <= 3 && aligned) {
+    Scale4 sc;
+    for (int l = 0; l < 4; ++l) sc.s[l] = lscale(l);
+    const float* px = (const float*)xyz;
+    float* po = (float*)out;
+    switch (lmax) {
+      case 0: launch_tile<0>(normalize, px, po, n, sc, st); break;
+      case 1: launch_tile<1>(normalize, px, po, n, sc, st); break;
+      case 2: launch_tile<2>(normalize, px, po, n, sc, st); break;
+      default: launch_tile<3>(normalize, px, po, n, sc, st); break;
+    }
+  } else {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return e3x::fail(E3X_ERR_HIP, "hipGetDevice failed");
+    std::lock_guard<std::mutex> lock(g_mu);
+    int rc = upload_tables(dev);
+    if (rc) return rc;
+    ColMap cm;
+    int c = 0;
+    for (int i = 0; i < n_ls; ++i)
+      for (int m = 0; m < 2 * ls[i] + 1; ++m, ++c) {
+        cm.src[c] = (unsigned char)(ls[i] * ls[i] + m);
+        cm.scale[c] = lscale(ls[i]);
+      }
+    long long blocks = (n + kWave - 1) / kWave;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    const size_t shmem = (size_t)(lmax + 1) * (lmax + 1) * kWave * sizeof(float);
+    hipLaunchKernelGGL(sh_generic_kernel, dim3((unsigned)blocks), dim3(kWave), shmem, st, (const float*)xyz,
+                       (float*)out, (long long)n, lmax, n_out, (int)normalize, cm);
+  }
+  if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_sh_forward: kernel launch failed");
+  return E3X_OK;
+}

@@ -1,0 +1,395 @@
+// Tensor-product plans: validation of an instruction set, emission of the constexpr
+// tables that specialise the device templates, code-object loading and kernel launches.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <memory>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "e3x_internal.h"
+#include "jit.h"
+
+namespace {
+
+struct PathInfo {
+  int in1, in2, out, mode, has_w;
+  double pw;
+  int woff;  // offset in the flat weight vector (weighted paths only)
+};
+
+constexpr int kMaxDevices = 64;
+
+}  // namespace
+
+struct e3x_plan {
+  std::vector<e3x_irrep> in1, in2, out;
+  std::vector<int> off1, off2, offo;
+  std::vector<PathInfo> paths;
+  int shared_weights = 1, dtype = E3X_F32;
+  int64_t in1_dim = 0, in2_dim = 0, out_dim = 0, weight_numel = 0;
+  std::string family, key, hsaco;
+  bool zero_fill = false;  // some output irrep is reached by no instruction
+  // launch geometry of the lane<->multiplicity kernels
+  int lanes = 64, chunks = 1;
+  // uvw_mfma geometry
+  int rows_per_block = 0;
+  std::mutex mu;
+  hipModule_t module[kMaxDevices] = {nullptr};
+  hipFunction_t fn_plain[kMaxDevices] = {nullptr};
+  hipFunction_t fn_fused[kMaxDevices] = {nullptr};
+};
+
+namespace {
+
+using e3x::fail;
+
+int dim_of(const e3x_irrep& r) { return r.mul * (2 * r.l + 1); }
+
+std::string fstr(double v) {
+  char buf[64];
+  std::snprintf(buf, sizeof(buf), "%.9ef", v);
+  return buf;
+}
+
+int pow2_at_least(int v, int lo) {
+  int p = lo;
+  while (p < v) p *= 2;
+  return p;
+}
+
+// ---- common part of the generated tables ------------------------------------------
+void emit_header(std::ostringstream& s, const e3x_plan& P) {
+  s << "// generated: tables of one instruction set\n#include <stdint.h>\nnamespace cfg {\n";
+  s << "typedef " << (P.dtype == E3X_BF16 ? "unsigned short" : "float") << " store_t;\n";
+  s << "constexpr bool SHARED_W = " << (P.shared_weights ? "true" : "false") << ";\n";
+  s << "constexpr int IN1_DIM = " << P.in1_dim << ", IN2_DIM = " << P.in2_dim << ", OUT_DIM = " << P.out_dim
+    << ", W_NUMEL = " << P.weight_numel << ";\n";
+  s << "constexpr int LANES = " << P.lanes << ", CHUNKS = " << P.chunks << ";\n";
+}
+
+struct NzList {
+  std::vector<std::string> rows;
+  std::vector<int> beg, end;
+};
+
+// non-zeros of pw * wigner_3j per path, as "{i, j, k, c}" rows
+NzList emit_nz(const e3x_plan& P) {
+  NzList L;
+  for (const auto& p : P.paths) {
+    const int l1 = P.in1[p.in1].l, l2 = P.in2[p.in2].l, l3 = P.out[p.out].l;
+    const auto& C = e3x::wigner_3j(l1, l2, l3);
+    const int d2 = 2 * l2 + 1, d3 = 2 * l3 + 1;
+    L.beg.push_back((int)L.rows.size());
+    for (int i = 0; i < 2 * l1 + 1; ++i)
+      for (int j = 0; j < d2; ++j)
+        for (int k = 0; k < d3; ++k) {
+          const double c = C[(i * d2 + j) * d3 + k] * p.pw;
+          if (c != 0.0) {
+            std::ostringstream r;
+            r << "{" << i << ", " << j << ", " << k << ", " << fstr(c) << "}";
+            L.rows.push_back(r.str());
+          }
+        }
+    L.end.push_back((int)L.rows.size());
+  }
+  return L;
+}
+
+void emit_nz_table(std::ostringstream& s, const NzList& L) {
+  s << "struct Nz { int i, j, k; float c; };\n";
+  s << "constexpr int N_NZ = " << L.rows.size() << ";\n";
+  s << "constexpr Nz nz[N_NZ > 0 ? N_NZ : 1] = {\n";
+  for (const auto& r : L.rows) s << "  " << r << ",\n";
+  if (L.rows.empty()) s << "  {0, 0, 0, 0.f}\n";
+  s << "};\n";
+}
+
+// ---- uvu ---------------------------------------------------------------------------
+int build_uvu_source(e3x_plan& P, std::string* src) {
+  int max_mul = 1;
+  std::vector<char> used1(P.in1.size(), 0), usedo(P.out.size(), 0);
+  long long unrolled = 0;
+  for (const auto& p : P.paths) {
+    if (P.in1[p.in1].mul != P.out[p.out].mul)
+      return fail(E3X_ERR_INVALID, "uvu instruction needs irreps_in1[i_in1].mul == irreps_out[i_out].mul");
+    used1[p.in1] = 1;
+    usedo[p.out] = 1;
+    max_mul = std::max(max_mul, P.in1[p.in1].mul);
+  }
+  P.lanes = max_mul > 32 ? 64 : pow2_at_least(max_mul, 16);
+  P.chunks = (max_mul + P.lanes - 1) / P.lanes;
+  if (P.in2_dim > 64) return fail(E3X_ERR_INVALID, "uvu kernel: irreps_in2.dim > 64 is not supported");
+
+  std::ostringstream s;
+  emit_header(s, P);
+  int reg = 0;
+  s << "struct In1 { int off, d, mul, reg; bool used; };\n";
+  s << "constexpr int N_IN1 = " << P.in1.size() << ";\nconstexpr In1 in1[N_IN1] = {\n";
+  for (size_t a = 0; a < P.in1.size(); ++a) {
+    const int d = 2 * P.in1[a].l + 1;
+    s << "  {" << P.off1[a] << ", " << d << ", " << P.in1[a].mul << ", " << reg << ", " << (used1[a] ? "true" : "false")
+      << "},\n";
+    if (used1[a]) reg += d;
+  }
+  s << "};\nconstexpr int X1_REGS = " << reg << ";\n";
+  if (reg > 96) return fail(E3X_ERR_INVALID, "uvu kernel: more than 96 input components per multiplicity index");
+  reg = 0;
+  s << "struct Out { int off, d, mul, reg; bool used; };\n";
+  s << "constexpr int N_OUT = " << P.out.size() << ";\nconstexpr Out outs[N_OUT] = {\n";
+  for (size_t c = 0; c < P.out.size(); ++c) {
+    const int d = 2 * P.out[c].l + 1;
+    s << "  {" << P.offo[c] << ", " << d << ", " << P.out[c].mul << ", " << reg << ", " << (usedo[c] ? "true" : "false")
+      << "},\n";
+    if (usedo[c]) reg += d;
+  }
+  s << "};\nconstexpr int ACC_REGS = " << reg << ";\n";
+  if (reg > 256) return fail(E3X_ERR_INVALID, "uvu kernel: more than 256 output components per multiplicity index");
+  NzList L = emit_nz(P);
+  int wreg = 0;
+  s << "struct Path { int in1, x2off, d2, V, out, woff, wreg; bool has_w; int nz_beg, nz_end; };\n";
+  s << "constexpr int N_PATH = " << P.paths.size() << ";\nconstexpr Path paths[N_PATH > 0 ? N_PATH : 1] = {\n";
+  for (size_t i = 0; i < P.paths.size(); ++i) {
+    const auto& p = P.paths[i];
+    const int V = P.in2[p.in2].mul;
+    s << "  {" << p.in1 << ", " << P.off2[p.in2] << ", " << 2 * P.in2[p.in2].l + 1 << ", " << V << ", " << p.out << ", "
+      << p.woff << ", " << wreg << ", " << (p.has_w ? "true" : "false") << ", " << L.beg[i] << ", " << L.end[i]
+      << "},\n";
+    if (p.has_w) wreg += V;
+    unrolled += (long long)V * (L.end[i] - L.beg[i]);
+  }
+  if (P.paths.empty()) s << "  {0, 0, 1, 0, 0, 0, 0, false, 0, 0}\n";
+  s << "};\nconstexpr int W_REGS = " << wreg << ";\n";
+  if (wreg > 128 || unrolled > 20000)
+    return fail(E3X_ERR_INVALID, "uvu kernel: instruction set too large to unroll (irreps_in2 multiplicities too high)");
+  emit_nz_table(s, L);
+  s << "}  // namespace cfg\n";
+  *src = s.str() + e3x::kTplCommon + e3x::kTplUvu;
+  return E3X_OK;
+}
+
+// ---- uvw (lane <-> output multiplicity, VALU) ----------------------------------------
+int build_uvw_small_source(e3x_plan& P, std::string* src) {
+  int max_mul = 1;
+  std::vector<char> usedo(P.out.size(), 0);
+  for (const auto& p : P.paths) {
+    if (!p.has_w) return fail(E3X_ERR_INVALID, "uvw instruction must have weights");
+    usedo[p.out] = 1;
+    max_mul = std::max(max_mul, P.out[p.out].mul);
+  }
+  P.lanes = max_mul > 32 ? 64 : pow2_at_least(max_mul, 16);
+  P.chunks = (max_mul + P.lanes - 1) / P.lanes;
+  if ((P.in1_dim + P.in2_dim) * 16 * (64 / P.lanes) > 65536)
+    return fail(E3X_ERR_INVALID, "uvw kernel: input rows too long for the LDS staging buffer");
+  std::ostringstream s;
+  emit_header(s, P);
+  int reg = 0;
+  s << "struct Out { int off, d, mul, reg; bool used; };\n";
+  s << "constexpr int N_OUT = " << P.out.size() << ";\nconstexpr Out outs[N_OUT] = {\n";
+  for (size_t c = 0; c < P.out.size(); ++c) {
+    const int d = 2 * P.out[c].l + 1;
+    s << "  {" << P.offo[c] << ", " << d << ", " << P.out[c].mul << ", " << reg << ", " << (usedo[c] ? "true" : "false")
+      << "},\n";
+    if (usedo[c]) reg += d;
+  }
+  s << "};\nconstexpr int ACC_REGS = " << reg << ";\n";
+  if (reg > 256) return fail(E3X_ERR_INVALID, "uvw kernel: more than 256 output components per multiplicity index");
+  NzList L = emit_nz(P);
+  s << "struct Path { int x1off, d1, U, x2off, d2, V, out, woff; int nz_beg, nz_end; };\n";
+  s << "constexpr int N_PATH = " << P.paths.size() << ";\nconstexpr Path paths[N_PATH > 0 ? N_PATH : 1] = {\n";
+  for (size_t i = 0; i < P.paths.size(); ++i) {
+    const auto& p = P.paths[i];
+    s << "  {" << P.off1[p.in1] << ", " << 2 * P.in1[p.in1].l + 1 << ", " << P.in1[p.in1].mul << ", " << P.off2[p.in2]
+      << ", " << 2 * P.in2[p.in2].l + 1 << ", " << P.in2[p.in2].mul << ", " << p.out << ", " << p.woff << ", "
+      << L.beg[i] << ", " << L.end[i] << "},\n";
+  }
+  if (P.paths.empty()) s << "  {0, 1, 0, 0, 1, 0, 0, 0, 0, 0}\n";
+  s << "};\n";
+  emit_nz_table(s, L);
+  s << "}  // namespace cfg\n";
+  *src = s.str() + e3x::kTplCommon + e3x::kTplUvwSmall;
+  return E3X_OK;
+}
+
+int load_functions(e3x_plan* P, int dev) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  if (P->module[dev]) return E3X_OK;
+  hipModule_t mod = nullptr;
+  hipError_t err = hipModuleLoad(&mod, P->hsaco.c_str());
+  if (err != hipSuccess)
+    return fail(E3X_ERR_HIP, "hipModuleLoad(" + P->hsaco + ") failed: " + hipGetErrorString(err));
+  const std::string plain = "e3x_" + P->family + "_plain";
+  if (hipModuleGetFunction(&P->fn_plain[dev], mod, plain.c_str()) != hipSuccess)
+    return fail(E3X_ERR_HIP, "kernel " + plain + " missing from " + P->hsaco);
+  if (P->family == "uvu") {
+    if (hipModuleGetFunction(&P->fn_fused[dev], mod, "e3x_uvu_fused") != hipSuccess)
+      return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused missing from " + P->hsaco);
+  }
+  P->module[dev] = mod;
+  return E3X_OK;
+}
+
+int current_device(int* dev) {
+  if (hipGetDevice(dev) != hipSuccess || *dev < 0 || *dev >= kMaxDevices) return fail(E3X_ERR_HIP, "hipGetDevice failed");
+  return E3X_OK;
+}
+
+}  // namespace
+
+extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
+  if (!d || !out) return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: null argument");
+  if (d->n_in1 < 0 || d->n_in2 < 0 || d->n_out < 0 || d->n_ins < 0 || (d->n_in1 && !d->in1) || (d->n_in2 && !d->in2) ||
+      (d->n_out && !d->out) || (d->n_ins && !d->ins))
+    return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: malformed descriptor");
+  if (d->dtype != E3X_F32 && d->dtype != E3X_BF16) return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: unknown dtype");
+  std::unique_ptr<e3x_plan> P(new e3x_plan);
+  P->shared_weights = d->shared_weights ? 1 : 0;
+  P->dtype = d->dtype;
+  auto take = [&](const e3x_irrep* src, int n, std::vector<e3x_irrep>& dst, std::vector<int>& off, int64_t& dim) -> int {
+    dim = 0;
+    for (int i = 0; i < n; ++i) {
+      if (src[i].mul < 0 || src[i].l < 0 || src[i].l > 12 || (src[i].p != 1 && src[i].p != -1))
+        return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: irrep needs mul >= 0, 0 <= l <= 12, p = +-1");
+      dst.push_back(src[i]);
+      off.push_back((int)dim);
+      dim += dim_of(src[i]);
+    }
+    return E3X_OK;
+  };
+  int rc;
+  if ((rc = take(d->in1, d->n_in1, P->in1, P->off1, P->in1_dim))) return rc;
+  if ((rc = take(d->in2, d->n_in2, P->in2, P->off2, P->in2_dim))) return rc;
+  if ((rc = take(d->out, d->n_out, P->out, P->offo, P->out_dim))) return rc;
+
+  int n_uvu = 0, n_uvw = 0;
+  std::vector<char> reached(P->out.size(), 0);
+  int64_t woff = 0;
+  for (int t = 0; t < d->n_ins; ++t) {
+    const e3x_instruction& I = d->ins[t];
+    if (I.i_in1 < 0 || I.i_in1 >= d->n_in1 || I.i_in2 < 0 || I.i_in2 >= d->n_in2 || I.i_out < 0 || I.i_out >= d->n_out)
+      return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: instruction index out of range");
+    const e3x_irrep &a = P->in1[I.i_in1], &b = P->in2[I.i_in2], &c = P->out[I.i_out];
+    // selection rules (reference _tensor_product.py:294-295)
+    if (a.p * b.p != c.p || c.l < std::abs(a.l - b.l) || c.l > a.l + b.l)
+      return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: instruction violates the selection rules");
+    if (I.mode != E3X_MODE_UVU && I.mode != E3X_MODE_UVW)
+      return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: only the uvu and uvw connection modes are implemented");
+    if (I.mode == E3X_MODE_UVW && !I.has_weight) return fail(E3X_ERR_INVALID, "uvw instruction must have weights");
+    const int64_t n_w = I.mode == E3X_MODE_UVU ? (int64_t)a.mul * b.mul : (int64_t)a.mul * b.mul * c.mul;
+    const bool empty = a.mul == 0 || b.mul == 0 || c.mul == 0;  // dropped, reference _codegen.py:51
+    if (!empty) {
+      PathInfo p{I.i_in1, I.i_in2, I.i_out, I.mode, I.has_weight ? 1 : 0, I.path_weight, (int)woff};
+      P->paths.push_back(p);
+      (I.mode == E3X_MODE_UVU ? n_uvu : n_uvw)++;
+      reached[I.i_out] = 1;
+    }
+    if (I.has_weight && !empty) woff += n_w;
+  }
+  if (woff >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: weight_numel must fit in int32");
+  P->weight_numel = woff;
+  for (size_t c = 0; c < P->out.size(); ++c)
+    if (!reached[c] && dim_of(P->out[c]) > 0) P->zero_fill = true;
+  if (n_uvu && n_uvw)
+    return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: mixing uvu and uvw instructions in one plan is not implemented");
+
+  std::string src;
+  if (n_uvw) {
+    P->family = "uvw_small";
+    rc = build_uvw_small_source(*P, &src);
+  } else {
+    P->family = "uvu";
+    rc = build_uvu_source(*P, &src);
+  }
+  if (rc) return rc;
+  if ((rc = e3x::get_code_object(P->family, src, &P->key, &P->hsaco))) return rc;
+  *out = P.release();
+  return E3X_OK;
+}
+
+extern "C" int e3x_tp_plan_destroy(e3x_plan* plan) {
+  if (!plan) return E3X_OK;
+  // code objects stay loaded: kernels of this plan may still be queued on a stream
+  delete plan;
+  return E3X_OK;
+}
+
+extern "C" int e3x_tp_plan_info(const e3x_plan* plan, int64_t* weight_numel, int64_t* in1_dim, int64_t* in2_dim,
+                                int64_t* out_dim, const char** family, const char** cache_key) {
+  if (!plan) return fail(E3X_ERR_INVALID, "e3x_tp_plan_info: null plan");
+  if (weight_numel) *weight_numel = plan->weight_numel;
+  if (in1_dim) *in1_dim = plan->in1_dim;
+  if (in2_dim) *in2_dim = plan->in2_dim;
+  if (out_dim) *out_dim = plan->out_dim;
+  if (family) *family = plan->family.c_str();
+  if (cache_key) *cache_key = plan->key.c_str();
+  return E3X_OK;
+}
+
+static int zero_output(e3x_plan* P, void* out, int64_t rows, hipStream_t st) {
+  const size_t bytes = (size_t)rows * P->out_dim * (P->dtype == E3X_BF16 ? 2 : 4);
+  if (bytes == 0) return E3X_OK;
+  return e3x::fill_zero_bytes(out, bytes, st);
+}
+
+extern "C" int e3x_tp_forward(e3x_plan* P, const void* x1, const void* x2, const void* w, void* out, int64_t Z,
+                              void* stream) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_forward: null plan");
+  if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_tp_forward: negative batch");
+  if (Z == 0 || P->out_dim == 0) return E3X_OK;
+  if (!out || (P->in1_dim && !x1) || (P->in2_dim && !x2) || (P->weight_numel && !w))
+    return fail(E3X_ERR_INVALID, "e3x_tp_forward: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  int dev, rc;
+  if ((rc = current_device(&dev))) return rc;
+  if (P->zero_fill || P->paths.empty()) {
+    if ((rc = zero_output(P, out, Z, st))) return rc;
+    if (P->paths.empty()) return E3X_OK;
+  }
+  if ((rc = load_functions(P, dev))) return rc;
+  long long n_rows = Z;
+  void* args[] = {(void*)&x1, (void*)&x2, (void*)&w, (void*)&out, (void*)&n_rows};
+  const int groups = 64 / P->lanes;
+  const long long items = (Z + groups - 1) / groups * P->chunks;
+  const long long blocks = (items + 3) / 4;
+  if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_forward: batch too large for one launch");
+  hipError_t err = hipModuleLaunchKernel(P->fn_plain[dev], (unsigned)blocks, 1, 1, 256, 1, 1, 0, st, args, nullptr);
+  if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_tp_forward: launch failed: ") + hipGetErrorString(err));
+  return E3X_OK;
+}
+
+extern "C" int e3x_tp_gather_scatter(e3x_plan* P, const void* node_x, const void* edge_attr, const void* w,
+                                     const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
+                                     void* out, int64_t E, int64_t num_src_nodes, int64_t num_out_nodes,
+                                     void* stream) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: null plan");
+  if (P->family != "uvu") return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: the plan must be all-uvu");
+  if (P->shared_weights && P->weight_numel)
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: per-edge weights (shared_weights = 0) are required");
+  if (idx_bits != 32 && idx_bits != 64) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: idx_bits must be 32 or 64");
+  if (E < 0 || num_src_nodes < 0 || num_out_nodes < 0) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: negative size");
+  if (num_out_nodes == 0 || P->out_dim == 0) return E3X_OK;
+  if (!out || !rowptr || (E > 0 && (!src || (P->in1_dim && !node_x) || (P->in2_dim && !edge_attr) || (P->weight_numel && !w))))
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  int dev, rc;
+  if ((rc = current_device(&dev))) return rc;
+  if (P->zero_fill || P->paths.empty()) {
+    if ((rc = zero_output(P, out, num_out_nodes, st))) return rc;
+    if (P->paths.empty()) return E3X_OK;
+  }
+  if ((rc = load_functions(P, dev))) return rc;
+  int idx64 = idx_bits == 64;
+  long long n_rows = num_out_nodes, n_src = num_src_nodes;
+  void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&w,    (void*)&out,    (void*)&src,
+                  (void*)&idx64,  (void*)&rowptr,    (void*)&perm, (void*)&n_rows, (void*)&n_src};
+  const long long items = n_rows * P->chunks;
+  const long long blocks = (items + 3) / 4;
+  if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
+  hipError_t err = hipModuleLaunchKernel(P->fn_fused[dev], (unsigned)blocks, 1, 1, 256, 1, 1, 0, st, args, nullptr);
+  if (err != hipSuccess)
+    return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
+  return E3X_OK;
+}

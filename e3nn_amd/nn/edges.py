@@ -1,0 +1,50 @@
+"""Edge lists grouped by destination node, the preprocessing of the fused scatter-sum.
+
+The message-passing step of the reference is
+``scatter(tp(node_features[edge_src], edge_attr, weight), edge_dst, dim_size=N)``
+(e3nn/nn/models/v2106/points_convolution.py:13-17,105-106).  The fused kernel needs the
+edges of each destination to be contiguous: ``DstSortedEdges`` validates both index
+arrays once and builds the row pointers and the stable permutation on the GPU.
+"""
+import torch
+
+from .. import _lib
+
+
+class DstSortedEdges:
+    """``edge_src[e] -> edge_dst[e]`` for ``e < E``, grouped by ``edge_dst``.
+
+    ``edge_src`` indexes rows of the node-feature table like torch advanced indexing
+    (values in ``[-num_src_nodes, num_src_nodes)``, negative ones wrap); ``edge_dst``
+    follows ``scatter_add_`` (values in ``[0, num_nodes)``).  Out-of-range values raise
+    ``IndexError``.  int32 and int64 indices give identical results.
+    """
+
+    def __init__(self, edge_src: torch.Tensor, edge_dst: torch.Tensor, num_nodes: int, num_src_nodes: int = None):
+        if not (edge_src.is_cuda and edge_dst.is_cuda):
+            raise RuntimeError("DstSortedEdges needs index tensors on the GPU")
+        if edge_src.dtype not in (torch.int32, torch.int64) or edge_dst.dtype not in (torch.int32, torch.int64):
+            raise TypeError("edge indices must be int32 or int64")
+        if edge_src.ndim != 1 or edge_src.shape != edge_dst.shape:
+            raise ValueError("edge_src and edge_dst must be 1-D tensors of the same length")
+        self.num_nodes = int(num_nodes)
+        self.num_src_nodes = int(num_nodes if num_src_nodes is None else num_src_nodes)
+        self.edge_src = edge_src.contiguous()
+        self.edge_dst = edge_dst.contiguous()
+        self.num_edges = E = edge_src.numel()
+        dev = edge_src.device
+        L = _lib.lib()
+        with torch.cuda.device(dev):
+            st = _lib.stream_ptr(dev)
+            _lib.check(L.e3x_index_check(_lib.ptr(self.edge_src), self.edge_src.element_size() * 8, E, self.num_src_nodes, st))
+            self.rowptr = torch.empty(self.num_nodes + 1, dtype=torch.int32, device=dev)
+            self.perm = torch.empty(E, dtype=torch.int32, device=dev)
+            ws_bytes = L.e3x_csr_workspace_bytes(E, self.num_nodes)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            _lib.check(
+                L.e3x_csr_build(
+                    _lib.ptr(self.edge_dst), self.edge_dst.element_size() * 8, E, self.num_nodes, _lib.ptr(self.rowptr),
+                    _lib.ptr(self.perm), _lib.ptr(ws), ws_bytes, st,
+                )  # fmt: skip
+            )
+

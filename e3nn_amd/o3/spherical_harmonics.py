@@ -1,0 +1,110 @@
+"""Spherical harmonics as polynomials of x, y, z, evaluated by a HIP kernel.
+
+API of the reference's ``e3nn.o3.SphericalHarmonics`` / ``e3nn.o3.spherical_harmonics``
+(e3nn/o3/_spherical_harmonics.py:14-112, :115-190).
+"""
+import ctypes
+from typing import Any, List, Union
+
+import torch
+
+from .. import _lib
+from .irreps import Irreps
+
+_NORMALIZATION = {"integral": _lib.NORM_INTEGRAL, "component": _lib.NORM_COMPONENT, "norm": _lib.NORM_NORM}
+
+
+class _SphericalHarmonicsFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, ls, normalize, normalization):
+        if not x.is_cuda:
+            raise RuntimeError("e3nn_amd.o3.spherical_harmonics runs on the GPU only; got a CPU tensor")
+        if x.dtype != torch.float32:
+            raise TypeError(f"spherical_harmonics kernel supports float32 input, got {x.dtype}")
+        batch = x.shape[:-1]
+        xyz = x.reshape(-1, 3).contiguous()
+        n = xyz.shape[0]
+        n_out = sum(2 * l + 1 for l in ls)
+        out = torch.empty(n, n_out, dtype=x.dtype, device=x.device)
+        arr = (ctypes.c_int32 * len(ls))(*ls)
+        with torch.cuda.device(x.device):
+            _lib.check(
+                _lib.lib().e3x_sh_forward(
+                    arr, len(ls), int(bool(normalize)), _NORMALIZATION[normalization], _lib.ptr(xyz), _lib.ptr(out), n,
+                    _lib.F32, _lib.stream_ptr(x.device),
+                )  # fmt: skip
+            )
+        return out.reshape(batch + (n_out,))
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("the spherical-harmonics backward kernel is not implemented")
+
+
+class SphericalHarmonics(torch.nn.Module):
+    """Module version of :func:`spherical_harmonics`; parameters as in the reference (:28-34)."""
+
+    def __init__(
+        self,
+        irreps_out: Union[int, List[int], str, Irreps],
+        normalize: bool,
+        normalization: str = "integral",
+        irreps_in: Any = None,
+    ) -> None:
+        super().__init__()
+        self.normalize = normalize
+        self.normalization = normalization
+        assert normalization in ["integral", "component", "norm"]
+
+        if isinstance(irreps_out, str):
+            irreps_out = Irreps(irreps_out)
+        if isinstance(irreps_out, Irreps) and irreps_in is None:
+            # an odd-l even-parity output can only come from a pseudovector input
+            if any(l % 2 == 1 and p == 1 for _, (l, p) in irreps_out):
+                irreps_in = Irreps("1e")
+        if irreps_in is None:
+            irreps_in = Irreps("1o")
+        irreps_in = Irreps(irreps_in)
+        if irreps_in not in (Irreps("1x1o"), Irreps("1x1e")):
+            raise ValueError(
+                f"irreps_in for SphericalHarmonics must be either a vector (`1x1o`) or a pseudovector (`1x1e`), "
+                f"not `{irreps_in}`"
+            )
+        self.irreps_in = irreps_in
+        input_p = irreps_in[0].ir.p
+
+        if isinstance(irreps_out, Irreps):
+            ls = []
+            for mul, (l, p) in irreps_out:
+                if p != input_p**l:
+                    raise ValueError(
+                        f"irreps_out `{irreps_out}` passed to SphericalHarmonics asked for an output of l = {l} with "
+                        f"parity p = {p}, which is inconsistent with the input parity {input_p} — the output parity "
+                        f"should have been p = {input_p**l}"
+                    )
+                ls.extend([l] * mul)
+        elif isinstance(irreps_out, int):
+            ls = [irreps_out]
+        else:
+            ls = list(irreps_out)
+
+        self.irreps_out = Irreps([(1, (l, input_p**l)) for l in ls]).simplify()
+        self._ls_list = ls
+        self._lmax = max(ls)
+        if self._lmax > 12:
+            raise NotImplementedError("spherical_harmonics maximum l implemented is 12, send us an email to ask for more")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return _SphericalHarmonicsFn.apply(x, tuple(self._ls_list), self.normalize, self.normalization)
+
+
+def spherical_harmonics(
+    l: Union[int, List[int], str, Irreps], x: torch.Tensor, normalize: bool, normalization: str = "integral"
+) -> torch.Tensor:
+    r"""Spherical harmonics :math:`Y^l(x)` of the vectors ``x[..., 3]``; output ``[..., sum(2l+1)]``.
+
+    ``normalize`` projects ``x`` onto the unit sphere first (the zero vector gives the
+    l = 0 constant and zeros elsewhere); ``normalization`` is ``'integral'``,
+    ``'component'`` (:math:`\|Y^l\|^2 = 2l+1` on the sphere) or ``'norm'``.
+    """
+    return SphericalHarmonics(l, normalize, normalization)(x)

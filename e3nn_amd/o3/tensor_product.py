@@ -1,0 +1,433 @@
+"""Tensor product with parametrised paths, evaluated by instruction-set-specialised HIP kernels.
+
+Public behaviour of the reference's ``e3nn.o3.TensorProduct``
+(e3nn/o3/_tensor_product/_tensor_product.py:196-609) and
+``e3nn.o3.FullyConnectedTensorProduct`` (e3nn/o3/_tensor_product/_sub.py:10-68) for the
+``uvu`` and ``uvw`` connection modes: constructor arguments, normalisation of the path
+weights, weight bookkeeping, ``output_mask``, ``forward`` with broadcasting of the batch
+dimensions, weight views.  Where the reference generates an fx graph of einsums per
+instruction set (``_codegen.py:24-395``), this module asks the C library for a plan: one
+fused kernel specialised to the instruction set.
+
+``forward_gather_scatter`` is additive: the message-passing step
+``scatter(tp(x[edge_src], edge_attr, w), edge_dst, N)`` in one kernel.
+"""
+import ctypes
+import warnings
+from collections import namedtuple
+from math import prod, sqrt
+from typing import List, Optional, Union
+
+import torch
+
+from .. import _lib, get_optimization_defaults
+from ..nn.edges import DstSortedEdges
+from .irreps import Irreps
+
+Instruction = namedtuple(
+    "Instruction", ["i_in1", "i_in2", "i_out", "connection_mode", "has_weight", "path_weight", "path_shape"]
+)
+
+_MODES = ["uvw", "uvu", "uvv", "uuw", "uuu", "uvuv", "uvu<v", "u<vw"]
+_KERNEL_MODES = {"uvw": _lib.MODE_UVW, "uvu": _lib.MODE_UVU}
+_DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}
+
+
+def _path_shape(mode, m1, m2, mo):
+    return {
+        "uvw": (m1, m2, mo),
+        "uvu": (m1, m2),
+        "uvv": (m1, m2),
+        "uuw": (m1, mo),
+        "uuu": (m1,),
+        "uvuv": (m1, m2),
+        "uvu<v": (m1 * (m2 - 1) // 2,),
+        "u<vw": (m1 * (m2 - 1) // 2, mo),
+    }[mode]
+
+
+def _num_elements(mode, m1, m2):
+    return {
+        "uvw": m1 * m2,
+        "uvu": m2,
+        "uvv": m1,
+        "uuw": m1,
+        "uuu": 1,
+        "uvuv": 1,
+        "uvu<v": 1,
+        "u<vw": m1 * (m2 - 1) // 2,
+    }[mode]
+
+
+class _Plan:
+    """Owner of one ``e3x_plan`` handle."""
+
+    def __init__(self, tp: "TensorProduct", dtype: torch.dtype):
+        L = _lib.lib()
+        mk = lambda irreps: (_lib.Irrep * max(1, len(irreps)))(*[_lib.Irrep(mul, ir.l, ir.p) for mul, ir in irreps])  # noqa: E731
+        in1, in2, out = mk(tp.irreps_in1), mk(tp.irreps_in2), mk(tp.irreps_out)
+        ins = (_lib.Instruction * max(1, len(tp.instructions)))(
+            *[
+                _lib.Instruction(t.i_in1, t.i_in2, t.i_out, _KERNEL_MODES[t.connection_mode], int(t.has_weight), t.path_weight)
+                for t in tp.instructions
+            ]
+        )
+        desc = _lib.TpDesc(
+            len(tp.irreps_in1), len(tp.irreps_in2), len(tp.irreps_out), len(tp.instructions), in1, in2, out, ins,
+            int(tp.shared_weights), _DTYPES[dtype],
+        )  # fmt: skip
+        handle = _lib.c_void_p()
+        _lib.check(L.e3x_tp_plan_create(ctypes.byref(desc), ctypes.byref(handle)))
+        self.handle = handle
+        wn, fam, key = ctypes.c_int64(), ctypes.c_char_p(), ctypes.c_char_p()
+        _lib.check(L.e3x_tp_plan_info(handle, ctypes.byref(wn), None, None, None, ctypes.byref(fam), ctypes.byref(key)))
+        assert wn.value == tp.weight_numel, (wn.value, tp.weight_numel)
+        self.family, self.key = fam.value.decode(), key.value.decode()
+
+    def __del__(self):
+        try:
+            if self.handle:
+                _lib.lib().e3x_tp_plan_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+class _TensorProductFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x1, x2, w, tp):
+        Z = x1.shape[0]
+        out = torch.empty(Z, tp.irreps_out.dim, dtype=x1.dtype, device=x1.device)
+        plan = tp._plan(x1.dtype)
+        with torch.cuda.device(x1.device):
+            _lib.check(
+                _lib.lib().e3x_tp_forward(
+                    plan.handle, _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(w), _lib.ptr(out), Z, _lib.stream_ptr(x1.device)
+                )
+            )
+        return out
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("the tensor-product backward kernels are not implemented")
+
+
+class _GatherScatterFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, node_x, edge_attr, w, tp, edges):
+        out = torch.empty(edges.num_nodes, tp.irreps_out.dim, dtype=node_x.dtype, device=node_x.device)
+        plan = tp._plan(node_x.dtype)
+        with torch.cuda.device(node_x.device):
+            _lib.check(
+                _lib.lib().e3x_tp_gather_scatter(
+                    plan.handle, _lib.ptr(node_x), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(edges.edge_src),
+                    edges.edge_src.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(out),
+                    edges.num_edges, node_x.shape[0], edges.num_nodes, _lib.stream_ptr(node_x.device),
+                )  # fmt: skip
+            )
+        return out
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("the tensor-product backward kernels are not implemented")
+
+
+class TensorProduct(torch.nn.Module):
+    r"""Tensor product with parametrised paths (see the reference docstring, ``_tensor_product.py:25-194``).
+
+    ``instructions`` is a list of ``(i_in1, i_in2, i_out, mode, has_weight[, path_weight])``.
+    Only the ``uvu`` and ``uvw`` connection modes have kernels; other modes raise
+    ``NotImplementedError`` at construction.
+    """
+
+    def __init__(
+        self,
+        irreps_in1,
+        irreps_in2,
+        irreps_out,
+        instructions: List[tuple],
+        in1_var=None,
+        in2_var=None,
+        out_var=None,
+        irrep_normalization: str = None,
+        path_normalization: str = None,
+        internal_weights: Optional[bool] = None,
+        shared_weights: Optional[bool] = None,
+        compile_left_right: bool = True,
+        compile_right: bool = False,
+        normalization=None,  # for backward compatibility
+        _specialized_code: Optional[bool] = None,
+        _optimize_einsums: Optional[bool] = None,
+    ) -> None:
+        super().__init__()
+        if normalization is not None:
+            warnings.warn("`normalization` is deprecated. Use `irrep_normalization` instead.", DeprecationWarning)
+            irrep_normalization = normalization
+        irrep_normalization = "component" if irrep_normalization is None else irrep_normalization
+        path_normalization = "element" if path_normalization is None else path_normalization
+        assert irrep_normalization in ["component", "norm", "none"]
+        assert path_normalization in ["element", "path", "none"]
+        if compile_right:
+            raise NotImplementedError("TensorProduct.right() has no kernel; construct with compile_right=False")
+
+        self.irreps_in1 = Irreps(irreps_in1)
+        self.irreps_in2 = Irreps(irreps_in2)
+        self.irreps_out = Irreps(irreps_out)
+        i1, i2, io = self.irreps_in1, self.irreps_in2, self.irreps_out
+
+        raw = [tuple(t) if len(t) == 6 else tuple(t) + (1.0,) for t in instructions]
+        for a, b, c, mode, _, _ in raw:
+            assert mode in _MODES
+            assert i1[a].ir.p * i2[b].ir.p == io[c].ir.p
+            assert abs(i1[a].ir.l - i2[b].ir.l) <= io[c].ir.l <= i1[a].ir.l + i2[b].ir.l
+
+        def variances(var, irreps, name):
+            if var is None:
+                return [1.0] * len(irreps)
+            var = [float(v) for v in var]
+            assert len(var) == len(irreps), f"Len of {name} must be equal to len of the irreps"
+            return var
+
+        in1_var = variances(in1_var, i1, "in1_var")
+        in2_var = variances(in2_var, i2, "in2_var")
+        out_var = variances(out_var, io, "out_var")
+
+        # path normalisation: alpha / (sum over the paths into the same output of the number of
+        # summed elements), times the variances and the user path weight; stored as sqrt
+        self.instructions = []
+        for a, b, c, mode, has_weight, pw in raw:
+            alpha = {"component": io[c].ir.dim, "norm": i1[a].ir.dim * i2[b].ir.dim, "none": 1}[irrep_normalization]
+            if path_normalization == "element":
+                x = sum(in1_var[a2] * in2_var[b2] * _num_elements(m, i1[a2].mul, i2[b2].mul) for a2, b2, c2, m, _, _ in raw if c2 == c)
+            elif path_normalization == "path":
+                x = in1_var[a] * in2_var[b] * _num_elements(mode, i1[a].mul, i2[b].mul)
+                x *= len([t for t in raw if t[2] == c])
+            else:
+                x = 1
+            if x > 0.0:
+                alpha /= x
+            alpha *= out_var[c]
+            alpha *= pw
+            self.instructions.append(
+                Instruction(a, b, c, mode, has_weight, sqrt(alpha), _path_shape(mode, i1[a].mul, i2[b].mul, io[c].mul))
+            )
+
+        self._in1_dim, self._in2_dim = i1.dim, i2.dim
+
+        if shared_weights is False and internal_weights is None:
+            internal_weights = False
+        if shared_weights is None:
+            shared_weights = True
+        if internal_weights is None:
+            internal_weights = shared_weights and any(t.has_weight for t in self.instructions)
+        assert shared_weights or not internal_weights
+        self.internal_weights = internal_weights
+        self.shared_weights = shared_weights
+
+        opt = get_optimization_defaults()
+        self._specialized_code = opt["specialized_code"] if _specialized_code is None else _specialized_code
+        self._optimize_einsums = opt["optimize_einsums"] if _optimize_einsums is None else _optimize_einsums
+        self._compile_left_right = compile_left_right
+
+        for t in self.instructions:
+            if t.connection_mode not in _KERNEL_MODES:
+                raise NotImplementedError(
+                    f"connection mode '{t.connection_mode}' has no HIP kernel; implemented modes: uvu, uvw"
+                )
+            if t.connection_mode == "uvu":
+                assert i1[t.i_in1].mul == io[t.i_out].mul
+            if t.connection_mode == "uvw":
+                assert t.has_weight
+        live = {t.connection_mode for t in self.instructions if 0 not in t.path_shape}
+        if len(live) > 1:
+            raise NotImplementedError("mixing uvu and uvw instructions in one TensorProduct has no HIP kernel")
+
+        self.weight_numel = sum(prod(t.path_shape) for t in self.instructions if t.has_weight)
+        if internal_weights and self.weight_numel > 0:
+            assert self.shared_weights, "Having internal weights impose shared weights"
+            self.weight = torch.nn.Parameter(torch.randn(self.weight_numel))
+        else:
+            self.register_buffer("weight", torch.Tensor())
+
+        if io.dim > 0:
+            output_mask = torch.cat(
+                [
+                    torch.ones(mul * ir.dim)
+                    if any(t.i_out == c and t.path_weight != 0 and 0 not in t.path_shape for t in self.instructions)
+                    else torch.zeros(mul * ir.dim)
+                    for c, (mul, ir) in enumerate(io)
+                ]
+            )
+        else:
+            output_mask = torch.ones(0)
+        self.register_buffer("output_mask", output_mask)
+        self._plans = {}
+
+    # ------------------------------------------------------------------ plans
+    def _plan(self, dtype: torch.dtype) -> _Plan:
+        if dtype not in _DTYPES:
+            raise TypeError(f"TensorProduct kernels support float32 and bfloat16 storage, got {dtype}")
+        plan = self._plans.get(dtype)
+        if plan is None:
+            plan = self._plans[dtype] = _Plan(self, dtype)
+        return plan
+
+    def compile(self, dtype: torch.dtype = torch.float32) -> "TensorProduct":
+        """Builds (or finds in the kernel cache) the specialised kernel now; needs no GPU."""
+        self._plan(dtype)
+        return self
+
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        state["_plans"] = {}
+        return state
+
+    def __deepcopy__(self, memo):
+        import copy
+
+        cls = self.__class__
+        new = cls.__new__(cls)
+        memo[id(self)] = new
+        for k, v in self.__dict__.items():
+            new.__dict__[k] = {} if k == "_plans" else copy.deepcopy(v, memo)
+        return new
+
+    def __repr__(self) -> str:
+        npath = sum(prod(t.path_shape) for t in self.instructions)
+        return (
+            f"{self.__class__.__name__}"
+            f"({self.irreps_in1.simplify()} x {self.irreps_in2.simplify()} "
+            f"-> {self.irreps_out.simplify()} | {npath} paths | {self.weight_numel} weights)"
+        )
+
+    # ------------------------------------------------------------------ weights
+    def _prep_weights(self, weight):
+        if isinstance(weight, list):
+            shapes = [t.path_shape for t in self.instructions if t.has_weight]
+            if not self.shared_weights:
+                weight = [w.reshape(-1, prod(s)) for w, s in zip(weight, shapes)]
+            else:
+                weight = [w.reshape(prod(s)) for w, s in zip(weight, shapes)]
+            return torch.cat(weight, dim=-1)
+        return weight
+
+    def _get_weights(self, weight) -> torch.Tensor:
+        weight = self._prep_weights(weight)
+        if weight is None:
+            if self.weight_numel > 0 and not self.internal_weights:
+                raise RuntimeError("Weights must be provided when the TensorProduct does not have `internal_weights`")
+            return self.weight
+        if self.shared_weights:
+            torch._assert(weight.shape == (self.weight_numel,), "Invalid weight shape")
+        else:
+            torch._assert(weight.shape[-1] == self.weight_numel, "Invalid weight shape")
+            torch._assert(weight.ndim > 1, "When shared weights is false, weights must have batch dimension")
+        return weight
+
+    def weight_view_for_instruction(self, instruction: int, weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if not self.instructions[instruction].has_weight:
+            raise ValueError(f"Instruction {instruction} has no weights.")
+        offset = sum(prod(t.path_shape) for t in self.instructions[:instruction])
+        t = self.instructions[instruction]
+        weight = self._get_weights(weight)
+        return weight.narrow(-1, offset, prod(t.path_shape)).view(weight.shape[:-1] + t.path_shape)
+
+    def weight_views(self, weight: Optional[torch.Tensor] = None, yield_instruction: bool = False):
+        weight = self._get_weights(weight)
+        batchshape = weight.shape[:-1]
+        offset = 0
+        for i, t in enumerate(self.instructions):
+            if t.has_weight:
+                n = prod(t.path_shape)
+                view = weight.narrow(-1, offset, n).view(batchshape + t.path_shape)
+                offset += n
+                yield (i, t, view) if yield_instruction else view
+
+    # ------------------------------------------------------------------ evaluation
+    def right(self, y, weight=None):
+        raise NotImplementedError("TensorProduct.right() has no HIP kernel")
+
+    def _check_device(self, *tensors):
+        for t in tensors:
+            if not t.is_cuda:
+                raise RuntimeError("e3nn_amd.o3.TensorProduct runs on the GPU only; got a CPU tensor")
+
+    def forward(self, x, y, weight: Optional[Union[torch.Tensor, List[torch.Tensor]]] = None):
+        r"""Evaluate :math:`w x \otimes y`: ``x[..., irreps_in1.dim]``, ``y[..., irreps_in2.dim]``,
+        ``weight[weight_numel]`` (shared) or ``weight[..., weight_numel]`` -> ``[..., irreps_out.dim]``."""
+        torch._assert(x.shape[-1] == self._in1_dim, "Incorrect last dimension for x")
+        torch._assert(y.shape[-1] == self._in2_dim, "Incorrect last dimension for y")
+        torch._assert(self._compile_left_right, "`left_right` method is not compiled, set `compile_left_right` to True when creating the TensorProduct")
+        w = self._get_weights(weight)
+        self._check_device(x, y)
+        if w.numel() and w.device != x.device:
+            raise RuntimeError("weights and inputs must be on the same device")
+        # broadcast all batch dimensions (everything but the last)
+        if self.shared_weights or self.weight_numel == 0:
+            batch = torch.broadcast_shapes(x.shape[:-1], y.shape[:-1])
+        else:
+            batch = torch.broadcast_shapes(x.shape[:-1], y.shape[:-1], w.shape[:-1])
+        x1 = x.expand(batch + (-1,)).reshape(-1, self._in1_dim).contiguous()
+        x2 = y.expand(batch + (-1,)).reshape(-1, self._in2_dim).to(x1.dtype).contiguous()
+        if self.weight_numel == 0:
+            wf = x1.new_empty(0)
+        elif self.shared_weights:
+            wf = w.to(x1.dtype).contiguous()
+        else:
+            wf = w.expand(batch + (-1,)).reshape(-1, self.weight_numel).to(x1.dtype).contiguous()
+        out = _TensorProductFn.apply(x1, x2, wf, self)
+        return out.reshape(batch + (self.irreps_out.dim,))
+
+    def forward_gather_scatter(
+        self,
+        node_x: torch.Tensor,
+        edge_attr: torch.Tensor,
+        weight: torch.Tensor,
+        edge_src: Optional[torch.Tensor] = None,
+        edge_dst: Optional[torch.Tensor] = None,
+        num_nodes: Optional[int] = None,
+        edges: Optional[DstSortedEdges] = None,
+    ) -> torch.Tensor:
+        """``scatter(self(node_x[edge_src], edge_attr, weight), edge_dst, num_nodes)`` in one kernel.
+
+        ``node_x[N_src, irreps_in1.dim]``, ``edge_attr[E, irreps_in2.dim]``, ``weight[E, weight_numel]``
+        (per-edge weights, ``shared_weights=False``); result ``[num_nodes, irreps_out.dim]``.
+        Pass a prebuilt ``DstSortedEdges`` as ``edges`` to amortise the index preprocessing
+        over several calls on the same graph.
+        """
+        if any(t.connection_mode != "uvu" for t in self.instructions):
+            raise NotImplementedError("forward_gather_scatter needs an all-uvu TensorProduct")
+        torch._assert(node_x.ndim == 2 and node_x.shape[-1] == self._in1_dim, "Incorrect shape for node_x")
+        torch._assert(edge_attr.ndim == 2 and edge_attr.shape[-1] == self._in2_dim, "Incorrect shape for edge_attr")
+        self._check_device(node_x, edge_attr)
+        if edges is None:
+            edges = DstSortedEdges(edge_src, edge_dst, node_x.shape[0] if num_nodes is None else num_nodes, node_x.shape[0])
+        torch._assert(edge_attr.shape[0] == edges.num_edges, "edge_attr must have one row per edge")
+        torch._assert(edges.num_src_nodes == node_x.shape[0], "edge list was built for another node count")
+        if self.weight_numel:
+            torch._assert(not self.shared_weights, "forward_gather_scatter needs per-edge weights (shared_weights=False)")
+            w = self._get_weights(weight)
+            torch._assert(w.shape == (edges.num_edges, self.weight_numel), "Invalid weight shape")
+            w = w.to(node_x.dtype).contiguous()
+        else:
+            w = node_x.new_empty(0)
+        return _GatherScatterFn.apply(node_x.contiguous(), edge_attr.to(node_x.dtype).contiguous(), w, self, edges)
+
+
+class FullyConnectedTensorProduct(TensorProduct):
+    r"""All paths allowed by :math:`|l_1 - l_2| \leq l_{out} \leq l_1 + l_2`, mode ``uvw``, weighted
+    (reference ``_sub.py:46-68``)."""
+
+    def __init__(self, irreps_in1, irreps_in2, irreps_out, irrep_normalization: str = None, path_normalization: str = None, **kwargs) -> None:
+        irreps_in1, irreps_in2, irreps_out = Irreps(irreps_in1), Irreps(irreps_in2), Irreps(irreps_out)
+        instr = [
+            (i_1, i_2, i_out, "uvw", True, 1.0)
+            for i_1, (_, ir_1) in enumerate(irreps_in1)
+            for i_2, (_, ir_2) in enumerate(irreps_in2)
+            for i_out, (_, ir_out) in enumerate(irreps_out)
+            if ir_out in ir_1 * ir_2
+        ]
+        super().__init__(
+            irreps_in1, irreps_in2, irreps_out, instr,
+            irrep_normalization=irrep_normalization, path_normalization=path_normalization, **kwargs,
+        )  # fmt: skip

@@ -1,0 +1,138 @@
+/*
+ * e3x — C ABI of the MI355X-native equivariant message-passing hot path.
+ *
+ * Plain pointers and sizes only.  Every device pointer is caller-owned memory on the
+ * current HIP device; the library allocates no device memory and frees nothing it did
+ * not create.  All launches are asynchronous on the `stream` argument (a hipStream_t
+ * passed as void*; NULL is the default stream).  Functions return 0 on success and a
+ * negative E3X_ERR_* code otherwise; e3x_last_error() gives the message for the calling
+ * thread.  Feature layout is the reference's: irreps concatenated in order, each block
+ * row-major [mul, 2l+1] (reference e3nn/o3/_tensor_product/_codegen.py:82-94, :314).
+ *
+ * File:line citations name the reference function each entry point replaces
+ * (paths relative to the e3nn source tree).
+ */
+#ifndef E3X_H
+#define E3X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define E3X_OK 0
+#define E3X_ERR_INVALID (-1)     /* bad argument / unsupported instruction set */
+#define E3X_ERR_COMPILE (-2)     /* kernel specialisation could not be built */
+#define E3X_ERR_HIP (-3)         /* a HIP runtime call failed */
+#define E3X_ERR_INDEX (-4)       /* edge index out of range */
+
+/* storage type of features / weights / outputs; accumulation is always fp32 */
+#define E3X_F32 0
+#define E3X_BF16 1
+
+/* connection modes (reference _tensor_product.py:245-254) */
+#define E3X_MODE_UVW 0
+#define E3X_MODE_UVU 1
+
+/* spherical-harmonics output normalisation (reference _spherical_harmonics.py:103-110) */
+#define E3X_NORM_INTEGRAL 0
+#define E3X_NORM_COMPONENT 1
+#define E3X_NORM_NORM 2
+
+typedef struct {
+  int32_t mul; /* multiplicity */
+  int32_t l;   /* degree */
+  int32_t p;   /* parity, +1 or -1 */
+} e3x_irrep;
+
+/* One row of TensorProduct.instructions (reference _tensor_product/_instruction.py:4-11)
+ * after normalisation: path_weight is sqrt(alpha) of _tensor_product.py:289-324. */
+typedef struct {
+  int32_t i_in1, i_in2, i_out;
+  int32_t mode;       /* E3X_MODE_* */
+  int32_t has_weight; /* 0 / 1 */
+  double path_weight;
+} e3x_instruction;
+
+typedef struct {
+  int32_t n_in1, n_in2, n_out, n_ins;
+  const e3x_irrep* in1;
+  const e3x_irrep* in2;
+  const e3x_irrep* out;
+  const e3x_instruction* ins;
+  int32_t shared_weights; /* 1: w is [weight_numel]; 0: w is [Z, weight_numel] */
+  int32_t dtype;          /* E3X_F32 / E3X_BF16 storage of x1, x2, w, out */
+} e3x_tp_desc;
+
+typedef struct e3x_plan e3x_plan;
+
+const char* e3x_last_error(void);
+int e3x_version(void);
+
+/* Real-basis Wigner 3j tensor, out[(2l1+1)(2l2+1)(2l3+1)] row-major doubles, Frobenius
+ * norm 1.  Host only.  Replaces o3.wigner_3j (e3nn/o3/_wigner.py:102-164). */
+int e3x_wigner_3j(int l1, int l2, int l3, double* out);
+
+/* Builds (or finds in the on-disk kernel cache) the fused kernel specialised to one
+ * instruction set: the role of codegen_tensor_product_left_right
+ * (e3nn/o3/_tensor_product/_codegen.py:24-395) behind the provider hook
+ * _CODEGEN_PROVIDERS_LEFT_RIGHT (e3nn/o3/_tensor_product/_tensor_product.py:17-21,348-361).
+ * Needs a HIP compiler only on a cache miss; needs no GPU (the code object is loaded on
+ * first launch).  The cache directory is $E3X_KERNEL_CACHE or <library dir>/../kernel_cache. */
+int e3x_tp_plan_create(const e3x_tp_desc* desc, e3x_plan** out);
+int e3x_tp_plan_destroy(e3x_plan* plan);
+/* weight_numel (reference _tensor_product.py:403), in1/in2/out dims, and the kernel family
+ * name ("uvu", "uvw_small", "uvw_mfma"); any out pointer may be NULL. */
+int e3x_tp_plan_info(const e3x_plan* plan, int64_t* weight_numel, int64_t* in1_dim, int64_t* in2_dim,
+                     int64_t* out_dim, const char** family, const char** cache_key);
+
+/* out[Z, out_dim] = TP(x1[Z, in1_dim], x2[Z, in2_dim], w).  Replaces the generated
+ * module called at e3nn/o3/_tensor_product/_tensor_product.py:554
+ * (contraction: _codegen.py:148-187, path weights :312, sum/cat :327-343).
+ * `out` is fully overwritten (output irreps no instruction reaches become 0). */
+int e3x_tp_forward(e3x_plan* plan, const void* x1, const void* x2, const void* w, void* out, int64_t Z,
+                   void* stream);
+
+/* Destination-sorted edge list for the fused scatter: stable sort of edge ids by dst.
+ * rowptr[num_nodes+1], perm[E] are int32 device arrays owned by the caller;
+ * `workspace` is device scratch of at least e3x_csr_workspace_bytes(E, num_nodes).
+ * Indices are int32 (idx_bits = 32) or int64 (idx_bits = 64) and must lie in
+ * [0, num_nodes): scatter_add_ semantics (e3nn/nn/models/v2106/points_convolution.py:13-17).
+ * Synchronises the stream once to report E3X_ERR_INDEX for out-of-range indices. */
+size_t e3x_csr_workspace_bytes(int64_t E, int64_t num_nodes);
+int e3x_csr_build(const void* dst, int idx_bits, int64_t E, int64_t num_nodes, int32_t* rowptr, int32_t* perm,
+                  void* workspace, size_t workspace_bytes, void* stream);
+/* Checks gather indices the way torch advanced indexing does (x[edge_src],
+ * points_convolution.py:105): values in [-num_nodes, num_nodes) are valid, negative
+ * ones wrap.  Synchronises the stream. */
+int e3x_index_check(const void* idx, int idx_bits, int64_t E, int64_t num_nodes, void* stream);
+
+/* out[n, out_dim] = sum over edges e with dst[e] == n of TP(node_x[src[e]], edge_attr[e], w[e]),
+ * i.e. scatter(tp(node_features[edge_src], edge_attr, weight), edge_dst, N) of
+ * e3nn/nn/models/v2106/points_convolution.py:105-106, with neither [E, .] tensor
+ * materialised.  rowptr / perm come from e3x_csr_build (perm may be NULL when the
+ * edges are already grouped by destination in rowptr order).  Within a row, edges are
+ * summed in perm order by a fixed reduction tree: results are bit-reproducible.
+ * `out` is fully overwritten; rows without in-edges become 0.  Only for plans whose
+ * instructions are all `uvu`. */
+int e3x_tp_gather_scatter(e3x_plan* plan, const void* node_x, const void* edge_attr, const void* w,
+                          const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm, void* out,
+                          int64_t E, int64_t num_src_nodes, int64_t num_out_nodes, void* stream);
+
+/* out[n, sum(2l+1 for l in ls)] = spherical harmonics of xyz[n, 3].  Replaces
+ * SphericalHarmonics.forward (e3nn/o3/_spherical_harmonics.py:93-112) and the polynomial
+ * chain _spherical_harmonics (:193-249 for l <= 3, recurrence of
+ * _spherical_harmonics_generator.py:57-65 above).  max(ls) <= 8. */
+int e3x_sh_forward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization, const void* xyz,
+                   void* out, int64_t n, int32_t dtype, void* stream);
+
+/* Plain device copy dst[i] = src[i], n_bytes multiple of 16: the calibration kernel
+ * for bandwidth counters (known traffic: n_bytes read + n_bytes written). */
+int e3x_copy_bytes(const void* src, void* dst, size_t n_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* E3X_H */

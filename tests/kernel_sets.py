@@ -1,0 +1,102 @@
+"""Every instruction set the GPU tests, the smoke check and the benchmark run.
+
+One place, so that the build step can compile all of their kernels into the in-tree
+cache before anything runs on a GPU.
+"""
+import json
+import os
+
+import torch
+
+from e3nn_amd import o3
+from e3nn_amd.nn.message import message_tensor_product
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+SH2 = str(o3.Irreps.spherical_harmonics(2))
+SH3 = str(o3.Irreps.spherical_harmonics(3))
+
+GOLDEN_GPU_CASES = [
+    "fctp_cfg1", "fctp_small_cfg5_like", "fctp_per_sample_weights", "fctp_norm_path",
+    "uvu_merged_cfg3_like_mul4", "uvu_builder_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2",
+    "uvu_builderB_cfg4_like_mul2", "uvu_shared_v2", "uvu_mixed_weightless", "empty_path_and_missing_output",
+    "conv_small",
+]  # fmt: skip
+
+
+def golden_meta():
+    with open(os.path.join(GOLDEN, "tp_cases.json")) as f:
+        return json.load(f)
+
+
+def tp_from_meta(m):
+    upw = m.get("user_path_weights", [1.0] * len(m["instructions"]))
+    ins = [tuple(t[:5]) + (pw,) for t, pw in zip(m["instructions"], upw)]
+    kw = {}
+    if m.get("irrep_normalization"):
+        kw = dict(irrep_normalization=m["irrep_normalization"], path_normalization=m["path_normalization"])
+    return o3.TensorProduct(
+        m["irreps_in1"], m["irreps_in2"], m["irreps_out"], ins,
+        internal_weights=m["internal_weights"], shared_weights=m["shared_weights"], **kw,
+    )  # fmt: skip
+
+
+def golden_tp(name, meta=None):
+    m = dict((meta or golden_meta())[name])
+    if name == "fctp_norm_path":
+        m.update(irrep_normalization="norm", path_normalization="path")
+    return tp_from_meta(m)
+
+
+def cfg1():
+    return o3.FullyConnectedTensorProduct("16x0e+16x1o", "0e+1o+2e", "16x0e+16x1o+16x2e")
+
+
+def cfg3(merged=True):
+    f = "32x0e+32x1o+32x2e"
+    return message_tensor_product(f, SH2, irreps_out=f) if merged else message_tensor_product(f, SH2, keep="0e+1o+2e")
+
+
+def cfg4(variant="A"):
+    f = "128x0e+128x1o+128x2e+128x3o"
+    keep = "0e+1o+2e+3o" if variant == "A" else "0e+0o+1e+1o+2e+2o+3e+3o"
+    return message_tensor_product(f, SH3, keep=keep)
+
+
+def cfg5():
+    f = "128x0e+128x1o+128x2e"
+    return o3.FullyConnectedTensorProduct(f, f, f)
+
+
+def scalar_exact():
+    # 1x1 Clebsch-Gordan, path weight 1: products and sums of small integers are exact in fp32
+    return message_tensor_product("32x0e", "0e", irreps_out="32x0e")
+
+
+def odd_mul():
+    # multiplicities that are no multiple of the lane-group width, several chunks
+    return message_tensor_product("80x0e+24x1o+5x2e", SH2, keep="0e+1o+2e")
+
+
+def all_tensor_products():
+    """(name, TensorProduct, dtypes) for everything that must be in the kernel cache."""
+    meta = golden_meta()
+    out = [(n, golden_tp(n, meta), (torch.float32,)) for n in GOLDEN_GPU_CASES]
+    out += [
+        ("cfg1", cfg1(), (torch.float32,)),
+        ("cfg3_merged", cfg3(True), (torch.float32, torch.bfloat16)),
+        ("cfg3_builder", cfg3(False), (torch.float32,)),
+        ("cfg4_A", cfg4("A"), (torch.float32, torch.bfloat16)),
+        ("cfg4_B", cfg4("B"), (torch.float32,)),
+        ("scalar_exact", scalar_exact(), (torch.float32,)),
+        ("odd_mul", odd_mul(), (torch.float32,)),
+    ]
+    return out
+
+
+def prebuild(verbose=True):
+    for name, tp, dtypes in all_tensor_products():
+        for dt in dtypes:
+            plan = tp._plan(dt)
+            if verbose:
+                print(f"kernel {name:32s} {str(dt):16s} {plan.key}", flush=True)

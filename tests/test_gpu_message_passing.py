@@ -1,0 +1,144 @@
+"""GPU parity: fused gather -> uvu tensor product -> scatter-sum against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from e3nn_amd import o3
+from e3nn_amd.nn import DstSortedEdges
+from oracle import tensor_product as otp
+from oracle.message_passing import tp_gather_scatter
+from tests import kernel_sets as ks
+from tests.helpers import assert_close, oracle_spec, seeded
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def random_graph(N, E, seed=0, dtype=torch.int64):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, N, (E,), generator=g).to(dtype), torch.randint(0, N, (E,), generator=g).to(dtype)
+
+
+def test_conv_matches_reference_golden(golden_tp):
+    meta, arr = golden_tp
+    tp = ks.golden_tp("conv_small", meta)
+    g = {k.split("/")[1]: torch.from_numpy(v) for k, v in arr.items() if k.startswith("conv_small/")}
+    attr = o3.spherical_harmonics([0, 1, 2], g["vec"].float().to(DEV), True, "component")
+    assert_close(attr, g["attr"].numpy(), what="edge attrs")
+    out = tp.forward_gather_scatter(
+        g["node_x"].float().to(DEV), attr, g["w"].float().to(DEV), g["src"].to(DEV), g["dst"].to(DEV), g["node_x"].shape[0]
+    )
+    assert_close(out, g["out"].numpy(), what="conv_small")
+    assert not out[-1].any()  # the last node receives no edge: exact zeros
+
+
+def test_index_handling_is_bit_exact():
+    # 1x1 Clebsch-Gordan and path weight 1: with small-integer payloads every product and every
+    # partial sum is an exact fp32 integer, so the result is independent of summation order
+    tp = ks.scalar_exact()
+    assert abs(tp.instructions[0].path_weight - 1.0) < 1e-15
+    N, E = 301, 20_000
+    g = torch.Generator().manual_seed(5)
+    node_x = torch.randint(-8, 9, (N, 32), generator=g).float()
+    attr = torch.randint(-4, 5, (E, 1), generator=g).float()
+    w = torch.randint(-4, 5, (E, 32), generator=g).float()
+    src, dst = random_graph(N, E, seed=6)
+    dst = torch.where(dst >= N - 3, dst - 3, dst)  # nodes N-3.. receive nothing
+    ref = np.zeros((N, 32), dtype=np.float64)
+    np.add.at(ref, dst.numpy(), (w * node_x[src] * attr).double().numpy())
+    outs = []
+    for dt in (torch.int64, torch.int32):
+        out = tp.forward_gather_scatter(node_x.to(DEV), attr.to(DEV), w.to(DEV), src.to(dt).to(DEV), dst.to(dt).to(DEV), N)
+        assert np.array_equal(out.cpu().numpy().astype(np.float64), ref)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    assert not outs[0][N - 3 :].any()
+    # negative source indices wrap like torch advanced indexing
+    out = tp.forward_gather_scatter(node_x.to(DEV), attr.to(DEV), w.to(DEV), (src - N).to(DEV), dst.to(DEV), N)
+    assert torch.equal(out, outs[0])
+    # already grouped by destination, and the reverse order: same exact sums
+    order = torch.argsort(dst, stable=True)
+    for o in (order, order.flip(0)):
+        out = tp.forward_gather_scatter(node_x.to(DEV), attr[o].to(DEV), w[o].to(DEV), src[o].to(DEV), dst[o].to(DEV), N)
+        assert torch.equal(out, outs[0])
+
+
+def test_out_of_range_indices_raise_and_empty_graph():
+    tp = ks.scalar_exact()
+    N, E = 10, 50
+    src, dst = random_graph(N, E, seed=1)
+    node_x, attr, w = seeded(N, 32).to(DEV), seeded(E, 1).to(DEV), seeded(E, 32).to(DEV)
+    bad = dst.clone()
+    bad[7] = N
+    with pytest.raises(IndexError):
+        tp.forward_gather_scatter(node_x, attr, w, src.to(DEV), bad.to(DEV), N)
+    bad = dst.clone()
+    bad[7] = -1  # scatter_add_ does not wrap
+    with pytest.raises(IndexError):
+        tp.forward_gather_scatter(node_x, attr, w, src.to(DEV), bad.to(DEV), N)
+    bad = src.clone()
+    bad[3] = N
+    with pytest.raises(IndexError):
+        tp.forward_gather_scatter(node_x, attr, w, bad.to(DEV), dst.to(DEV), N)
+    bad[3] = -N - 1
+    with pytest.raises(IndexError):
+        tp.forward_gather_scatter(node_x, attr, w, bad.to(DEV), dst.to(DEV), N)
+    e = torch.zeros(0, dtype=torch.int64, device=DEV)
+    out = tp.forward_gather_scatter(node_x, attr[:0], w[:0], e, e, N)
+    assert out.shape == (N, 32) and not out.any()
+
+
+def test_run_to_run_bit_reproducible_and_prebuilt_edges():
+    tp = ks.cfg3(True)
+    N, E = 500, 20_000
+    src, dst = random_graph(N, E, seed=2)
+    node_x, attr, w = seeded(N, 288, seed=1).to(DEV), seeded(E, 9, seed=2).to(DEV), seeded(E, 352, seed=3).to(DEV)
+    edges = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    assert edges.rowptr[-1].item() == E and edges.rowptr[0].item() == 0
+    # stable sort: perm lists the edges of each destination in their original order
+    perm = edges.perm.cpu().long()
+    assert torch.equal(perm, torch.argsort(dst, stable=True))
+    a = tp.forward_gather_scatter(node_x, attr, w, edges=edges)
+    b = tp.forward_gather_scatter(node_x, attr, w, src.to(DEV), dst.to(DEV), N)
+    assert torch.equal(a, b)
+    assert torch.equal(a, tp.forward_gather_scatter(node_x, attr, w, edges=edges))
+
+
+@pytest.mark.parametrize("maker,N,E,idx", [
+    (lambda: ks.cfg3(True), 700, 26_000, torch.int64),
+    (lambda: ks.cfg3(False), 300, 9_000, torch.int64),
+    (lambda: ks.cfg4("A"), 60, 1_500, torch.int32),
+    (lambda: ks.cfg4("B"), 40, 700, torch.int32),
+    (ks.odd_mul, 90, 2_000, torch.int32),
+])  # fmt: skip
+def test_fused_matches_oracle(maker, N, E, idx):
+    tp = maker()
+    src, dst = random_graph(N, E, seed=3, dtype=idx)
+    node_x = seeded(N, tp.irreps_in1.dim, seed=1)
+    vec = seeded(E, 3, seed=2)
+    lmax = tp.irreps_in2.lmax
+    attr = o3.spherical_harmonics(list(range(lmax + 1)), vec.to(DEV), True, "component")
+    w = seeded(E, tp.weight_numel, seed=4)
+    out = tp.forward_gather_scatter(node_x.to(DEV), attr, w.to(DEV), src.to(DEV), dst.to(DEV), N)
+    ref = tp_gather_scatter(oracle_spec(tp), node_x.numpy(), attr.cpu().numpy(), w.numpy(), src.numpy(), dst.numpy(), N)
+    # sums of ~E/N messages of magnitude up to ~50: tolerance scales with the accumulated magnitude
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert_close(out, ref, atol=1e-4 * scale ** 0.5, rtol=1e-5, what=str(tp))
+    # same thing as the unfused product path
+    msg = tp(node_x.to(DEV)[src.long().to(DEV)], attr, w.to(DEV))
+    unfused = torch.zeros_like(out).index_add_(0, dst.long().to(DEV), msg)
+    assert (out - unfused).abs().max().item() < 1e-4 * scale
+
+
+def test_fused_bf16_storage():
+    tp = ks.cfg4("A")
+    N, E = 50, 1000
+    src, dst = random_graph(N, E, seed=9, dtype=torch.int32)
+    node_x, attr, w = seeded(N, 2048, seed=1), seeded(E, 16, seed=2), seeded(E, 2944, seed=3)
+    nb, ab, wb = (t.to(DEV).to(torch.bfloat16) for t in (node_x, attr, w))
+    out = tp.forward_gather_scatter(nb, ab, wb, src.to(DEV), dst.to(DEV), N)
+    ref = tp_gather_scatter(
+        oracle_spec(tp), nb.float().cpu().numpy(), ab.float().cpu().numpy(), wb.float().cpu().numpy(), src.numpy(), dst.numpy(), N
+    )
+    scale = float(np.abs(ref).max())
+    assert_close(out, ref, atol=1e-2 * scale, rtol=1e-2, what="bf16 fused")

@@ -1,0 +1,137 @@
+"""GPU parity: o3.TensorProduct / FullyConnectedTensorProduct (HIP, through the C ABI) against the CPU oracle
+and the golden outputs written from the reference."""
+import numpy as np
+import pytest
+import torch
+
+from e3nn_amd import o3
+from oracle import tensor_product as otp
+from tests import kernel_sets as ks
+from tests.helpers import assert_close, oracle_spec, seeded
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+PLAIN_CASES = [c for c in ks.GOLDEN_GPU_CASES if c != "conv_small"]
+
+
+@pytest.mark.parametrize("name", PLAIN_CASES)
+def test_matches_reference_golden(golden_tp, name):
+    meta, arr = golden_tp
+    tp = ks.golden_tp(name, meta).to(DEV)
+    x1 = torch.from_numpy(arr[name + "/x1"]).float().to(DEV)
+    x2 = torch.from_numpy(arr[name + "/x2"]).float().to(DEV)
+    w = torch.from_numpy(arr[name + "/w"]).float().to(DEV)
+    if tp.internal_weights:
+        with torch.no_grad():
+            tp.weight.copy_(w)
+        out = tp(x1, x2)
+    elif tp.weight_numel:
+        out = tp(x1, x2, w)
+    else:
+        out = tp(x1, x2)
+    assert_close(out, arr[name + "/out"], what=name)
+    # structure against the reference's tables
+    m = meta[name]
+    assert tp.weight_numel == m["weight_numel"]
+    for t, ref in zip(tp.instructions, m["instructions"]):
+        assert abs(t.path_weight - ref[5]) < 1e-14 and list(t.path_shape) == ref[6]
+    for sl, flag in zip(tp.irreps_out.slices(), m["output_mask_blocks"]):
+        if flag >= 0:
+            assert (tp.output_mask[sl] == flag).all()
+
+
+def test_cfg1_full_size_against_oracle():
+    # FCTP('16x0e+16x1o', '0e+1o+2e' -> '16x0e+16x1o+16x2e'), batch 4096, x2 = SH(lmax 2) of unit vectors, seed 0
+    g = torch.Generator().manual_seed(0)
+    tp = ks.cfg1().to(DEV)
+    w = torch.randn(tp.weight_numel, generator=g)
+    x1 = torch.randn(4096, 64, generator=g)
+    v = torch.randn(4096, 3, generator=g)
+    v = v / v.norm(dim=1, keepdim=True)
+    x2 = o3.spherical_harmonics([0, 1, 2], v.to(DEV), True, "component")
+    with torch.no_grad():
+        tp.weight.copy_(w)
+    out = tp(x1.to(DEV), x2)
+    ref = otp.tp_forward(oracle_spec(tp), x1.numpy(), x2.cpu().numpy(), w.numpy())
+    assert_close(out, ref, what="cfg1")
+    assert abs(out.var().item() - 1) < 0.2  # unit output variance
+
+
+def test_batch_broadcasting_weight_lists_and_errors():
+    tp = ks.golden_tp("fctp_per_sample_weights").to(DEV)  # shared_weights=False
+    spec = oracle_spec(tp)
+    x1 = seeded(3, 1, tp.irreps_in1.dim, seed=1)
+    x2 = seeded(1, 4, tp.irreps_in2.dim, seed=2)
+    w = seeded(3, 4, tp.weight_numel, seed=3)
+    out = tp(x1.to(DEV), x2.to(DEV), w.to(DEV))
+    assert out.shape == (3, 4, tp.irreps_out.dim)
+    ref = otp.tp_forward(
+        spec, x1.expand(3, 4, -1).reshape(12, -1).numpy(), x2.expand(3, 4, -1).reshape(12, -1).numpy(), w.reshape(12, -1).numpy()
+    ).reshape(3, 4, -1)
+    assert_close(out, ref)
+    # weights given as a list of per-instruction tensors
+    wl = [v.contiguous() for v in tp.weight_views(w.to(DEV))]
+    assert torch.equal(tp(x1.to(DEV), x2.to(DEV), wl), out)
+    with pytest.raises(RuntimeError):
+        tp(x1.to(DEV), x2.to(DEV))  # external weights are mandatory
+    with pytest.raises(RuntimeError):
+        tp(x1.to(DEV), x2.to(DEV), w.to(DEV)[..., :-1])
+    with pytest.raises(RuntimeError):
+        tp(x1.to(DEV), x2.to(DEV), w.to(DEV)[0, 0])  # no batch dimension on per-sample weights
+    with pytest.raises(RuntimeError):
+        tp(x1.to(DEV)[..., :-1], x2.to(DEV), w.to(DEV))
+    with pytest.raises(RuntimeError):
+        tp(x1, x2, w)  # CPU tensors: no silent fallback
+    shared = ks.golden_tp("fctp_cfg1").to(DEV)
+    with pytest.raises(RuntimeError):
+        shared(seeded(2, 64).to(DEV), seeded(2, 9).to(DEV), seeded(2, shared.weight_numel).to(DEV))
+    # empty batch
+    assert shared(torch.zeros(0, 64, device=DEV), torch.zeros(0, 9, device=DEV)).shape == (0, 144)
+
+
+def test_missing_output_paths_are_exact_zeros():
+    tp = ks.golden_tp("empty_path_and_missing_output").to(DEV)
+    out = tp(seeded(6, tp.irreps_in1.dim).to(DEV), seeded(6, tp.irreps_in2.dim, seed=1).to(DEV))
+    sl = tp.irreps_out.slices()[1]
+    assert not out[:, sl].any() and out[:, tp.irreps_out.slices()[0]].any()
+    assert tp.output_mask[sl].sum() == 0
+
+
+def test_bilinearity_and_weight_linearity():
+    tp = ks.cfg3(True)
+    Z = 257
+    x1, x1b = seeded(Z, 288, seed=1).to(DEV), seeded(Z, 288, seed=2).to(DEV)
+    x2 = seeded(Z, 9, seed=3).to(DEV)
+    w, wb = seeded(Z, 352, seed=4).to(DEV), seeded(Z, 352, seed=5).to(DEV)
+    a = tp(x1 + 0.5 * x1b, x2, w)
+    b = tp(x1, x2, w) + 0.5 * tp(x1b, x2, w)
+    assert (a - b).abs().max().item() < 2e-5
+    a = tp(x1, x2, w + 2 * wb)
+    b = tp(x1, x2, w) + 2 * tp(x1, x2, wb)
+    assert (a - b).abs().max().item() < 5e-5
+
+
+@pytest.mark.parametrize("maker,Z", [(lambda: ks.cfg3(True), 1000), (lambda: ks.cfg3(False), 333), (lambda: ks.cfg4("A"), 130),
+                                     (lambda: ks.cfg4("B"), 70), (ks.odd_mul, 129)])  # fmt: skip
+def test_plain_uvu_benchmark_instruction_sets(maker, Z):
+    tp = maker()
+    x1 = seeded(Z, tp.irreps_in1.dim, seed=11)
+    x2 = seeded(Z, tp.irreps_in2.dim, seed=12)
+    w = seeded(Z, tp.weight_numel, seed=13)
+    out = tp(x1.to(DEV), x2.to(DEV), w.to(DEV))
+    ref = otp.tp_forward(oracle_spec(tp), x1.numpy(), x2.numpy(), w.numpy())
+    # |out| reaches ~50 for these un-normalised random inputs: the relative term matters
+    assert_close(out, ref, atol=1e-4, rtol=1e-5, what=str(tp))
+
+
+def test_bf16_storage_variant():
+    tp = ks.cfg3(True)
+    Z = 500
+    x1, x2, w = seeded(Z, 288, seed=1), seeded(Z, 9, seed=2), seeded(Z, 352, seed=3)
+    xb, yb, wb = (t.to(DEV).to(torch.bfloat16) for t in (x1, x2, w))
+    out = tp(xb, yb, wb)
+    assert out.dtype == torch.bfloat16
+    # oracle on the bf16-rounded inputs; the output is rounded to bf16 once
+    ref = otp.tp_forward(oracle_spec(tp), xb.float().cpu().numpy(), yb.float().cpu().numpy(), wb.float().cpu().numpy())
+    assert_close(out, ref, atol=1e-2, rtol=1e-2, what="bf16 storage")

@@ -1,0 +1,154 @@
+"""CPU-only tests: the C-ABI library loads and exports what include/e3x.h declares, host-side
+functions (Wigner 3j, plan creation) and the Python mirror of the reference API."""
+import copy
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from e3nn_amd import _lib, get_optimization_defaults, o3, set_optimization_defaults
+from e3nn_amd.nn.message import message_instructions, message_tensor_product
+from oracle import tensor_product as otp
+from oracle.wigner import wigner_3j as oracle_w3j
+from tests import kernel_sets as ks
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "e3x.h")).read()
+    declared = set(re.findall(r"\b(e3x_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 12
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), f"{name} declared in e3x.h but not exported"
+    assert declared == set(_lib._SIGNATURES), "ctypes signatures out of sync with e3x.h"
+    assert _lib.lib().e3x_version() >= 100
+
+
+def test_wigner_3j_matches_oracle_and_golden(golden_w3j):
+    for key, ref in golden_w3j.items():
+        l1, l2, l3 = map(int, key.split("_"))
+        got = o3.wigner_3j(l1, l2, l3, dtype=torch.float64).numpy()
+        np.testing.assert_allclose(got, ref, atol=1e-13)
+    for l1, l2, l3 in ((6, 5, 3), (8, 8, 8), (10, 9, 4), (12, 1, 11)):
+        np.testing.assert_allclose(o3.wigner_3j(l1, l2, l3, dtype=torch.float64).numpy(), oracle_w3j(l1, l2, l3), atol=1e-13)
+    assert o3.wigner_3j(1, 1, 1).dtype == torch.get_default_dtype()
+    with pytest.raises(AssertionError):
+        o3.wigner_3j(1, 1, 3)
+    buf = (ctypes.c_double * 27)()
+    assert _lib.lib().e3x_wigner_3j(1, 1, 3, buf) != 0
+    assert b"l1" in _lib.lib().e3x_last_error()
+
+
+def test_irreps_api():
+    assert repr(o3.Irrep("1y")) == "1o" and o3.Irrep("2o").dim == 5
+    assert o3.Irrep("2e") in list(o3.Irrep("1o") * o3.Irrep("1o"))
+    assert repr(o3.Irrep("1o") + o3.Irrep("2o")) == "1x1o+1x2o"
+    it = o3.Irrep.iterator()
+    assert [repr(next(it)) for _ in range(4)] == ["0e", "0o", "1o", "1e"]
+    irreps = o3.Irreps("2x0e + 1e")
+    assert irreps.slices() == [slice(0, 2), slice(2, 5)] and irreps.dim == 5 and irreps.num_irreps == 3
+    assert repr(o3.Irreps.spherical_harmonics(3)) == "1x0e+1x1o+1x2e+1x3o"
+    assert repr(o3.Irreps.spherical_harmonics(4, p=1)) == "1x0e+1x1e+1x2e+1x3e+1x4e"
+    assert repr(o3.Irreps("1e + 1e + 0e").simplify()) == "2x1e+1x0e"
+    assert repr(o3.Irreps("1e + 1e + 0e + 1e").simplify()) == "2x1e+1x0e+1x1e"
+    assert repr(o3.Irreps("4x0e + 0x1o + 2x3e").remove_zero_multiplicities()) == "4x0e+2x3e"
+    assert repr(o3.Irreps("1e + 0e + 1e + 0x2e").regroup()) == "1x0e+2x1e"
+    assert repr(o3.Irreps("1e + 2e + 0e").filter(keep=["0e", "1e"])) == "1x1e+1x0e"
+    assert repr(o3.Irreps("1e + 2e + 0e").filter(drop="2e + 2x1e")) == "1x0e"
+    assert repr(o3.Irreps("1e + 2e + 0e").filter(lmax=1)) == "1x1e+1x0e"
+    assert repr(2 * o3.Irreps("0e + 1e")) == "1x0e+1x1e+1x0e+1x1e" and repr(3 * o3.Irrep("1e")) == "3x1e"
+    assert o3.Irreps("5x0e + 10x1o").randn(5, -1, 5, normalization="norm").shape == (5, 35, 5)
+    assert o3.Irreps("3x1o + 2x1o").count("1o") == 5 and "2e" not in o3.Irreps("1o")
+    for bad in ("1x", "-1e", "2x1z"):
+        with pytest.raises(ValueError):
+            o3.Irreps(bad)
+    with pytest.raises(NotImplementedError):
+        o3.Irreps("1o") * o3.Irreps("1o")
+
+
+def test_sort_matches_reference_golden(golden_tp):
+    for s, ref in golden_tp[0]["sort"].items():
+        r = o3.Irreps(s).sort()
+        assert str(r.irreps) == ref["irreps"] and list(r.p) == ref["p"] and list(r.inv) == ref["inv"]
+
+
+def test_constructor_tables_match_reference_golden(golden_tp):
+    meta = golden_tp[0]
+    n = 0
+    for name, m in meta.items():
+        if "instructions" not in m or any(t[3] not in ("uvu", "uvw") for t in m["instructions"]):
+            continue
+        tp = ks.golden_tp(name, meta)
+        assert tp.weight_numel == m["weight_numel"] and tp.shared_weights == m["shared_weights"]
+        assert tp.internal_weights == m["internal_weights"]
+        for t, ref in zip(tp.instructions, m["instructions"]):
+            assert abs(t.path_weight - ref[5]) <= 1e-15 * max(1.0, abs(ref[5])) and list(t.path_shape) == ref[6]
+        for sl, flag in zip(tp.irreps_out.slices(), m["output_mask_blocks"]):
+            if flag >= 0:
+                assert (tp.output_mask[sl] == flag).all()
+        n += 1
+    assert n >= 15
+
+
+def test_builders_match_reference_golden(golden_tp):
+    meta = golden_tp[0]
+    for name, tp in (("fctp_cfg1", ks.cfg1()), ("fctp_cfg5_structure", ks.cfg5()), ("uvu_merged_cfg3_structure", ks.cfg3(True)),
+                     ("uvu_builder_cfg3_structure", ks.cfg3(False)), ("uvu_builderA_cfg4_structure", ks.cfg4("A")),
+                     ("uvu_builderB_cfg4_structure", ks.cfg4("B"))):  # fmt: skip
+        m = meta[name]
+        assert str(tp.irreps_out) == m["irreps_out"], name
+        assert [[t.i_in1, t.i_in2, t.i_out, t.connection_mode] for t in tp.instructions] == [t[:4] for t in m["instructions"]]
+        assert tp.weight_numel == m["weight_numel"]
+        for t, ref in zip(tp.instructions, m["instructions"]):
+            assert abs(t.path_weight - ref[5]) < 1e-15
+    mid, ins = message_instructions("4x0e+4x1o", "0e+1o", "0e+1o")
+    omid, oins = otp.convolution_instructions("4x0e+4x1o", "0e+1o", lambda l, p: (l, p) in {(0, 1), (1, -1)})
+    assert [tuple(t) for t in ins] == [tuple(t) for t in oins] and str(mid) == "4x0e+4x0e+4x1o+4x1o"
+
+
+def test_module_state_and_api_details():
+    tp = ks.cfg1()
+    assert set(tp.state_dict()) == {"weight", "output_mask"}
+    assert repr(tp).startswith("FullyConnectedTensorProduct(16x0e+16x1o x 1x0e+1x1o+1x2e -> 16x0e+16x1o+16x2e | 1792 paths | 1792 weights")
+    views = list(tp.weight_views())
+    assert [tuple(v.shape) for v in views] == [(16, 1, 16)] * 7
+    assert tp.weight_view_for_instruction(2).shape == (16, 1, 16)
+    assert tp.weight_view_for_instruction(2).data_ptr() == views[2].data_ptr()
+    tp2 = copy.deepcopy(tp)
+    assert torch.equal(tp2.weight, tp.weight) and tp2.instructions == tp.instructions
+    ext = ks.cfg3(True)
+    assert ext.weight.numel() == 0 and not ext.internal_weights and not ext.shared_weights
+    with pytest.raises(RuntimeError):
+        ext._get_weights(None)
+    with pytest.raises(AssertionError):
+        o3.TensorProduct("1o", "1o", "1o", [(0, 0, 0, "uvu", True)])  # parity violates the selection rule
+    with pytest.raises(AssertionError):
+        o3.TensorProduct("1o", "1o", "3e", [(0, 0, 0, "uvu", True)])
+    with pytest.raises(AssertionError):
+        o3.TensorProduct("1o", "1o", "1e", [(0, 0, 0, "uvu", True)], internal_weights=True, shared_weights=False)
+    with pytest.raises(NotImplementedError):
+        o3.TensorProduct("2x1o", "2x1o", "2x1e", [(0, 0, 0, "uuu", True)])
+    set_optimization_defaults(specialized_code=False)
+    assert get_optimization_defaults()["specialized_code"] is False
+    set_optimization_defaults(specialized_code=True)
+    with pytest.raises(ValueError):
+        set_optimization_defaults(nonsense=1)
+
+
+def test_plan_creation_needs_no_gpu_and_reports_family():
+    tp = message_tensor_product("4x0e+4x1o+4x2e", ks.SH2, keep="0e+1o+2e")
+    plan = tp.compile()._plans[torch.float32]
+    assert plan.family == "uvu" and plan.key.startswith("uvu_")
+    assert ks.cfg1().compile()._plans[torch.float32].family == "uvw_small"
+    L = _lib.lib()
+    bad = _lib.TpDesc(1, 1, 1, 1, (_lib.Irrep * 1)(_lib.Irrep(2, 1, -1)), (_lib.Irrep * 1)(_lib.Irrep(1, 1, -1)),
+                      (_lib.Irrep * 1)(_lib.Irrep(2, 1, -1)), (_lib.Instruction * 1)(_lib.Instruction(0, 0, 0, 1, 1, 1.0)), 0, 0)  # fmt: skip
+    h = _lib.c_void_p()
+    assert L.e3x_tp_plan_create(ctypes.byref(bad), ctypes.byref(h)) == -1  # 1o x 1o -> 1o violates parity
+    assert b"selection" in L.e3x_last_error()
+    assert L.e3x_csr_workspace_bytes(1000, 10) > 3 * 4000
