@@ -1,0 +1,245 @@
+"""Benchmark of the equivariant message-passing hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[2], "NequIP-style interaction"): N = 50 000 nodes uniform in a
+cube, radius graph with a 5 A cutoff (cube side 86.8 A -> ~1.87 M directed edges, degree ~37), node
+features 32x0e+32x1o+32x2e fp32, edge attributes = SH(lmax 2) of the edge vectors, uvu tensor product
+(11 paths) with per-edge weights from a 2-layer radial MLP, scatter-summed onto the destination nodes.
+One step = one launch of the fused gather -> tensor product -> scatter kernel over the whole graph, all
+inputs resident in HBM.  The other configurations are reported in "other".
+
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+FP32_MFMA_PEAK_TFLOPS = 157.3
+BF16_MFMA_PEAK_TFLOPS = 2500.0
+
+
+def event_time_ms(fn, steps, warmup):
+    """Average duration of fn() over `steps` launches, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    beg.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return beg.elapsed_time(end) / steps
+
+
+def bench_copy(args, dev):
+    """Plain 16-byte-per-lane copy of 1 GiB: the measured streaming ceiling and the calibration
+    kernel for the FETCH_SIZE / WRITE_SIZE counters (known traffic: 1 GiB read + 1 GiB written)."""
+    from e3nn_amd import _lib
+
+    n = 1 << 30
+    a = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
+    b = torch.empty_like(a)
+    L = _lib.lib()
+
+    def step():
+        _lib.check(L.e3x_copy_bytes(_lib.ptr(a), _lib.ptr(b), n, _lib.stream_ptr(dev)))
+
+    ms = event_time_ms(step, max(3, args.steps // 5), 2)
+    assert torch.equal(a[:4096], b[:4096])
+    return {"bytes_read": n, "bytes_written": n, "ms": ms, "gbs": 2 * n / (ms * 1e-3) / 1e9}
+
+
+def radius_graph(n, side, cutoff, seed=0):
+    from scipy.spatial import cKDTree
+
+    rng = np.random.default_rng(seed)
+    pos = rng.uniform(0.0, side, size=(n, 3))
+    pairs = cKDTree(pos).query_pairs(cutoff, output_type="ndarray")
+    src = np.concatenate([pairs[:, 0], pairs[:, 1]])
+    dst = np.concatenate([pairs[:, 1], pairs[:, 0]])
+    return pos, src.astype(np.int64), dst.astype(np.int64)
+
+
+def radial_weights(r, cutoff, weight_numel, gen, dev):
+    """8 Bessel functions -> 64 -> weight_numel, SiLU, N(0,1) weights, scaled as the reference's
+    FullyConnectedNet (e3nn/nn/_fc.py:38-48; basis e3nn/math/_bessel.py:30-37).  Untimed input generation."""
+    n = torch.arange(1, 9, dtype=torch.float32, device=dev)
+    x = r[:, None]
+    basis = math.sqrt(2.0 / cutoff) * torch.sin(n * math.pi / cutoff * x) / x
+    w1 = torch.randn(8, 64, generator=gen).to(dev)
+    w2 = torch.randn(64, weight_numel, generator=gen).to(dev)
+    h = torch.nn.functional.silu(basis @ (w1 / math.sqrt(8))) * 1.679177  # second-moment normalisation of SiLU
+    return (h @ (w2 / math.sqrt(64))).contiguous()
+
+
+def bench_nequip(args, dev):
+    from e3nn_amd import o3
+    from e3nn_amd.nn import DstSortedEdges
+    from tests import kernel_sets as ks
+
+    N, side, cutoff = 50_000, 86.8, 5.0
+    pos, src, dst = radius_graph(N, side, cutoff)
+    E = src.shape[0]
+    gen = torch.Generator().manual_seed(0)
+    tp = ks.cfg3(merged=True)
+    node_x = torch.randn(N, tp.irreps_in1.dim, generator=gen).to(dev)
+    pos_t = torch.from_numpy(pos).float().to(dev)
+    src_t, dst_t = torch.from_numpy(src).to(dev), torch.from_numpy(dst).to(dev)
+    vec = pos_t[src_t] - pos_t[dst_t]
+    attr = o3.spherical_harmonics([0, 1, 2], vec, True, "component")
+    w = radial_weights(vec.norm(dim=1), cutoff, tp.weight_numel, gen, dev)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    edges = DstSortedEdges(src_t, dst_t, N)
+    torch.cuda.synchronize()
+    sort_ms = (time.perf_counter() - t0) * 1e3
+
+    out = [None]
+
+    def step():
+        out[0] = tp.forward_gather_scatter(node_x, attr, w, edges=edges)
+
+    ms = event_time_ms(step, args.steps, args.warmup)
+    # algorithmic bytes: per edge weights + SH + two int64 indices, node table read once, output written once
+    bytes_algo = E * (4 * tp.weight_numel + 4 * 9 + 2 * 8) + N * 4 * (tp.irreps_in1.dim + tp.irreps_out.dim)
+    gbs = bytes_algo / (ms * 1e-3) / 1e9
+    res = {
+        "edges": E, "nodes": N, "ms": ms, "edges_per_s": E / (ms * 1e-3), "bytes_per_launch": bytes_algo,
+        "achieved_gbs": gbs, "edge_sort_ms_one_off": sort_ms,
+        "edges_per_s_incl_sort": E / ((ms + sort_ms) * 1e-3),
+    }  # fmt: skip
+    ctx = dict(tp=tp, node_x=node_x, attr=attr, w=w, src=src_t, dst=dst_t, N=N, out=out[0])
+    return res, ctx
+
+
+def cpu_baseline_nequip(ctx, n_edges=200_000, reps=3):
+    """The reference's CPU path (torch einsum graph + index + scatter_add_) on a slice of the same workload."""
+    from oracle.torch_cpu import tp_gather_scatter_torch
+    from tests.helpers import oracle_spec
+
+    torch.set_num_threads(os.cpu_count())
+    spec = oracle_spec(ctx["tp"])
+    E = min(n_edges, ctx["src"].shape[0])
+    node_x = ctx["node_x"].cpu()
+    attr, w = ctx["attr"][:E].cpu(), ctx["w"][:E].cpu()
+    src, dst = ctx["src"][:E].cpu(), ctx["dst"][:E].cpu()
+    tp_gather_scatter_torch(spec, node_x, attr, w, src, dst, ctx["N"])
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        tp_gather_scatter_torch(spec, node_x, attr, w, src, dst, ctx["N"])
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[len(times) // 2]
+    return {
+        "value": E / t, "unit": "edges/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"first {E} edges of the same graph, fp32, median of {reps}, torch {torch.__version__} CPU einsum "
+                  f"restatement of the reference graph ({os.cpu_count()} host cpus)",
+    }  # fmt: skip
+
+
+def bench_sh(args, dev):
+    from e3nn_amd import o3
+
+    n = 4_000_000
+    gen = torch.Generator().manual_seed(0)
+    d = torch.randn(n, 3, generator=gen)
+    d = d / d.norm(dim=1, keepdim=True)
+    x = (d * torch.exp(0.5 * torch.randn(n, 1, generator=gen))).to(dev)
+    sh = o3.SphericalHarmonics([0, 1, 2, 3], True, "component")
+    ms = event_time_ms(lambda: sh(x), args.steps, args.warmup)
+    b = n * 76
+    return {"vectors": n, "ms": ms, "mvec_per_s": n / (ms * 1e-3) / 1e6, "achieved_gbs": b / (ms * 1e-3) / 1e9,
+            "roofline_frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "bytes_per_launch": b}  # fmt: skip
+
+
+def bench_mace(args, dev, dtype=torch.float32):
+    from e3nn_amd.nn import DstSortedEdges
+    from tests import kernel_sets as ks
+
+    N, E = 20_000, 500_000
+    gen = torch.Generator().manual_seed(0)
+    tp = ks.cfg4("A")
+    src = torch.randint(0, N, (E,), generator=gen, dtype=torch.int32).to(dev)
+    dst = torch.randint(0, N, (E,), generator=gen, dtype=torch.int32).to(dev)
+    node_x = torch.randn(N, tp.irreps_in1.dim, generator=gen).to(dev).to(dtype)
+    from e3nn_amd import o3
+
+    v = torch.randn(E, 3, generator=gen).to(dev)
+    attr = o3.spherical_harmonics([0, 1, 2, 3], v, True, "component").to(dtype)
+    w = torch.randn(E, tp.weight_numel, generator=gen).to(dev).to(dtype)
+    edges = DstSortedEdges(src, dst, N)
+    ms = event_time_ms(lambda: tp.forward_gather_scatter(node_x, attr, w, edges=edges), max(3, args.steps // 4), 2)
+    fb = 2 if dtype == torch.bfloat16 else 4
+    b = E * (fb * tp.weight_numel + fb * 16 + 2 * 4) + N * fb * (tp.irreps_in1.dim + tp.irreps_out.dim)
+    return {"edges": E, "nodes": N, "ms": ms, "edges_per_s": E / (ms * 1e-3), "achieved_gbs": b / (ms * 1e-3) / 1e9,
+            "roofline_frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "bytes_per_launch": b}  # fmt: skip
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16 (default all)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported (no collectives, no sharding)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    neq, ctx = bench_nequip(args, dev)
+    other = {"nequip_uvu": neq}
+    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_bf16"}
+    if "copy" in want:
+        other["copy_1GiB"] = bench_copy(args, dev)
+    if "sh" in want:
+        other["sh_lmax3_4M"] = bench_sh(args, dev)
+    if "mace" in want:
+        other["mace_uvu_fp32"] = bench_mace(args, dev)
+    if "mace_bf16" in want:
+        other["mace_uvu_bf16_storage"] = bench_mace(args, dev, torch.bfloat16)
+    line = {
+        "metric": "per-edge uvu TP edges/sec (L=2, fused gather + tensor product + scatter)",
+        "value": neq["edges_per_s"],
+        "unit": "edges/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": neq["ms"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "NequIP-style uvu interaction: N=50000 nodes, cube side 86.8 A, 5 A cutoff radius graph "
+                        f"(E={neq['edges']}), 32x0e+32x1o+32x2e x SH(lmax 2), 11 paths, 352 weights/edge, int64 indices, "
+                        "fused scatter-sum; edge sort by destination built once per graph (edge_sort_ms_one_off)",
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": neq["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": neq["achieved_gbs"] / HBM_PEAK_GBS, "traffic": None, "kernel": "e3x_uvu_fused",
+        },
+        "other": other,
+    }  # fmt: skip
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_nequip(ctx)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

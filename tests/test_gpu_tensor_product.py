@@ -70,21 +70,27 @@ def test_batch_broadcasting_weight_lists_and_errors():
         spec, x1.expand(3, 4, -1).reshape(12, -1).numpy(), x2.expand(3, 4, -1).reshape(12, -1).numpy(), w.reshape(12, -1).numpy()
     ).reshape(3, 4, -1)
     assert_close(out, ref)
-    # weights given as a list of per-instruction tensors
-    wl = [v.contiguous() for v in tp.weight_views(w.to(DEV))]
-    assert torch.equal(tp(x1.to(DEV), x2.to(DEV), wl), out)
+    # weights given as a list of per-instruction tensors (the reference flattens their batch dims to one)
+    x1f, x2f = x1.expand(3, 4, -1).reshape(12, -1).to(DEV), x2.expand(3, 4, -1).reshape(12, -1).to(DEV)
+    wl = [v.contiguous() for v in tp.weight_views(w.reshape(12, -1).to(DEV))]
+    assert torch.equal(tp(x1f, x2f, wl), out.reshape(12, -1))
     with pytest.raises(RuntimeError):
         tp(x1.to(DEV), x2.to(DEV))  # external weights are mandatory
-    with pytest.raises(RuntimeError):
+    # shape checks are torch._assert like the reference's: AssertionError in eager mode
+    with pytest.raises((RuntimeError, AssertionError)):
         tp(x1.to(DEV), x2.to(DEV), w.to(DEV)[..., :-1])
-    with pytest.raises(RuntimeError):
+    with pytest.raises((RuntimeError, AssertionError)):
         tp(x1.to(DEV), x2.to(DEV), w.to(DEV)[0, 0])  # no batch dimension on per-sample weights
-    with pytest.raises(RuntimeError):
+    with pytest.raises((RuntimeError, AssertionError)):
         tp(x1.to(DEV)[..., :-1], x2.to(DEV), w.to(DEV))
+    # "weird" batch dimensions broadcast like the reference (tests/o3/tensor_product_test.py:346-358)
+    a, b, c = seeded(2, 1, 4, tp.irreps_in1.dim, seed=5).to(DEV), seeded(2, 3, 1, tp.irreps_in2.dim, seed=6).to(DEV), seeded(3, 4, tp.weight_numel, seed=7).to(DEV)
+    full = tp(a.expand(2, 3, 4, -1).reshape(24, -1), b.expand(2, 3, 4, -1).reshape(24, -1), c[None].expand(2, 3, 4, -1).reshape(24, -1))
+    assert torch.equal(tp(a, b, c).reshape(24, -1), full)
     with pytest.raises(RuntimeError):
         tp(x1, x2, w)  # CPU tensors: no silent fallback
     shared = ks.golden_tp("fctp_cfg1").to(DEV)
-    with pytest.raises(RuntimeError):
+    with pytest.raises((RuntimeError, AssertionError)):
         shared(seeded(2, 64).to(DEV), seeded(2, 9).to(DEV), seeded(2, shared.weight_numel).to(DEV))
     # empty batch
     assert shared(torch.zeros(0, 64, device=DEV), torch.zeros(0, 9, device=DEV)).shape == (0, 144)
