@@ -186,13 +186,34 @@ def bench_mace(args, dev, dtype=torch.float32):
             "roofline_frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "bytes_per_launch": b}  # fmt: skip
 
 
+def bench_uvw(args, dev, dtype=torch.float32):
+    """Dense uvw: FCTP(128x0e+128x1o+128x2e x same -> same), 65536 rows, shared weights N(0, 1/fan_in)."""
+    from tests import kernel_sets as ks
+
+    tp = ks.cfg5().to(dev)
+    Z = 65536
+    gen = torch.Generator().manual_seed(0)
+    with torch.no_grad():
+        tp.weight.copy_(torch.randn(tp.weight_numel, generator=gen) / 128.0)
+    tp = tp.to(dtype)
+    x1 = torch.randn(Z, 1152, generator=gen).to(dev).to(dtype)
+    x2 = torch.randn(Z, 1152, generator=gen).to(dev).to(dtype)
+    ms = event_time_ms(lambda: tp(x1, x2), 3, 1)
+    f_min = 2 * Z * 128**3 * 21  # cheapest contraction order per path: sum of min(2l1+1, 2l2+1, 2l3+1) = 21
+    f_gemm = 2 * Z * 128**3 * 35  # outer-product order: sum of (2l3+1) = 35
+    peak = BF16_MFMA_PEAK_TFLOPS if dtype == torch.bfloat16 else FP32_MFMA_PEAK_TFLOPS
+    return {"rows": Z, "ms": ms, "tflops_fmin": f_min / (ms * 1e-3) / 1e12, "tflops_fgemm_equiv": f_gemm / (ms * 1e-3) / 1e12,
+            "roofline": {"bound": "mfma", "achieved": f_min / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
+                         "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16 (default all)")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16,uvw,uvw_bf16 (default: all but uvw_bf16)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported (no collectives, no sharding)")
@@ -203,7 +224,7 @@ def main():
 
     neq, ctx = bench_nequip(args, dev)
     other = {"nequip_uvu": neq}
-    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_bf16"}
+    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_bf16", "uvw"}
     if "copy" in want:
         other["copy_1GiB"] = bench_copy(args, dev)
     if "sh" in want:
@@ -212,6 +233,10 @@ def main():
         other["mace_uvu_fp32"] = bench_mace(args, dev)
     if "mace_bf16" in want:
         other["mace_uvu_bf16_storage"] = bench_mace(args, dev, torch.bfloat16)
+    if "uvw" in want:
+        other["uvw_dense_fp32"] = bench_uvw(args, dev)
+    if "uvw_bf16" in want:
+        other["uvw_dense_bf16_storage"] = bench_uvw(args, dev, torch.bfloat16)
     line = {
         "metric": "per-edge uvu TP edges/sec (L=2, fused gather + tensor product + scatter)",
         "value": neq["edges_per_s"],

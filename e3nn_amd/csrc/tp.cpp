@@ -4,6 +4,7 @@
 
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <memory>
 #include <mutex>
 #include <sstream>
@@ -35,8 +36,8 @@ struct e3x_plan {
   bool zero_fill = false;  // some output irrep is reached by no instruction
   // launch geometry of the lane<->multiplicity kernels
   int lanes = 64, chunks = 1;
-  // uvw_mfma geometry
-  int rows_per_block = 0;
+  // uvw_mfma geometry: grid.y
+  int n_targets = 0;
   std::mutex mu;
   hipModule_t module[kMaxDevices] = {nullptr};
   hipFunction_t fn_plain[kMaxDevices] = {nullptr};
@@ -214,6 +215,75 @@ int build_uvw_small_source(e3x_plan& P, std::string* src) {
   return E3X_OK;
 }
 
+// ---- uvw on the matrix cores ----------------------------------------------------------
+bool uvw_mfma_eligible(const e3x_plan& P) {
+  if (!P.shared_weights || P.paths.empty()) return false;
+  for (const auto& p : P.paths) {
+    const int U = P.in1[p.in1].mul, V = P.in2[p.in2].mul, W = P.out[p.out].mul;
+    if (U % 32 || V % 32 || W % 64 || U > 256 || V > 256 || P.out[p.out].l > 3) return false;
+  }
+  return true;
+}
+
+int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
+  int wt = 128, kmax = 32;
+  for (const auto& p : P.paths) {
+    if (P.out[p.out].mul % 128) wt = 64;
+    kmax = std::max(kmax, std::max(P.in1[p.in1].mul, P.in2[p.in2].mul));
+  }
+  std::ostringstream s, nzs, ps, ts;
+  emit_header(s, P);
+  s << "constexpr int WT = " << wt << ", KMAX = " << kmax << ";\n";
+  int n_nz = 0, n_path = 0, n_target = 0;
+  for (size_t c = 0; c < P.out.size(); ++c) {
+    std::ostringstream mine;
+    const int beg = n_path;
+    for (const auto& p : P.paths) {
+      if (p.out != (int)c) continue;
+      const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2];
+      const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1, d3 = 2 * P.out[c].l + 1;
+      const bool k_is_x2 = d2 < d1;  // fewer GEMM passes: K operand = the input with the smaller irrep
+      const auto& C = e3x::wigner_3j(a.l, b.l, P.out[c].l);
+      const int nz_beg = n_nz;
+      for (int i = 0; i < d1; ++i)
+        for (int j = 0; j < d2; ++j)
+          for (int k = 0; k < d3; ++k) {
+            const double cv = C[(i * d2 + j) * d3 + k] * p.pw;
+            if (cv != 0.0) {
+              nzs << "  {" << (k_is_x2 ? j : i) << ", " << (k_is_x2 ? i : j) << ", " << k << ", " << fstr(cv) << "},\n";
+              ++n_nz;
+            }
+          }
+      const long long W = P.out[c].mul;
+      // W_p[u, v, w] at woff + (u * V + v) * W + w
+      const long long stride_u = (long long)b.mul * W, stride_v = W;
+      mine << "  {" << (k_is_x2 ? "true" : "false") << ", " << (k_is_x2 ? P.off2[p.in2] : P.off1[p.in1]) << ", "
+           << (k_is_x2 ? d2 : d1) << ", " << (k_is_x2 ? b.mul : a.mul) << ", "
+           << (k_is_x2 ? P.off1[p.in1] : P.off2[p.in2]) << ", " << (k_is_x2 ? d1 : d2) << ", "
+           << (k_is_x2 ? a.mul : b.mul) << ", " << p.woff << ", " << (k_is_x2 ? stride_v : stride_u) << ", "
+           << (k_is_x2 ? stride_u : stride_v) << ", " << nz_beg << ", " << n_nz << "},\n";
+      ++n_path;
+    }
+    if (n_path == beg) continue;
+    ps << mine.str();
+    for (int w0 = 0; w0 < P.out[c].mul; w0 += wt) {
+      ts << "  {" << P.offo[c] << ", " << 2 * P.out[c].l + 1 << ", " << w0 << ", " << beg << ", " << n_path << "},\n";
+      ++n_target;
+    }
+  }
+  s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
+    << nzs.str() << "};\n";
+  s << "struct MPath { bool k_is_x2; int koff, dK, K, roff, dR, O; long long wbase, wk_stride, wo_stride; int nz_beg, "
+       "nz_end; };\n";
+  s << "constexpr int N_MPATH = " << n_path << ";\nconstexpr MPath mpaths[N_MPATH] = {\n" << ps.str() << "};\n";
+  s << "struct Target { int out_off, d3, w0, path_beg, path_end; };\n";
+  s << "constexpr int N_TARGET = " << n_target << ";\nconstexpr Target targets[N_TARGET] = {\n" << ts.str() << "};\n";
+  s << "}  // namespace cfg\n";
+  P.n_targets = n_target;
+  *src = s.str() + e3x::kTplCommon + e3x::kTplUvwMfma;
+  return E3X_OK;
+}
+
 int load_functions(e3x_plan* P, int dev) {
   std::lock_guard<std::mutex> lock(P->mu);
   if (P->module[dev]) return E3X_OK;
@@ -296,7 +366,11 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
     return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: mixing uvu and uvw instructions in one plan is not implemented");
 
   std::string src;
-  if (n_uvw) {
+  const char* force_small = std::getenv("E3X_UVW_FORCE_VALU");
+  if (n_uvw && uvw_mfma_eligible(*P) && !(force_small && force_small[0] == '1')) {
+    P->family = "uvw_mfma";
+    rc = build_uvw_mfma_source(*P, &src);
+  } else if (n_uvw) {
     P->family = "uvw_small";
     rc = build_uvw_small_source(*P, &src);
   } else {
@@ -351,11 +425,19 @@ extern "C" int e3x_tp_forward(e3x_plan* P, const void* x1, const void* x2, const
   if ((rc = load_functions(P, dev))) return rc;
   long long n_rows = Z;
   void* args[] = {(void*)&x1, (void*)&x2, (void*)&w, (void*)&out, (void*)&n_rows};
-  const int groups = 64 / P->lanes;
-  const long long items = (Z + groups - 1) / groups * P->chunks;
-  const long long blocks = (items + 3) / 4;
+  long long blocks;
+  unsigned grid_y = 1;
+  if (P->family == "uvw_mfma") {
+    blocks = (Z + 63) / 64;
+    grid_y = (unsigned)P->n_targets;
+  } else {
+    const int groups = 64 / P->lanes;
+    const long long items = (Z + groups - 1) / groups * P->chunks;
+    blocks = (items + 3) / 4;
+  }
   if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_forward: batch too large for one launch");
-  hipError_t err = hipModuleLaunchKernel(P->fn_plain[dev], (unsigned)blocks, 1, 1, 256, 1, 1, 0, st, args, nullptr);
+  hipError_t err =
+      hipModuleLaunchKernel(P->fn_plain[dev], (unsigned)blocks, grid_y, 1, 256, 1, 1, 0, st, args, nullptr);
   if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_tp_forward: launch failed: ") + hipGetErrorString(err));
   return E3X_OK;
 }

@@ -186,7 +186,7 @@ def tp_forward(spec, x1, x2, w=None, dtype=np.float64):
                 "uvu<v": f"{z}w,ijk,zwij->zwk",
                 "u<vw": f"{z}qw,ijk,zqij->zwk",
             }[mode]
-            r = np.einsum(expr, wt, C, xx)
+            r = np.einsum(expr, wt, C, xx, optimize=True)
         else:
             expr = {
                 "uvu": "ijk,zuvij->zuk",

@@ -68,6 +68,11 @@ def cfg5():
     return o3.FullyConnectedTensorProduct(f, f, f)
 
 
+def mfma_small():
+    # smallest shapes the matrix-core uvw kernel takes: multiplicities 32 / 64, three output irreps
+    return o3.FullyConnectedTensorProduct("64x0e+32x1o", "32x0e+32x1o+32x2e", "64x0e+64x1o+64x1e+64x2e")
+
+
 def scalar_exact():
     # 1x1 Clebsch-Gordan, path weight 1: products and sums of small integers are exact in fp32
     return message_tensor_product("32x0e", "0e", irreps_out="32x0e")
@@ -88,6 +93,8 @@ def all_tensor_products():
         ("cfg3_builder", cfg3(False), (torch.float32,)),
         ("cfg4_A", cfg4("A"), (torch.float32, torch.bfloat16)),
         ("cfg4_B", cfg4("B"), (torch.float32,)),
+        ("cfg5", cfg5(), (torch.float32, torch.bfloat16)),
+        ("mfma_small", mfma_small(), (torch.float32,)),
         ("scalar_exact", scalar_exact(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),
     ]

@@ -141,3 +141,67 @@ def test_bf16_storage_variant():
     # oracle on the bf16-rounded inputs; the output is rounded to bf16 once
     ref = otp.tp_forward(oracle_spec(tp), xb.float().cpu().numpy(), yb.float().cpu().numpy(), wb.float().cpu().numpy())
     assert_close(out, ref, atol=1e-2, rtol=1e-2, what="bf16 storage")
+
+
+def _fan_in_weights(tp, seed=0):
+    # N(0, 1/fan_in) per instruction, fan_in = U*V  (benchmark definition of the dense uvw configuration)
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(tp.weight_numel, generator=g)
+    off = 0
+    for t in tp.instructions:
+        n = t.path_shape[0] * t.path_shape[1] * t.path_shape[2]
+        w[off : off + n] /= (t.path_shape[0] * t.path_shape[1]) ** 0.5
+        off += n
+    return w
+
+
+@pytest.mark.parametrize("maker,Z", [(ks.mfma_small, 150), (ks.cfg5, 70)])
+def test_uvw_matrix_core_kernel_against_oracle(maker, Z):
+    tp = maker().to(DEV)
+    assert tp._plan(torch.float32).family == "uvw_mfma"
+    w = _fan_in_weights(tp)
+    with torch.no_grad():
+        tp.weight.copy_(w)
+    x1, x2 = seeded(Z, tp.irreps_in1.dim, seed=21), seeded(Z, tp.irreps_in2.dim, seed=22)
+    out = tp(x1.to(DEV), x2.to(DEV))
+    ref = otp.tp_forward(oracle_spec(tp), x1.numpy(), x2.numpy(), w.numpy())
+    assert_close(out, ref, what=str(tp))
+
+
+def test_uvw_full_size_dense_configuration():
+    # FCTP(128x0e+128x1o+128x2e x same -> same), batch 65536, weights N(0, 1/fan_in), inputs N(0, 1)
+    tp = ks.cfg5().to(DEV)
+    w = _fan_in_weights(tp)
+    with torch.no_grad():
+        tp.weight.copy_(w)
+    Z = 65536
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x1 = torch.randn(Z, 1152, device=DEV, generator=g)
+    x2 = torch.randn(Z, 1152, device=DEV, generator=g)
+    out = tp(x1, x2)
+    # rows are independent: the oracle on a few rows from both ends and the middle
+    rows = torch.tensor([0, 1, 63, 64, 32767, 32768, 65471, 65535])
+    ref = otp.tp_forward(oracle_spec(tp), x1[rows].cpu().numpy(), x2[rows].cpu().numpy(), w.numpy())
+    assert_close(out[rows], ref, what="cfg5 rows")
+    # size-independent properties: bilinearity in (x1, x2), output scale
+    out2 = tp(2.0 * x1, -0.5 * x2)
+    assert torch.equal(out2, -out)  # exact: powers of two commute with every rounding
+    # weights N(0, 1/fan_in) on top of the path normalisation 1/sqrt(fan_in * paths): variance 1/fan_in
+    assert abs(out.var().item() * 16384 - 1.0) < 0.1
+    # batch slices give the same rows
+    assert torch.equal(tp(x1[1000:1100], x2[1000:1100]), out[1000:1100])
+
+
+def test_uvw_bf16_storage():
+    tp = ks.cfg5().to(DEV)
+    w = _fan_in_weights(tp)
+    Z = 40
+    x1, x2 = seeded(Z, 1152, seed=31), seeded(Z, 1152, seed=32)
+    tpb = ks.cfg5().to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        tpb.weight.copy_(w.to(torch.bfloat16))
+    xb, yb = x1.to(DEV).to(torch.bfloat16), x2.to(DEV).to(torch.bfloat16)
+    out = tpb(xb, yb)
+    assert out.dtype == torch.bfloat16
+    ref = otp.tp_forward(oracle_spec(tp), xb.float().cpu().numpy(), yb.float().cpu().numpy(), tpb.weight.float().cpu().numpy())
+    assert_close(out, ref, atol=2e-2, rtol=1e-2, what="bf16 uvw")
