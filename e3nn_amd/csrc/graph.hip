@@ -62,9 +62,11 @@ __global__ __launch_bounds__(kBlock) void fill_zero_kernel(int* p, int n) {
   if (i < n) p[i] = 0;
 }
 
+// one 16-byte element per thread and a grid that covers the buffer once
 __global__ __launch_bounds__(kBlock) void copy16_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                                         size_t n16) {
-  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += (size_t)gridDim.x * kBlock) dst[i] = src[i];
+  const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n16) dst[i] = src[i];
 }
 
 __global__ __launch_bounds__(kBlock) void fill_zero_bytes_kernel(unsigned char* p, size_t n) {
@@ -190,7 +192,9 @@ extern "C" int e3x_copy_bytes(const void* src, void* dst, size_t n_bytes, void* 
   if (n_bytes % 16 || ((uintptr_t)src % 16) || ((uintptr_t)dst % 16))
     return e3x::fail(E3X_ERR_INVALID, "e3x_copy_bytes: size and pointers must be multiples of 16");
   if (n_bytes == 0) return E3X_OK;
-  hipLaunchKernelGGL(copy16_kernel, dim3(grid_for((long long)(n_bytes / 16), kBlock * 4)), dim3(kBlock), 0,
-                     (hipStream_t)stream, (const uint4*)src, (uint4*)dst, n_bytes / 16);
+  const size_t blocks = (n_bytes / 16 + kBlock - 1) / kBlock;
+  if (blocks > 0x7fffffffULL) return e3x::fail(E3X_ERR_INVALID, "e3x_copy_bytes: buffer too large for one launch");
+  hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, (hipStream_t)stream, (const uint4*)src,
+                     (uint4*)dst, n_bytes / 16);
   return hipGetLastError() == hipSuccess ? E3X_OK : e3x::fail(E3X_ERR_HIP, "e3x_copy_bytes: launch failed");
 }

@@ -253,7 +253,9 @@ template <int LMAX>
 void launch_tile(bool normalize, const float* xyz, float* out, long long n, Scale4 sc, hipStream_t st) {
   const long long tiles = (n + kWave - 1) / kWave;
   long long blocks = (tiles + kWavesPerBlock - 1) / kWavesPerBlock;
-  if (blocks > 256 * 32) blocks = 256 * 32;  // grid-stride beyond 32 blocks per CU
+  // one tile per wavefront: on this chip a grid that covers the data once streams faster than a
+  // capped grid with a grid-stride loop (the loop in the kernel only runs for n > 2^31 * 256 vectors)
+  if (blocks > 0x7fffffffLL) blocks = 0x7fffffffLL;
   if (normalize)
     hipLaunchKernelGGL((sh_tile_kernel<LMAX, true>), dim3((unsigned)blocks), dim3(kWave * kWavesPerBlock), 0, st, xyz,
                        out, n, sc);

@@ -26,22 +26,28 @@ constexpr int kMaxDevices = 64;
 
 }  // namespace
 
+// One compiled code object.  A plan is usually one kernel; large uvu instruction sets are split
+// into several kernels over disjoint output irreps so that each keeps its accumulators in registers.
+struct SubKernel {
+  std::string key, hsaco;
+  std::vector<int> path_ids;  // indices into e3x_plan::paths
+  int lanes = 64, chunks = 1, upl = 1, waves_per_block = 4;
+  hipModule_t module[kMaxDevices] = {nullptr};
+  hipFunction_t fn_plain[kMaxDevices] = {nullptr};
+  hipFunction_t fn_fused[kMaxDevices] = {nullptr};
+};
+
 struct e3x_plan {
   std::vector<e3x_irrep> in1, in2, out;
   std::vector<int> off1, off2, offo;
   std::vector<PathInfo> paths;
   int shared_weights = 1, dtype = E3X_F32;
   int64_t in1_dim = 0, in2_dim = 0, out_dim = 0, weight_numel = 0;
-  std::string family, key, hsaco;
+  std::string family, key;
   bool zero_fill = false;  // some output irrep is reached by no instruction
-  // launch geometry of the lane<->multiplicity kernels
-  int lanes = 64, chunks = 1;
-  // uvw_mfma geometry: grid.y
-  int n_targets = 0;
+  int n_targets = 0;       // uvw_mfma: grid.y
   std::mutex mu;
-  hipModule_t module[kMaxDevices] = {nullptr};
-  hipFunction_t fn_plain[kMaxDevices] = {nullptr};
-  hipFunction_t fn_fused[kMaxDevices] = {nullptr};
+  std::vector<std::unique_ptr<SubKernel>> subs;
 };
 
 namespace {
@@ -49,6 +55,11 @@ namespace {
 using e3x::fail;
 
 int dim_of(const e3x_irrep& r) { return r.mul * (2 * r.l + 1); }
+
+int env_int(const char* name, int fallback) {
+  const char* v = std::getenv(name);
+  return (v && v[0]) ? std::atoi(v) : fallback;
+}
 
 std::string fstr(double v) {
   char buf[64];
@@ -63,13 +74,13 @@ int pow2_at_least(int v, int lo) {
 }
 
 // ---- common part of the generated tables ------------------------------------------
-void emit_header(std::ostringstream& s, const e3x_plan& P) {
+void emit_header(std::ostringstream& s, const e3x_plan& P, int lanes = 64, int chunks = 1) {
   s << "// generated: tables of one instruction set\n#include <stdint.h>\nnamespace cfg {\n";
   s << "typedef " << (P.dtype == E3X_BF16 ? "unsigned short" : "float") << " store_t;\n";
   s << "constexpr bool SHARED_W = " << (P.shared_weights ? "true" : "false") << ";\n";
   s << "constexpr int IN1_DIM = " << P.in1_dim << ", IN2_DIM = " << P.in2_dim << ", OUT_DIM = " << P.out_dim
     << ", W_NUMEL = " << P.weight_numel << ";\n";
-  s << "constexpr int LANES = " << P.lanes << ", CHUNKS = " << P.chunks << ";\n";
+  s << "constexpr int LANES = " << lanes << ", CHUNKS = " << chunks << ";\n";
 }
 
 struct NzList {
@@ -78,9 +89,10 @@ struct NzList {
 };
 
 // non-zeros of pw * wigner_3j per path, as "{i, j, k, c}" rows
-NzList emit_nz(const e3x_plan& P) {
+NzList emit_nz(const e3x_plan& P, const std::vector<int>& ids) {
   NzList L;
-  for (const auto& p : P.paths) {
+  for (int id : ids) {
+    const auto& p = P.paths[id];
     const int l1 = P.in1[p.in1].l, l2 = P.in2[p.in2].l, l3 = P.out[p.out].l;
     const auto& C = e3x::wigner_3j(l1, l2, l3);
     const int d2 = 2 * l2 + 1, d3 = 2 * l3 + 1;
@@ -110,23 +122,77 @@ void emit_nz_table(std::ostringstream& s, const NzList& L) {
 }
 
 // ---- uvu ---------------------------------------------------------------------------
-int build_uvu_source(e3x_plan& P, std::string* src) {
+
+// Splits the paths into kernels over disjoint output irreps when one kernel would need too many
+// accumulator registers: paths sharing an output stay together, groups are formed per input-1 irrep
+// (so each kernel gathers only its own slice of the source row).
+std::vector<std::vector<int>> split_uvu_paths(const e3x_plan& P) {
+  std::vector<int> all(P.paths.size());
+  for (size_t i = 0; i < all.size(); ++i) all[i] = (int)i;
+  int acc = 0;
+  std::vector<char> usedo(P.out.size(), 0);
+  for (const auto& p : P.paths)
+    if (!usedo[p.out]) { usedo[p.out] = 1; acc += 2 * P.out[p.out].l + 1; }
+  const int want = env_int("E3X_UVU_SPLIT", acc > 128 ? 1 : 0);
+  if (!want || P.paths.empty()) return {all};
+  // an output irrep fed from several input-1 irreps ties those inputs together
+  std::vector<int> group_of_in1(P.in1.size());
+  for (size_t a = 0; a < group_of_in1.size(); ++a) group_of_in1[a] = (int)a;
+  auto find = [&](int a) { while (group_of_in1[a] != a) a = group_of_in1[a]; return a; };
+  std::vector<int> first_in1(P.out.size(), -1);
+  for (const auto& p : P.paths) {
+    if (first_in1[p.out] < 0) first_in1[p.out] = p.in1;
+    else group_of_in1[find(p.in1)] = find(first_in1[p.out]);
+  }
+  std::vector<std::vector<int>> parts;
+  std::vector<int> part_of_group(P.in1.size(), -1);
+  for (size_t i = 0; i < P.paths.size(); ++i) {
+    const int gsel = find(P.paths[i].in1);
+    if (part_of_group[gsel] < 0) { part_of_group[gsel] = (int)parts.size(); parts.emplace_back(); }
+    parts[part_of_group[gsel]].push_back((int)i);
+  }
+  return parts;
+}
+
+int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src) {
   int max_mul = 1;
   std::vector<char> used1(P.in1.size(), 0), usedo(P.out.size(), 0);
   long long unrolled = 0;
-  for (const auto& p : P.paths) {
+  for (int id : K.path_ids) {
+    const auto& p = P.paths[id];
     if (P.in1[p.in1].mul != P.out[p.out].mul)
       return fail(E3X_ERR_INVALID, "uvu instruction needs irreps_in1[i_in1].mul == irreps_out[i_out].mul");
     used1[p.in1] = 1;
     usedo[p.out] = 1;
     max_mul = std::max(max_mul, P.in1[p.in1].mul);
   }
-  P.lanes = max_mul > 32 ? 64 : pow2_at_least(max_mul, 16);
-  P.chunks = (max_mul + P.lanes - 1) / P.lanes;
   if (P.in2_dim > 64) return fail(E3X_ERR_INVALID, "uvu kernel: irreps_in2.dim > 64 is not supported");
+  int x1regs = 0, accregs = 0, wregs = 0;
+  for (size_t a = 0; a < P.in1.size(); ++a) if (used1[a]) x1regs += 2 * P.in1[a].l + 1;
+  for (size_t c = 0; c < P.out.size(); ++c) if (usedo[c]) accregs += 2 * P.out[c].l + 1;
+  for (int id : K.path_ids) if (P.paths[id].has_w) wregs += P.in2[P.paths[id].in2].mul;
+  if (x1regs > 96) return fail(E3X_ERR_INVALID, "uvu kernel: more than 96 input components per multiplicity index");
+  if (accregs > 256) return fail(E3X_ERR_INVALID, "uvu kernel: more than 256 output components per multiplicity index");
+  // multiplicity indices per lane: 4 makes every per-lane access a 16-byte run; needs mul % 4 == 0
+  // and a register budget of about 200 for one set of edge registers plus the accumulators
+  int upl = 4;
+  auto fits = [&](int u) {
+    for (size_t a = 0; a < P.in1.size(); ++a) if (used1[a] && P.in1[a].mul % u) return false;
+    return u * (accregs + x1regs + wregs) + (int)P.in2_dim <= 200;
+  };
+  while (upl > 1 && !fits(upl)) upl /= 2;
+  upl = env_int("E3X_UVU_UPL", upl);
+  if (upl != 1 && upl != 2 && upl != 4) return fail(E3X_ERR_INVALID, "E3X_UVU_UPL must be 1, 2 or 4");
+  for (size_t a = 0; a < P.in1.size(); ++a)
+    if (used1[a] && P.in1[a].mul % upl) return fail(E3X_ERR_INVALID, "uvu kernel: multiplicity not divisible by UPL");
+  const int lane_units = (max_mul + upl - 1) / upl;
+  K.upl = upl;
+  K.lanes = lane_units > 32 ? 64 : pow2_at_least(lane_units, 8);
+  K.chunks = (lane_units + K.lanes - 1) / K.lanes;
 
   std::ostringstream s;
-  emit_header(s, P);
+  emit_header(s, P, K.lanes, K.chunks);
+  s << "constexpr int UPL = " << upl << ";\n";
   int reg = 0;
   s << "struct In1 { int off, d, mul, reg; bool used; };\n";
   s << "constexpr int N_IN1 = " << P.in1.size() << ";\nconstexpr In1 in1[N_IN1] = {\n";
@@ -137,7 +203,6 @@ int build_uvu_source(e3x_plan& P, std::string* src) {
     if (used1[a]) reg += d;
   }
   s << "};\nconstexpr int X1_REGS = " << reg << ";\n";
-  if (reg > 96) return fail(E3X_ERR_INVALID, "uvu kernel: more than 96 input components per multiplicity index");
   reg = 0;
   s << "struct Out { int off, d, mul, reg; bool used; };\n";
   s << "constexpr int N_OUT = " << P.out.size() << ";\nconstexpr Out outs[N_OUT] = {\n";
@@ -148,13 +213,12 @@ int build_uvu_source(e3x_plan& P, std::string* src) {
     if (usedo[c]) reg += d;
   }
   s << "};\nconstexpr int ACC_REGS = " << reg << ";\n";
-  if (reg > 256) return fail(E3X_ERR_INVALID, "uvu kernel: more than 256 output components per multiplicity index");
-  NzList L = emit_nz(P);
+  NzList L = emit_nz(P, K.path_ids);
   int wreg = 0;
   s << "struct Path { int in1, x2off, d2, V, out, woff, wreg; bool has_w; int nz_beg, nz_end; };\n";
-  s << "constexpr int N_PATH = " << P.paths.size() << ";\nconstexpr Path paths[N_PATH > 0 ? N_PATH : 1] = {\n";
-  for (size_t i = 0; i < P.paths.size(); ++i) {
-    const auto& p = P.paths[i];
+  s << "constexpr int N_PATH = " << K.path_ids.size() << ";\nconstexpr Path paths[N_PATH > 0 ? N_PATH : 1] = {\n";
+  for (size_t i = 0; i < K.path_ids.size(); ++i) {
+    const auto& p = P.paths[K.path_ids[i]];
     const int V = P.in2[p.in2].mul;
     s << "  {" << p.in1 << ", " << P.off2[p.in2] << ", " << 2 * P.in2[p.in2].l + 1 << ", " << V << ", " << p.out << ", "
       << p.woff << ", " << wreg << ", " << (p.has_w ? "true" : "false") << ", " << L.beg[i] << ", " << L.end[i]
@@ -162,18 +226,26 @@ int build_uvu_source(e3x_plan& P, std::string* src) {
     if (p.has_w) wreg += V;
     unrolled += (long long)V * (L.end[i] - L.beg[i]);
   }
-  if (P.paths.empty()) s << "  {0, 0, 1, 0, 0, 0, 0, false, 0, 0}\n";
+  if (K.path_ids.empty()) s << "  {0, 0, 1, 0, 0, 0, 0, false, 0, 0}\n";
   s << "};\nconstexpr int W_REGS = " << wreg << ";\n";
-  if (wreg > 128 || unrolled > 20000)
+  if (wreg > 128 || unrolled * upl > 40000)
     return fail(E3X_ERR_INVALID, "uvu kernel: instruction set too large to unroll (irreps_in2 multiplicities too high)");
   emit_nz_table(s, L);
+  // two register sets (software prefetch of the next edge) while they fit a high-occupancy budget
+  bool prefetch = upl * (accregs + 2 * (x1regs + wregs)) + 2 * (int)P.in2_dim <= 96;
+  prefetch = env_int("E3X_UVU_PREFETCH", prefetch ? 1 : 0) != 0;
+  s << "constexpr bool PREFETCH = " << (prefetch ? "true" : "false") << ";\n";
+  if (env_int("E3X_EXPERIMENT_NO_MATH", 0)) s << "#define E3X_EXPERIMENT_NO_MATH 1\n";
+  if (env_int("E3X_NO_STREAM_HINT", 0)) s << "#define E3X_NO_STREAM_HINT 1\n";
+  K.waves_per_block = env_int("E3X_UVU_WAVES_PER_BLOCK", 4);
+  s << "#define E3X_WAVES_PER_BLOCK " << K.waves_per_block << "\n";
   s << "}  // namespace cfg\n";
   *src = s.str() + e3x::kTplCommon + e3x::kTplUvu;
   return E3X_OK;
 }
 
 // ---- uvw (lane <-> output multiplicity, VALU) ----------------------------------------
-int build_uvw_small_source(e3x_plan& P, std::string* src) {
+int build_uvw_small_source(e3x_plan& P, SubKernel& K, std::string* src) {
   int max_mul = 1;
   std::vector<char> usedo(P.out.size(), 0);
   for (const auto& p : P.paths) {
@@ -181,12 +253,12 @@ int build_uvw_small_source(e3x_plan& P, std::string* src) {
     usedo[p.out] = 1;
     max_mul = std::max(max_mul, P.out[p.out].mul);
   }
-  P.lanes = max_mul > 32 ? 64 : pow2_at_least(max_mul, 16);
-  P.chunks = (max_mul + P.lanes - 1) / P.lanes;
-  if ((P.in1_dim + P.in2_dim) * 16 * (64 / P.lanes) > 65536)
+  K.lanes = max_mul > 32 ? 64 : pow2_at_least(max_mul, 16);
+  K.chunks = (max_mul + K.lanes - 1) / K.lanes;
+  if ((P.in1_dim + P.in2_dim) * 16 * (64 / K.lanes) > 65536)
     return fail(E3X_ERR_INVALID, "uvw kernel: input rows too long for the LDS staging buffer");
   std::ostringstream s;
-  emit_header(s, P);
+  emit_header(s, P, K.lanes, K.chunks);
   int reg = 0;
   s << "struct Out { int off, d, mul, reg; bool used; };\n";
   s << "constexpr int N_OUT = " << P.out.size() << ";\nconstexpr Out outs[N_OUT] = {\n";
@@ -198,7 +270,7 @@ int build_uvw_small_source(e3x_plan& P, std::string* src) {
   }
   s << "};\nconstexpr int ACC_REGS = " << reg << ";\n";
   if (reg > 256) return fail(E3X_ERR_INVALID, "uvw kernel: more than 256 output components per multiplicity index");
-  NzList L = emit_nz(P);
+  NzList L = emit_nz(P, K.path_ids);
   s << "struct Path { int x1off, d1, U, x2off, d2, V, out, woff; int nz_beg, nz_end; };\n";
   s << "constexpr int N_PATH = " << P.paths.size() << ";\nconstexpr Path paths[N_PATH > 0 ? N_PATH : 1] = {\n";
   for (size_t i = 0; i < P.paths.size(); ++i) {
@@ -226,7 +298,9 @@ bool uvw_mfma_eligible(const e3x_plan& P) {
 }
 
 int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
-  int wt = 128, kmax = 32;
+  // 64 output channels per workgroup: 80 accumulator registers, two workgroups per CU (measured faster
+  // than 128 channels at one workgroup per CU)
+  int wt = env_int("E3X_UVW_WT", 64), kmax = 32;
   for (const auto& p : P.paths) {
     if (P.out[p.out].mul % 128) wt = 64;
     kmax = std::max(kmax, std::max(P.in1[p.in1].mul, P.in2[p.in2].mul));
@@ -234,7 +308,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   std::ostringstream s, nzs, ps, ts;
   emit_header(s, P);
   s << "constexpr int WT = " << wt << ", KMAX = " << kmax << ";\n";
-  int n_nz = 0, n_path = 0, n_target = 0;
+  int n_nz = 0, n_path = 0, n_target = 0, dka = 1;
   for (size_t c = 0; c < P.out.size(); ++c) {
     std::ostringstream mine;
     const int beg = n_path;
@@ -242,7 +316,11 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
       if (p.out != (int)c) continue;
       const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2];
       const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1, d3 = 2 * P.out[c].l + 1;
-      const bool k_is_x2 = d2 < d1;  // fewer GEMM passes: K operand = the input with the smaller irrep
+      // GEMM passes per outer index: 2l+1 of the K operand when accumulators are scaled, 2 l3 + 1 when the
+      // operand is synthesised; take the cheapest
+      const bool synth = env_int("E3X_UVW_SYNTH", 1) && d3 < std::min(d1, d2);
+      const bool k_is_x2 = !synth && d2 < d1;
+      if (synth) dka = std::max(dka, d1);
       const auto& C = e3x::wigner_3j(a.l, b.l, P.out[c].l);
       const int nz_beg = n_nz;
       for (int i = 0; i < d1; ++i)
@@ -257,7 +335,8 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
       const long long W = P.out[c].mul;
       // W_p[u, v, w] at woff + (u * V + v) * W + w
       const long long stride_u = (long long)b.mul * W, stride_v = W;
-      mine << "  {" << (k_is_x2 ? "true" : "false") << ", " << (k_is_x2 ? P.off2[p.in2] : P.off1[p.in1]) << ", "
+      mine << "  {" << (synth ? "true" : "false") << ", " << (k_is_x2 ? "true" : "false") << ", "
+           << (k_is_x2 ? P.off2[p.in2] : P.off1[p.in1]) << ", "
            << (k_is_x2 ? d2 : d1) << ", " << (k_is_x2 ? b.mul : a.mul) << ", "
            << (k_is_x2 ? P.off1[p.in1] : P.off2[p.in2]) << ", " << (k_is_x2 ? d1 : d2) << ", "
            << (k_is_x2 ? a.mul : b.mul) << ", " << p.woff << ", " << (k_is_x2 ? stride_v : stride_u) << ", "
@@ -273,7 +352,8 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   }
   s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
     << nzs.str() << "};\n";
-  s << "struct MPath { bool k_is_x2; int koff, dK, K, roff, dR, O; long long wbase, wk_stride, wo_stride; int nz_beg, "
+  s << "constexpr int DKA = " << dka << ";\n";
+  s << "struct MPath { bool synth, k_is_x2; int koff, dK, K, roff, dR, O; long long wbase, wk_stride, wo_stride; int nz_beg, "
        "nz_end; };\n";
   s << "constexpr int N_MPATH = " << n_path << ";\nconstexpr MPath mpaths[N_MPATH] = {\n" << ps.str() << "};\n";
   s << "struct Target { int out_off, d3, w0, path_beg, path_end; };\n";
@@ -286,19 +366,21 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
 
 int load_functions(e3x_plan* P, int dev) {
   std::lock_guard<std::mutex> lock(P->mu);
-  if (P->module[dev]) return E3X_OK;
-  hipModule_t mod = nullptr;
-  hipError_t err = hipModuleLoad(&mod, P->hsaco.c_str());
-  if (err != hipSuccess)
-    return fail(E3X_ERR_HIP, "hipModuleLoad(" + P->hsaco + ") failed: " + hipGetErrorString(err));
-  const std::string plain = "e3x_" + P->family + "_plain";
-  if (hipModuleGetFunction(&P->fn_plain[dev], mod, plain.c_str()) != hipSuccess)
-    return fail(E3X_ERR_HIP, "kernel " + plain + " missing from " + P->hsaco);
-  if (P->family == "uvu") {
-    if (hipModuleGetFunction(&P->fn_fused[dev], mod, "e3x_uvu_fused") != hipSuccess)
-      return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused missing from " + P->hsaco);
+  for (auto& K : P->subs) {
+    if (K->module[dev]) continue;
+    hipModule_t mod = nullptr;
+    hipError_t err = hipModuleLoad(&mod, K->hsaco.c_str());
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, "hipModuleLoad(" + K->hsaco + ") failed: " + hipGetErrorString(err));
+    const std::string plain = "e3x_" + P->family + "_plain";
+    if (hipModuleGetFunction(&K->fn_plain[dev], mod, plain.c_str()) != hipSuccess)
+      return fail(E3X_ERR_HIP, "kernel " + plain + " missing from " + K->hsaco);
+    if (P->family == "uvu") {
+      if (hipModuleGetFunction(&K->fn_fused[dev], mod, "e3x_uvu_fused") != hipSuccess)
+        return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused missing from " + K->hsaco);
+    }
+    K->module[dev] = mod;
   }
-  P->module[dev] = mod;
   return E3X_OK;
 }
 
@@ -365,20 +447,29 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
   if (n_uvu && n_uvw)
     return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: mixing uvu and uvw instructions in one plan is not implemented");
 
-  std::string src;
   const char* force_small = std::getenv("E3X_UVW_FORCE_VALU");
-  if (n_uvw && uvw_mfma_eligible(*P) && !(force_small && force_small[0] == '1')) {
-    P->family = "uvw_mfma";
-    rc = build_uvw_mfma_source(*P, &src);
-  } else if (n_uvw) {
-    P->family = "uvw_small";
-    rc = build_uvw_small_source(*P, &src);
+  std::vector<std::vector<int>> parts;
+  if (n_uvw) {
+    P->family = (uvw_mfma_eligible(*P) && !(force_small && force_small[0] == '1')) ? "uvw_mfma" : "uvw_small";
+    std::vector<int> all(P->paths.size());
+    for (size_t i = 0; i < all.size(); ++i) all[i] = (int)i;
+    parts.push_back(all);
   } else {
     P->family = "uvu";
-    rc = build_uvu_source(*P, &src);
+    parts = split_uvu_paths(*P);
   }
-  if (rc) return rc;
-  if ((rc = e3x::get_code_object(P->family, src, &P->key, &P->hsaco))) return rc;
+  for (auto& ids : parts) {
+    std::unique_ptr<SubKernel> K(new SubKernel);
+    K->path_ids = ids;
+    std::string src;
+    if (P->family == "uvw_mfma") rc = build_uvw_mfma_source(*P, &src);
+    else if (P->family == "uvw_small") rc = build_uvw_small_source(*P, *K, &src);
+    else rc = build_uvu_source(*P, *K, &src);
+    if (rc) return rc;
+    if ((rc = e3x::get_code_object(P->family, src, &K->key, &K->hsaco))) return rc;
+    P->key += (P->key.empty() ? "" : "+") + K->key;
+    P->subs.push_back(std::move(K));
+  }
   *out = P.release();
   return E3X_OK;
 }
@@ -425,20 +516,23 @@ extern "C" int e3x_tp_forward(e3x_plan* P, const void* x1, const void* x2, const
   if ((rc = load_functions(P, dev))) return rc;
   long long n_rows = Z;
   void* args[] = {(void*)&x1, (void*)&x2, (void*)&w, (void*)&out, (void*)&n_rows};
-  long long blocks;
-  unsigned grid_y = 1;
-  if (P->family == "uvw_mfma") {
-    blocks = (Z + 63) / 64;
-    grid_y = (unsigned)P->n_targets;
-  } else {
-    const int groups = 64 / P->lanes;
-    const long long items = (Z + groups - 1) / groups * P->chunks;
-    blocks = (items + 3) / 4;
+  for (auto& K : P->subs) {
+    long long blocks;
+    unsigned grid_y = 1;
+    if (P->family == "uvw_mfma") {
+      blocks = (Z + 63) / 64;
+      grid_y = (unsigned)P->n_targets;
+    } else {
+      const int groups = 64 / K->lanes;
+      const long long items = (Z + groups - 1) / groups * K->chunks;
+      blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
+    }
+    if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_forward: batch too large for one launch");
+    hipError_t err =
+        hipModuleLaunchKernel(K->fn_plain[dev], (unsigned)blocks, grid_y, 1, 64 * K->waves_per_block, 1, 1, 0, st, args, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_forward: launch failed: ") + hipGetErrorString(err));
   }
-  if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_forward: batch too large for one launch");
-  hipError_t err =
-      hipModuleLaunchKernel(P->fn_plain[dev], (unsigned)blocks, grid_y, 1, 256, 1, 1, 0, st, args, nullptr);
-  if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_tp_forward: launch failed: ") + hipGetErrorString(err));
   return E3X_OK;
 }
 
@@ -467,11 +561,14 @@ extern "C" int e3x_tp_gather_scatter(e3x_plan* P, const void* node_x, const void
   long long n_rows = num_out_nodes, n_src = num_src_nodes;
   void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&w,    (void*)&out,    (void*)&src,
                   (void*)&idx64,  (void*)&rowptr,    (void*)&perm, (void*)&n_rows, (void*)&n_src};
-  const long long items = n_rows * P->chunks;
-  const long long blocks = (items + 3) / 4;
-  if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
-  hipError_t err = hipModuleLaunchKernel(P->fn_fused[dev], (unsigned)blocks, 1, 1, 256, 1, 1, 0, st, args, nullptr);
-  if (err != hipSuccess)
-    return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
+  for (auto& K : P->subs) {
+    const long long items = n_rows * K->chunks;
+    const long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
+    if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
+    hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1, 0, st,
+                                           args, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
+  }
   return E3X_OK;
 }

@@ -203,5 +203,5 @@ def test_uvw_bf16_storage():
     xb, yb = x1.to(DEV).to(torch.bfloat16), x2.to(DEV).to(torch.bfloat16)
     out = tpb(xb, yb)
     assert out.dtype == torch.bfloat16
-    ref = otp.tp_forward(oracle_spec(tp), xb.float().cpu().numpy(), yb.float().cpu().numpy(), tpb.weight.float().cpu().numpy())
+    ref = otp.tp_forward(oracle_spec(tp), xb.float().cpu().numpy(), yb.float().cpu().numpy(), tpb.weight.detach().float().cpu().numpy())
     assert_close(out, ref, atol=2e-2, rtol=1e-2, what="bf16 uvw")
