@@ -133,7 +133,10 @@ std::vector<std::vector<int>> split_uvu_paths(const e3x_plan& P) {
   std::vector<char> usedo(P.out.size(), 0);
   for (const auto& p : P.paths)
     if (!usedo[p.out]) { usedo[p.out] = 1; acc += 2 * P.out[p.out].l + 1; }
-  const int want = env_int("E3X_UVU_SPLIT", acc > 128 ? 1 : 0);
+  // fp32: one kernel up to 128 accumulators per multiplicity index (measured faster on the 99-accumulator
+  // MACE set than four kernels); bf16 storage is ALU-bound and prefers the smaller kernels
+  const int limit = P.dtype == E3X_BF16 ? 48 : 128;
+  const int want = env_int("E3X_UVU_SPLIT", acc > limit ? 1 : 0);
   if (!want || P.paths.empty()) return {all};
   // an output irrep fed from several input-1 irreps ties those inputs together
   std::vector<int> group_of_in1(P.in1.size());
@@ -178,6 +181,7 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src) {
   int upl = 4;
   auto fits = [&](int u) {
     for (size_t a = 0; a < P.in1.size(); ++a) if (used1[a] && P.in1[a].mul % u) return false;
+    if (P.dtype == E3X_BF16 && u == 4 && accregs > 24) return false;  // measured: 2 per lane is faster there
     return u * (accregs + x1regs + wregs) + (int)P.in2_dim <= 200;
   };
   while (upl > 1 && !fits(upl)) upl /= 2;
@@ -563,7 +567,8 @@ extern "C" int e3x_tp_gather_scatter(e3x_plan* P, const void* node_x, const void
                   (void*)&idx64,  (void*)&rowptr,    (void*)&perm, (void*)&n_rows, (void*)&n_src};
   for (auto& K : P->subs) {
     const long long items = n_rows * K->chunks;
-    const long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
+    long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
+    blocks = (blocks + 7) / 8 * 8;  // the kernel deals contiguous eighths of the rows to the 8 XCDs
     if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
     hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1, 0, st,
                                            args, nullptr);
