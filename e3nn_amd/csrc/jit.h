@@ -9,6 +9,7 @@ extern const char* const kTplCommon;
 extern const char* const kTplUvu;
 extern const char* const kTplUvwSmall;
 extern const char* const kTplUvwMfma;
+extern const char* const kTplUvwMfmaBf16;
 
 std::string cache_dir();
 

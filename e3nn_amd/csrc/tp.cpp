@@ -322,7 +322,8 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
       const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1, d3 = 2 * P.out[c].l + 1;
       // GEMM passes per outer index: 2l+1 of the K operand when accumulators are scaled, 2 l3 + 1 when the
       // operand is synthesised; take the cheapest
-      const bool synth = env_int("E3X_UVW_SYNTH", 1) && d3 < std::min(d1, d2);
+      // (the bf16 kernel scales accumulators only: its matrix passes are cheap next to the fp32 epilogue)
+      const bool synth = P.dtype == E3X_F32 && env_int("E3X_UVW_SYNTH", 1) && d3 < std::min(d1, d2);
       const bool k_is_x2 = !synth && d2 < d1;
       if (synth) dka = std::max(dka, d1);
       const auto& C = e3x::wigner_3j(a.l, b.l, P.out[c].l);
@@ -364,7 +365,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   s << "constexpr int N_TARGET = " << n_target << ";\nconstexpr Target targets[N_TARGET] = {\n" << ts.str() << "};\n";
   s << "}  // namespace cfg\n";
   P.n_targets = n_target;
-  *src = s.str() + e3x::kTplCommon + e3x::kTplUvwMfma;
+  *src = s.str() + e3x::kTplCommon + (P.dtype == E3X_BF16 ? e3x::kTplUvwMfmaBf16 : e3x::kTplUvwMfma);
   return E3X_OK;
 }
 
