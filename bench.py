@@ -218,7 +218,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16,uvw,uvw_bf16 (default: all but uvw_bf16)")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16,uvw,uvw_bf16 (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported (no collectives, no sharding)")
@@ -229,7 +229,7 @@ def main():
 
     neq, ctx = bench_nequip(args, dev)
     other = {"nequip_uvu": neq}
-    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_bf16", "uvw"}
+    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_bf16", "uvw", "uvw_bf16"}
     if "copy" in want:
         other["copy_1GiB"] = bench_copy(args, dev)
     if "sh" in want:
@@ -241,7 +241,7 @@ def main():
     if "uvw" in want:
         other["uvw_dense_fp32"] = bench_uvw(args, dev)
     if "uvw_bf16" in want:
-        other["uvw_dense_bf16_storage"] = bench_uvw(args, dev, torch.bfloat16)
+        other["uvw_dense_bf16"] = bench_uvw(args, dev, torch.bfloat16)
     line = {
         "metric": "per-edge uvu TP edges/sec (L=2, fused gather + tensor product + scatter)",
         "value": neq["edges_per_s"],
