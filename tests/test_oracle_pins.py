@@ -266,3 +266,30 @@ def test_conv_matches_reference_golden(golden_tp):
     out = tp_gather_scatter(spec, g["node_x"], g["attr"], g["w"], g["src"], g["dst"], g["node_x"].shape[0])
     np.testing.assert_allclose(out, g["out"], atol=1e-12)
     assert not out[-1].any()
+
+
+# ---------------------------------------------------------------- rotations (equivariance tooling)
+def test_wigner_D_is_a_representation_and_w3j_is_invariant():
+    from oracle.rotation import irreps_D, random_rotation, wigner_D
+
+    rng = np.random.default_rng(7)
+    R1, R2 = random_rotation(rng), random_rotation(rng)
+    np.testing.assert_allclose(wigner_D(1, R1), R1, atol=1e-12)  # reference tests/o3/wigner_test.py:28-32 (x,y,z order)
+    for l in range(5):
+        D1, D2, D12 = wigner_D(l, R1), wigner_D(l, R2), wigner_D(l, R1 @ R2)
+        np.testing.assert_allclose(D1 @ D2, D12, atol=1e-10)
+        np.testing.assert_allclose(D1 @ D1.T, np.eye(2 * l + 1), atol=1e-10)
+    # C_ijk D_il D_jm D_kn = C_lmn  (reference tests/o3/wigner_test.py:15-25)
+    for l1, l2, l3 in ((1, 1, 1), (1, 2, 3), (2, 2, 2), (3, 3, 2), (2, 3, 3), (1, 3, 3)):
+        C = wigner_3j(l1, l2, l3)
+        Cr = np.einsum("ijk,il,jm,kn->lmn", C, wigner_D(l1, R1), wigner_D(l2, R1), wigner_D(l3, R1))
+        np.testing.assert_allclose(Cr, C, atol=1e-10)
+    # the oracle tensor product is equivariant under rotation and inversion
+    ins = otp.fully_connected_instructions("2x0e+2x1o+1x2e", "0e+1o+2e", "2x0e+2x1o+2x2e+1x1e")
+    spec = otp.make_spec("2x0e+2x1o+1x2e", "0e+1o+2e", "2x0e+2x1o+2x2e+1x1e", ins)
+    x1, x2, w = rng.standard_normal((4, 13)), rng.standard_normal((4, 9)), rng.standard_normal(spec.weight_numel)
+    for improper in (False, True):
+        Da, Db, Dc = (irreps_D(s, R1, improper) for s in ("2x0e+2x1o+1x2e", "0e+1o+2e", "2x0e+2x1o+2x2e+1x1e"))
+        lhs = otp.tp_forward(spec, x1 @ Da.T, x2 @ Db.T, w)
+        rhs = otp.tp_forward(spec, x1, x2, w) @ Dc.T
+        np.testing.assert_allclose(lhs, rhs, atol=1e-10)
