@@ -125,6 +125,36 @@ def bench_nequip(args, dev):
         "edges_per_s_incl_sort": E / ((ms + sort_ms) * 1e-3),
     }  # fmt: skip
     ctx = dict(tp=tp, node_x=node_x, attr=attr, w=w, src=src_t, dst=dst_t, N=N, out=out[0])
+    if getattr(args, "locality_variants", False):
+        # same graph, friendlier numbering: (a) edge list sorted by destination, as neighbour-list codes emit it;
+        # (b) nodes renumbered along a Morton curve of their positions as well (a spatially sorted system)
+        def timed(order_nodes):
+            if order_nodes:
+                c = np.floor(pos / 2.5).astype(np.uint64)
+
+                def spread(v):
+                    v = v & np.uint64(0x3FF)
+                    for sh, m in ((16, 0x30000FF), (8, 0x300F00F), (4, 0x30C30C3), (2, 0x9249249)):
+                        v = (v | (v << np.uint64(sh))) & np.uint64(m)
+                    return v
+
+                key = spread(c[:, 0]) | (spread(c[:, 1]) << np.uint64(1)) | (spread(c[:, 2]) << np.uint64(2))
+                rank = np.empty(N, np.int64)
+                rank[np.argsort(key, kind="stable")] = np.arange(N)
+                s2, d2 = rank[src], rank[dst]
+                nx = torch.empty_like(node_x)
+                nx[torch.from_numpy(rank).to(dev)] = node_x
+            else:
+                s2, d2, nx = src, dst, node_x
+            o = np.argsort(d2, kind="stable")
+            ot = torch.from_numpy(o).to(dev)
+            e2 = DstSortedEdges(torch.from_numpy(s2[o]).to(dev), torch.from_numpy(d2[o]).to(dev), N)
+            a2, w2 = attr[ot].contiguous(), w[ot].contiguous()
+            return event_time_ms(lambda: tp.forward_gather_scatter(nx, a2, w2, edges=e2), args.steps, args.warmup)
+
+        for name, flag in (("sorted_edges", False), ("sorted_edges_morton_nodes", True)):
+            t = timed(flag)
+            res[name] = {"ms": t, "edges_per_s": E / (t * 1e-3), "roofline_frac": bytes_algo / (t * 1e-3) / 1e9 / HBM_PEAK_GBS}
     return res, ctx
 
 
@@ -218,6 +248,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--locality-variants", action="store_true", help="also time the headline graph with sorted edges / Morton node ids")
     ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16,uvw,uvw_bf16 (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
