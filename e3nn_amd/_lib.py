@@ -48,6 +48,8 @@ _SIGNATURES = {
     "e3x_index_check": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p]),
     "e3x_tp_gather_scatter": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_int64, c_int64, c_int64, c_void_p]),
+    "e3x_tp_backward_w_x2": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                     c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     "e3x_sh_forward": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int64,
                                c_int32, c_void_p]),
     "e3x_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -35,6 +35,7 @@ struct SubKernel {
   hipModule_t module[kMaxDevices] = {nullptr};
   hipFunction_t fn_plain[kMaxDevices] = {nullptr};
   hipFunction_t fn_fused[kMaxDevices] = {nullptr};
+  hipFunction_t fn_bwd_edge[kMaxDevices] = {nullptr};
 };
 
 struct e3x_plan {
@@ -136,7 +137,12 @@ std::vector<std::vector<int>> split_uvu_paths(const e3x_plan& P) {
   // fp32: one kernel up to 128 accumulators per multiplicity index (measured faster on the 99-accumulator
   // MACE set than four kernels); bf16 storage is ALU-bound and prefers the smaller kernels
   const int limit = P.dtype == E3X_BF16 ? 48 : 128;
-  const int want = env_int("E3X_UVU_SPLIT", acc > limit ? 1 : 0);
+  int x1regs = 0;
+  std::vector<char> used1(P.in1.size(), 0);
+  for (const auto& p : P.paths)
+    if (!used1[p.in1]) { used1[p.in1] = 1; x1regs += 2 * P.in1[p.in1].l + 1; }
+  // (transposed plans of the backward pass have many input irreps instead of many outputs)
+  const int want = env_int("E3X_UVU_SPLIT", (acc > limit || x1regs > 64) ? 1 : 0);
   if (!want || P.paths.empty()) return {all};
   // an output irrep fed from several input-1 irreps ties those inputs together
   std::vector<int> group_of_in1(P.in1.size());
@@ -384,6 +390,8 @@ int load_functions(e3x_plan* P, int dev) {
     if (P->family == "uvu") {
       if (hipModuleGetFunction(&K->fn_fused[dev], mod, "e3x_uvu_fused") != hipSuccess)
         return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused missing from " + K->hsaco);
+      if (hipModuleGetFunction(&K->fn_bwd_edge[dev], mod, "e3x_uvu_bwd_edge") != hipSuccess)
+        return fail(E3X_ERR_HIP, "kernel e3x_uvu_bwd_edge missing from " + K->hsaco);
     }
     K->module[dev] = mod;
   }
@@ -572,10 +580,62 @@ extern "C" int e3x_tp_gather_scatter(e3x_plan* P, const void* node_x, const void
     long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
     blocks = (blocks + 7) / 8 * 8;  // the kernel deals contiguous eighths of the rows to the 8 XCDs
     if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
-    hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1, 0, st,
-                                           args, nullptr);
+    hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1,
+                                           (unsigned)env_int("E3X_UVU_LDS_PAD", 0), st, args, nullptr);
     if (err != hipSuccess)
       return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
+  }
+  return E3X_OK;
+}
+
+extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2, const void* w, const void* grad_out,
+                                    const void* src, const void* dst, int idx_bits, void* grad_w, void* grad_x2,
+                                    int64_t E, int64_t num_src_nodes, int64_t num_out_nodes, void* stream) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: null plan");
+  if (P->family != "uvu") return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: the plan must be all-uvu");
+  if (P->shared_weights && P->weight_numel && grad_w)
+    return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: the gradient of shared weights is not implemented");
+  if (idx_bits != 32 && idx_bits != 64) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: idx_bits must be 32 or 64");
+  if (E < 0 || num_src_nodes < 0 || num_out_nodes < 0) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: negative size");
+  if ((src == nullptr) != (dst == nullptr))
+    return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: give both index arrays or neither");
+  if (E == 0 || (!grad_w && !grad_x2)) return E3X_OK;
+  if (!grad_out || (P->in1_dim && !x1) || (P->in2_dim && !x2) || (P->weight_numel && !w))
+    return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  int dev, rc;
+  if ((rc = current_device(&dev))) return rc;
+  const size_t esz = P->dtype == E3X_BF16 ? 2 : 4;
+  if (P->paths.empty() || P->in2_dim == 0) grad_x2 = P->paths.empty() ? grad_x2 : nullptr;
+  if (P->paths.empty()) {
+    if (grad_x2 && (rc = e3x::fill_zero_bytes(grad_x2, (size_t)E * P->in2_dim * esz, st))) return rc;
+    return E3X_OK;
+  }
+  if ((rc = load_functions(P, dev))) return rc;
+  int x2_atomic = 0;
+  for (auto& K : P->subs)
+    if (K->chunks > 1) x2_atomic = 1;
+  if (P->subs.size() > 1) x2_atomic = 1;
+  if (grad_x2 && x2_atomic) {
+    if (P->dtype != E3X_F32)
+      return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: grad_x2 in bf16 storage needs a single-kernel plan");
+    if ((rc = e3x::fill_zero_bytes(grad_x2, (size_t)E * P->in2_dim * esz, st))) return rc;
+  }
+  // weights of paths with an unused multiplicity tail and unweighted paths are never written: start from zero
+  if (grad_w && P->weight_numel && (rc = e3x::fill_zero_bytes(grad_w, (size_t)E * P->weight_numel * esz, st))) return rc;
+  int idx64 = idx_bits == 64;
+  long long n_edges = E, n_src = num_src_nodes;
+  void* args[] = {(void*)&x1,  (void*)&x2,     (void*)&w,       (void*)&grad_out,  (void*)&src,     (void*)&dst,
+                  (void*)&idx64, (void*)&grad_w, (void*)&grad_x2, (void*)&x2_atomic, (void*)&n_edges, (void*)&n_src};
+  for (auto& K : P->subs) {
+    const int groups = 64 / K->lanes;
+    const long long items = (E + groups - 1) / groups * K->chunks;
+    const long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
+    if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: too many edges for one launch");
+    hipError_t err =
+        hipModuleLaunchKernel(K->fn_bwd_edge[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1, 0, st, args, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_backward_w_x2: launch failed: ") + hipGetErrorString(err));
   }
   return E3X_OK;
 }

@@ -20,7 +20,16 @@ class DstSortedEdges:
     ``IndexError``.  int32 and int64 indices give identical results.
     """
 
+    def transposed(self) -> "DstSortedEdges":
+        """The same edges with source and destination exchanged (grouped by ``edge_src``); the backward
+        pass with respect to the node features scatters onto the sources.  Built once, cached."""
+        if self._transposed is None:
+            self._transposed = DstSortedEdges(self.edge_dst, self.edge_src, self.num_src_nodes, self.num_nodes)
+            self._transposed._transposed = self
+        return self._transposed
+
     def __init__(self, edge_src: torch.Tensor, edge_dst: torch.Tensor, num_nodes: int, num_src_nodes: int = None):
+        self._transposed = None
         if not (edge_src.is_cuda and edge_dst.is_cuda):
             raise RuntimeError("DstSortedEdges needs index tensors on the GPU")
         if edge_src.dtype not in (torch.int32, torch.int64) or edge_dst.dtype not in (torch.int32, torch.int64):

@@ -60,29 +60,27 @@ def _num_elements(mode, m1, m2):
 
 
 class _Plan:
-    """Owner of one ``e3x_plan`` handle."""
+    """Owner of one ``e3x_plan`` handle: a fused kernel specialised to one instruction set."""
 
-    def __init__(self, tp: "TensorProduct", dtype: torch.dtype):
+    def __init__(self, irreps_in1, irreps_in2, irreps_out, instructions, shared_weights: bool, dtype: torch.dtype):
+        """``instructions``: tuples ``(i_in1, i_in2, i_out, mode, has_weight, path_weight)``, path weights final."""
         L = _lib.lib()
         mk = lambda irreps: (_lib.Irrep * max(1, len(irreps)))(*[_lib.Irrep(mul, ir.l, ir.p) for mul, ir in irreps])  # noqa: E731
-        in1, in2, out = mk(tp.irreps_in1), mk(tp.irreps_in2), mk(tp.irreps_out)
-        ins = (_lib.Instruction * max(1, len(tp.instructions)))(
-            *[
-                _lib.Instruction(t.i_in1, t.i_in2, t.i_out, _KERNEL_MODES[t.connection_mode], int(t.has_weight), t.path_weight)
-                for t in tp.instructions
-            ]
+        in1, in2, out = mk(irreps_in1), mk(irreps_in2), mk(irreps_out)
+        ins = (_lib.Instruction * max(1, len(instructions)))(
+            *[_lib.Instruction(a, b, c, _KERNEL_MODES[mode], int(hw), pw) for a, b, c, mode, hw, pw in instructions]
         )
         desc = _lib.TpDesc(
-            len(tp.irreps_in1), len(tp.irreps_in2), len(tp.irreps_out), len(tp.instructions), in1, in2, out, ins,
-            int(tp.shared_weights), _DTYPES[dtype],
+            len(irreps_in1), len(irreps_in2), len(irreps_out), len(instructions), in1, in2, out, ins,
+            int(shared_weights), _DTYPES[dtype],
         )  # fmt: skip
         handle = _lib.c_void_p()
         _lib.check(L.e3x_tp_plan_create(ctypes.byref(desc), ctypes.byref(handle)))
         self.handle = handle
         wn, fam, key = ctypes.c_int64(), ctypes.c_char_p(), ctypes.c_char_p()
         _lib.check(L.e3x_tp_plan_info(handle, ctypes.byref(wn), None, None, None, ctypes.byref(fam), ctypes.byref(key)))
-        assert wn.value == tp.weight_numel, (wn.value, tp.weight_numel)
-        self.family, self.key = fam.value.decode(), key.value.decode()
+        self.weight_numel, self.family, self.key = wn.value, fam.value.decode(), key.value.decode()
+        self.out_dim = irreps_out.dim
 
     def __del__(self):
         try:
@@ -92,44 +90,127 @@ class _Plan:
         except Exception:
             pass
 
-
-class _TensorProductFn(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, x1, x2, w, tp):
+    def forward(self, x1, x2, w):
         Z = x1.shape[0]
-        out = torch.empty(Z, tp.irreps_out.dim, dtype=x1.dtype, device=x1.device)
-        plan = tp._plan(x1.dtype)
+        out = torch.empty(Z, self.out_dim, dtype=x1.dtype, device=x1.device)
         with torch.cuda.device(x1.device):
             _lib.check(
                 _lib.lib().e3x_tp_forward(
-                    plan.handle, _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(w), _lib.ptr(out), Z, _lib.stream_ptr(x1.device)
+                    self.handle, _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(w), _lib.ptr(out), Z, _lib.stream_ptr(x1.device)
                 )
             )
         return out
 
-    @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("the tensor-product backward kernels are not implemented")
-
-
-class _GatherScatterFn(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, node_x, edge_attr, w, tp, edges):
-        out = torch.empty(edges.num_nodes, tp.irreps_out.dim, dtype=node_x.dtype, device=node_x.device)
-        plan = tp._plan(node_x.dtype)
-        with torch.cuda.device(node_x.device):
+    def gather_scatter(self, table, edge_attr, w, gather_idx, edges, num_table_rows):
+        """``out[n] = sum_{e: edges groups e under n} TP(table[gather_idx[e]], edge_attr[e], w[e])``."""
+        out = torch.empty(edges.num_nodes, self.out_dim, dtype=table.dtype, device=table.device)
+        with torch.cuda.device(table.device):
             _lib.check(
                 _lib.lib().e3x_tp_gather_scatter(
-                    plan.handle, _lib.ptr(node_x), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(edges.edge_src),
-                    edges.edge_src.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(out),
-                    edges.num_edges, node_x.shape[0], edges.num_nodes, _lib.stream_ptr(node_x.device),
+                    self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(gather_idx),
+                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(out),
+                    edges.num_edges, num_table_rows, edges.num_nodes, _lib.stream_ptr(table.device),
                 )  # fmt: skip
             )
         return out
 
+    def backward_w_x2(self, x1, x2, w, grad_out, src, dst, want_w, want_x2, num_edges):
+        gw = torch.empty(num_edges, self.weight_numel, dtype=x1.dtype, device=x1.device) if want_w else None
+        gx2 = torch.empty(num_edges, x2.shape[1], dtype=x1.dtype, device=x1.device) if want_x2 else None
+        bits = src.element_size() * 8 if src is not None else 64
+        with torch.cuda.device(x1.device):
+            _lib.check(
+                _lib.lib().e3x_tp_backward_w_x2(
+                    self.handle, _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(w), _lib.ptr(grad_out), _lib.ptr(src), _lib.ptr(dst),
+                    bits, _lib.ptr(gw), _lib.ptr(gx2), num_edges, x1.shape[0], grad_out.shape[0], _lib.stream_ptr(x1.device),
+                )  # fmt: skip
+            )
+        return gw, gx2
+
+
+def _w3j_swap_sign(tp, t):
+    # exchanging two indices of the real Wigner 3j tensor multiplies it by (-1)^(l1 + l2 + l3)
+    l = tp.irreps_in1[t.i_in1].ir.l + tp.irreps_in2[t.i_in2].ir.l + tp.irreps_out[t.i_out].ir.l
+    return -1.0 if l % 2 else 1.0
+
+
+def _permuted_weights(tp, w, perm):
+    """Per-instruction ``[..., U, V, W]`` weight blocks of a ``uvw`` product with their last three axes permuted."""
+    if tp.weight_numel == 0:
+        return w
+    batch = w.shape[:-1]
+    nb = len(batch)
+    blocks = [v.permute(*range(nb), *(nb + p for p in perm)).reshape(batch + (-1,)) for v in tp.weight_views(w)]
+    return torch.cat(blocks, dim=-1).contiguous()
+
+
+class _TensorProductFn(torch.autograd.Function):
+    """Plain tensor product.  The map is trilinear, so every gradient is again a tensor product:
+    d/dx1 and (for ``uvw``) d/dx2 run the forward kernels on transposed plans; d/dw and d/dx2 of
+    ``uvu`` have their own edge-parallel kernel."""
+
     @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("the tensor-product backward kernels are not implemented")
+    def forward(ctx, x1, x2, w, tp):
+        ctx.tp = tp
+        ctx.save_for_backward(x1, x2, w)
+        return tp._plan(x1.dtype).forward(x1, x2, w)
+
+    @staticmethod
+    def backward(ctx, g):
+        tp = ctx.tp
+        x1, x2, w = ctx.saved_tensors
+        g = g.contiguous()
+        need1, need2, needw = ctx.needs_input_grad[:3]
+        g1 = g2 = gw = None
+        mode = tp._live_mode()
+        if mode == "uvu":
+            if need1:
+                g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, w)
+            if need2 or (needw and tp.weight_numel):
+                if tp.shared_weights and needw and tp.weight_numel:
+                    raise NotImplementedError("the gradient of shared uvu weights has no kernel")
+                gw, g2 = tp._plan(x1.dtype).backward_w_x2(x1, x2, w, g, None, None, needw and tp.weight_numel > 0, need2, x1.shape[0])
+        elif mode == "uvw":
+            if needw and tp.weight_numel:
+                raise NotImplementedError(
+                    "the weight gradient of uvw tensor products has no kernel yet; call weight.requires_grad_(False) "
+                    "to differentiate with respect to the inputs only"
+                )
+            if need1:
+                g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, _permuted_weights(tp, w, (2, 1, 0)))
+            if need2:
+                g2 = tp._grad_plan("x2", x1.dtype).forward(x1, g, _permuted_weights(tp, w, (0, 2, 1)))
+        else:
+            g1, g2 = torch.zeros_like(x1), torch.zeros_like(x2)
+            gw = torch.zeros_like(w) if needw else None
+        return g1, g2, gw, None
+
+
+class _GatherScatterFn(torch.autograd.Function):
+    """``scatter(tp(node_x[src], edge_attr, w), dst)``; d/dnode_x is the same fused kernel on the transposed
+    plan with the roles of source and destination exchanged."""
+
+    @staticmethod
+    def forward(ctx, node_x, edge_attr, w, tp, edges):
+        ctx.tp, ctx.edges = tp, edges
+        ctx.save_for_backward(node_x, edge_attr, w)
+        return tp._plan(node_x.dtype).gather_scatter(node_x, edge_attr, w, edges.edge_src, edges, node_x.shape[0])
+
+    @staticmethod
+    def backward(ctx, g):
+        tp, edges = ctx.tp, ctx.edges
+        node_x, edge_attr, w = ctx.saved_tensors
+        g = g.contiguous()
+        need1, need2, needw = ctx.needs_input_grad[:3]
+        g1 = g2 = gw = None
+        if need1:
+            rev = edges.transposed()
+            g1 = tp._grad_plan("x1", node_x.dtype).gather_scatter(g, edge_attr, w, edges.edge_dst, rev, g.shape[0])
+        if need2 or (needw and tp.weight_numel):
+            gw, g2 = tp._plan(node_x.dtype).backward_w_x2(
+                node_x, edge_attr, w, g, edges.edge_src, edges.edge_dst, needw and tp.weight_numel > 0, need2, edges.num_edges
+            )
+        return g1, g2, gw, None, None
 
 
 class TensorProduct(torch.nn.Module):
@@ -264,17 +345,59 @@ class TensorProduct(torch.nn.Module):
         self._plans = {}
 
     # ------------------------------------------------------------------ plans
+    def _kernel_instructions(self):
+        return [(t.i_in1, t.i_in2, t.i_out, t.connection_mode, t.has_weight, t.path_weight) for t in self.instructions]
+
+    def _live_mode(self):
+        live = {t.connection_mode for t in self.instructions if 0 not in t.path_shape}
+        return next(iter(live)) if live else None
+
     def _plan(self, dtype: torch.dtype) -> _Plan:
         if dtype not in _DTYPES:
             raise TypeError(f"TensorProduct kernels support float32 and bfloat16 storage, got {dtype}")
         plan = self._plans.get(dtype)
         if plan is None:
-            plan = self._plans[dtype] = _Plan(self, dtype)
+            plan = self._plans[dtype] = _Plan(
+                self.irreps_in1, self.irreps_in2, self.irreps_out, self._kernel_instructions(), self.shared_weights, dtype
+            )
+            assert plan.weight_numel == self.weight_numel, (plan.weight_numel, self.weight_numel)
+        return plan
+
+    def _grad_plan(self, wrt: str, dtype: torch.dtype) -> _Plan:
+        """Transposed plan whose forward pass is the gradient with respect to ``x1`` or (``uvw`` only) ``x2``.
+
+        d out / d x1 contracts the same Wigner tensor over (j, k) instead of (i, j): a tensor product
+        ``irreps_out x irreps_in2 -> irreps_in1`` with the index-swap sign folded into the path weight
+        (``uvw`` also needs the weight blocks transposed, see ``_permuted_weights``)."""
+        key = (wrt, dtype)
+        plan = self._plans.get(key)
+        if plan is None:
+            ins = []
+            for t in self.instructions:
+                pw = t.path_weight * _w3j_swap_sign(self, t)
+                if wrt == "x1":
+                    ins.append((t.i_out, t.i_in2, t.i_in1, t.connection_mode, t.has_weight, pw))
+                else:
+                    ins.append((t.i_in1, t.i_out, t.i_in2, t.connection_mode, t.has_weight, pw))
+            if wrt == "x1":
+                plan = _Plan(self.irreps_out, self.irreps_in2, self.irreps_in1, ins, self.shared_weights, dtype)
+            else:
+                assert self._live_mode() in ("uvw", None)
+                plan = _Plan(self.irreps_in1, self.irreps_out, self.irreps_in2, ins, self.shared_weights, dtype)
+            self._plans[key] = plan
         return plan
 
     def compile(self, dtype: torch.dtype = torch.float32) -> "TensorProduct":
-        """Builds (or finds in the kernel cache) the specialised kernel now; needs no GPU."""
+        """Builds (or finds in the kernel cache) the specialised kernels now; needs no GPU."""
         self._plan(dtype)
+        return self
+
+    def compile_backward(self, dtype: torch.dtype = torch.float32) -> "TensorProduct":
+        """Also builds the transposed plans the backward pass uses."""
+        self._plan(dtype)
+        self._grad_plan("x1", dtype)
+        if self._live_mode() == "uvw":
+            self._grad_plan("x2", dtype)
         return self
 
     def __getstate__(self):

@@ -101,9 +101,16 @@ def all_tensor_products():
     return out
 
 
+# instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
+BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
+                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "mfma_small", "odd_mul"]  # fmt: skip
+
+
 def prebuild(verbose=True):
     for name, tp, dtypes in all_tensor_products():
         for dt in dtypes:
             plan = tp._plan(dt)
             if verbose:
                 print(f"kernel {name:32s} {str(dt):16s} {plan.key}", flush=True)
+        if name in BACKWARD_CASES:
+            tp.compile_backward(torch.float32)

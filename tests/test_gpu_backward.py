@@ -1,0 +1,91 @@
+"""GPU parity of the backward pass: gradients from the HIP kernels against torch autograd (float64) through the
+CPU restatement of the reference's einsum graph (oracle/torch_cpu.py)."""
+import numpy as np
+import pytest
+import torch
+
+from e3nn_amd.nn import DstSortedEdges
+from oracle.torch_cpu import tp_forward_torch, tp_gather_scatter_torch
+from tests import kernel_sets as ks
+from tests.helpers import assert_close, oracle_spec, seeded
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _oracle_grads(fn, tensors, cot):
+    ts = [t.double().clone().requires_grad_(True) for t in tensors]
+    out = fn(*ts)
+    out.backward(cot.double())
+    return out.detach(), [t.grad for t in ts]
+
+
+@pytest.mark.parametrize("maker,Z", [
+    (lambda: ks.golden_tp("uvu_merged_cfg3_like_mul4"), 9), (lambda: ks.golden_tp("uvu_builderA_cfg4_like_mul2"), 7),
+    (lambda: ks.cfg3(True), 130), (lambda: ks.cfg3(False), 65), (lambda: ks.cfg4("A"), 17), (ks.odd_mul, 33),
+])  # fmt: skip
+def test_uvu_plain_gradients(maker, Z):
+    tp = maker()
+    spec = oracle_spec(tp)
+    x1, x2, w = seeded(Z, tp.irreps_in1.dim, seed=1), seeded(Z, tp.irreps_in2.dim, seed=2), seeded(Z, tp.weight_numel, seed=3)
+    cot = seeded(Z, tp.irreps_out.dim, seed=4)
+    ref_out, (r1, r2, rw) = _oracle_grads(lambda a, b, c: tp_forward_torch(spec, a, b, c), (x1, x2, w), cot)
+    a, b, c = (t.to(DEV).requires_grad_(True) for t in (x1, x2, w))
+    out = tp(a, b, c)
+    out.backward(cot.to(DEV))
+    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
+    assert_close(out, ref_out.numpy(), atol=1e-4 * scale(ref_out))
+    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dx1")
+    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
+    assert_close(c.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dw")
+
+
+@pytest.mark.parametrize("maker,N,E,idx", [(lambda: ks.cfg3(True), 120, 3000, torch.int64), (lambda: ks.cfg3(False), 50, 900, torch.int32),
+                                           (lambda: ks.cfg4("A"), 25, 300, torch.int32)])  # fmt: skip
+def test_fused_message_gradients(maker, N, E, idx):
+    tp = maker()
+    spec = oracle_spec(tp)
+    g = torch.Generator().manual_seed(7)
+    src, dst = torch.randint(0, N, (E,), generator=g), torch.randint(0, N - 2, (E,), generator=g)
+    node_x, attr, w = seeded(N, tp.irreps_in1.dim, seed=1), seeded(E, tp.irreps_in2.dim, seed=2), seeded(E, tp.weight_numel, seed=3)
+    cot = seeded(N, tp.irreps_out.dim, seed=4)
+    ref_out, (r1, r2, rw) = _oracle_grads(lambda a, b, c: tp_gather_scatter_torch(spec, a, b, c, src, dst, N), (node_x, attr, w), cot)
+    a, b, c = (t.to(DEV).requires_grad_(True) for t in (node_x, attr, w))
+    edges = DstSortedEdges(src.to(idx).to(DEV), dst.to(idx).to(DEV), N)
+    out = tp.forward_gather_scatter(a, b, c, edges=edges)
+    out.backward(cot.to(DEV))
+    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
+    assert_close(out, ref_out.numpy(), atol=1e-4 * scale(ref_out))
+    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dnode_x")
+    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dedge_attr")
+    assert_close(c.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dweight")
+    # only some inputs require a gradient
+    a2, c2 = node_x.to(DEV).requires_grad_(True), w.to(DEV)
+    tp.forward_gather_scatter(a2, attr.to(DEV), c2, edges=edges).backward(cot.to(DEV))
+    assert torch.equal(a2.grad, a.grad)
+
+
+@pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.mfma_small, 70),
+                                     (lambda: ks.golden_tp("fctp_per_sample_weights"), 5)])  # fmt: skip
+def test_uvw_input_gradients(maker, Z):
+    tp = maker().to(DEV)
+    spec = oracle_spec(tp)
+    x1, x2 = seeded(Z, tp.irreps_in1.dim, seed=1), seeded(Z, tp.irreps_in2.dim, seed=2)
+    w = seeded(*((Z,) if not tp.shared_weights else ()), tp.weight_numel, seed=3) / 4
+    cot = seeded(Z, tp.irreps_out.dim, seed=4)
+    ref_out, (r1, r2) = _oracle_grads(lambda a, b: tp_forward_torch(spec, a, b, w.double()), (x1, x2), cot)
+    a, b = (t.to(DEV).requires_grad_(True) for t in (x1, x2))
+    out = tp(a, b, w.to(DEV))
+    out.backward(cot.to(DEV))
+    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
+    assert_close(out, ref_out.numpy(), atol=1e-4 * scale(ref_out))
+    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dx1")
+    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
+
+
+def test_missing_backward_kernels_fail_loudly():
+    tp = ks.cfg1().to(DEV)
+    x1, x2 = seeded(4, 64).to(DEV), seeded(4, 9).to(DEV)
+    out = tp(x1, x2)  # internal weights require a gradient
+    with pytest.raises(NotImplementedError):
+        out.sum().backward()
