@@ -52,6 +52,8 @@ _SIGNATURES = {
                                      c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     "e3x_sh_forward": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int64,
                                c_int32, c_void_p]),
+    "e3x_sh_backward": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+                                c_int32, c_void_p]),
     "e3x_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
 }  # fmt: skip
 

@@ -144,6 +144,108 @@ __global__ __launch_bounds__(kWave* kWavesPerBlock) void sh_tile_kernel(const fl
   }
 }
 
+// ---------------------------------------------------------------- backward, l <= 3
+// Forward-mode duals: every polynomial carries its gradient with respect to the (normalised)
+// input, so the derivative code is the forward code (no hand-derived formulas to get wrong).
+struct Dual {
+  float v, dx, dy, dz;
+};
+__device__ __forceinline__ Dual operator+(Dual a, Dual b) { return {a.v + b.v, a.dx + b.dx, a.dy + b.dy, a.dz + b.dz}; }
+__device__ __forceinline__ Dual operator-(Dual a, Dual b) { return {a.v - b.v, a.dx - b.dx, a.dy - b.dy, a.dz - b.dz}; }
+__device__ __forceinline__ Dual operator*(Dual a, Dual b) {
+  return {a.v * b.v, fmaf(a.v, b.dx, a.dx * b.v), fmaf(a.v, b.dy, a.dy * b.v), fmaf(a.v, b.dz, a.dz * b.v)};
+}
+__device__ __forceinline__ Dual operator*(float c, Dual a) { return {c * a.v, c * a.dx, c * a.dy, c * a.dz}; }
+
+template <int LMAX>
+__device__ __forceinline__ void sh_poly_dual(Dual x, Dual y, Dual z, Dual (&o)[(LMAX + 1) * (LMAX + 1)]) {
+  o[0] = {1.f, 0.f, 0.f, 0.f};
+  if constexpr (LMAX >= 1) {
+    const float c = 1.7320508075688772f;
+    o[1] = c * x;
+    o[2] = c * y;
+    o[3] = c * z;
+  }
+  if constexpr (LMAX >= 2) {
+    const float r15 = 3.872983346207417f, r5 = 2.23606797749979f;
+    const Dual y2 = y * y, s = x * x + z * z;
+    const Dual a20 = r15 * (x * z);
+    const Dual a24 = (0.5f * r15) * (z * z - x * x);
+    o[4] = a20;
+    o[5] = r15 * (x * y);
+    o[6] = r5 * (y2 - 0.5f * s);
+    o[7] = r15 * (y * z);
+    o[8] = a24;
+    if constexpr (LMAX >= 3) {
+      const float r7 = 2.6457513110645907f, c0 = 1.0801234497346435f, c2 = 1.6201851746019651f;
+      const Dual t = 4.0f * y2 - s;
+      o[9] = c0 * (a20 * z + a24 * x);
+      o[10] = r7 * (a20 * y);
+      o[11] = c2 * (t * x);
+      o[12] = (0.5f * r7) * (y * (2.0f * y2 - 3.0f * s));
+      o[13] = c2 * (z * t);
+      o[14] = r7 * (a24 * y);
+      o[15] = c0 * (a24 * z - a20 * x);
+    }
+  }
+}
+
+template <int LMAX, bool NORMALIZE>
+__global__ __launch_bounds__(256) void sh_bwd_kernel(const float* __restrict__ xyz, const float* __restrict__ gout,
+                                                     float* __restrict__ gxyz, long long n, Scale4 sc) {
+  constexpr int NC = (LMAX + 1) * (LMAX + 1);
+  const long long v = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (v >= n) return;
+  float x = xyz[v * 3 + 0], y = xyz[v * 3 + 1], z = xyz[v * 3 + 2];
+  float inv = 1.0f;
+  bool clamped = false;
+  if constexpr (NORMALIZE) {
+    const float nrm = sqrtf(x * x + y * y + z * z);
+    clamped = nrm < 1e-12f;
+    inv = 1.0f / fmaxf(nrm, 1e-12f);
+    x *= inv;
+    y *= inv;
+    z *= inv;
+  }
+  Dual o[NC];
+  sh_poly_dual<LMAX>(Dual{x, 1.f, 0.f, 0.f}, Dual{y, 0.f, 1.f, 0.f}, Dual{z, 0.f, 0.f, 1.f}, o);
+  float gx = 0.f, gy = 0.f, gz = 0.f;
+  const float* g = gout + v * NC;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int l = c >= 9 ? 3 : (c >= 4 ? 2 : (c >= 1 ? 1 : 0));
+    const float gc = g[c] * sc.s[l];
+    gx = fmaf(gc, o[c].dx, gx);
+    gy = fmaf(gc, o[c].dy, gy);
+    gz = fmaf(gc, o[c].dz, gz);
+  }
+  if constexpr (NORMALIZE) {
+    // x / max(|x|, eps): for |x| >= eps the Jacobian is (I - u u^T) / |x|, below it is I / eps
+    if (!clamped) {
+      const float dot = gx * x + gy * y + gz * z;
+      gx = (gx - x * dot) * inv;
+      gy = (gy - y * dot) * inv;
+      gz = (gz - z * dot) * inv;
+    } else {
+      gx *= inv;
+      gy *= inv;
+      gz *= inv;
+    }
+  }
+  gxyz[v * 3 + 0] = gx;
+  gxyz[v * 3 + 1] = gy;
+  gxyz[v * 3 + 2] = gz;
+}
+
+template <int LMAX>
+void launch_bwd(bool normalize, const float* xyz, const float* gout, float* gxyz, long long n, Scale4 sc, hipStream_t st) {
+  const long long blocks = (n + 255) / 256;
+  if (normalize)
+    hipLaunchKernelGGL((sh_bwd_kernel<LMAX, true>), dim3((unsigned)blocks), dim3(256), 0, st, xyz, gout, gxyz, n, sc);
+  else
+    hipLaunchKernelGGL((sh_bwd_kernel<LMAX, false>), dim3((unsigned)blocks), dim3(256), 0, st, xyz, gout, gxyz, n, sc);
+}
+
 // ---------------------------------------------------------------- generic path
 constexpr int kMaxL = 12;
 constexpr int kMaxCols = (kMaxL + 1) * (kMaxL + 1);
@@ -322,5 +424,38 @@ extern "C" int e3x_sh_forward(const int32_t* ls, int32_t n_ls, int32_t normalize
                        (float*)out, (long long)n, lmax, n_out, (int)normalize, cm);
   }
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_sh_forward: kernel launch failed");
+  return E3X_OK;
+}
+
+extern "C" int e3x_sh_backward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization,
+                               const void* xyz, const void* grad_out, void* grad_xyz, int64_t n, int32_t dtype,
+                               void* stream) {
+  if (!ls || n_ls <= 0 || n < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: empty l list or negative n");
+  if (dtype != E3X_F32) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: only fp32 storage is implemented");
+  if (normalization < 0 || normalization > 2)
+    return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: normalization must be integral, component or norm");
+  for (int i = 0; i < n_ls; ++i)
+    if (ls[i] != i) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: the l list must be 0, 1, ..., lmax");
+  const int lmax = n_ls - 1;
+  if (lmax > 3) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: implemented for lmax <= 3");
+  if (n == 0) return E3X_OK;
+  if (!xyz || !grad_out || !grad_xyz) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: null pointer");
+  if (n >= (1LL << 31) * 256) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: too many vectors for one launch");
+  Scale4 sc;
+  for (int l = 0; l < 4; ++l) {
+    sc.s[l] = 1.0f;
+    if (normalization == E3X_NORM_INTEGRAL) sc.s[l] = (float)(1.0 / std::sqrt(4.0 * M_PI));
+    if (normalization == E3X_NORM_NORM) sc.s[l] = (float)(1.0 / std::sqrt(2.0 * l + 1.0));
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const float *px = (const float*)xyz, *pg = (const float*)grad_out;
+  float* po = (float*)grad_xyz;
+  switch (lmax) {
+    case 0: launch_bwd<0>(normalize, px, pg, po, n, sc, st); break;
+    case 1: launch_bwd<1>(normalize, px, pg, po, n, sc, st); break;
+    case 2: launch_bwd<2>(normalize, px, pg, po, n, sc, st); break;
+    default: launch_bwd<3>(normalize, px, pg, po, n, sc, st); break;
+  }
+  if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_sh_backward: kernel launch failed");
   return E3X_OK;
 }

@@ -34,11 +34,28 @@ class _SphericalHarmonicsFn(torch.autograd.Function):
                     _lib.F32, _lib.stream_ptr(x.device),
                 )  # fmt: skip
             )
+        ctx.save_for_backward(xyz)
+        ctx.cfg = (ls, normalize, normalization, batch)
         return out.reshape(batch + (n_out,))
 
     @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("the spherical-harmonics backward kernel is not implemented")
+    def backward(ctx, g):
+        (xyz,) = ctx.saved_tensors
+        ls, normalize, normalization, batch = ctx.cfg
+        if list(ls) != list(range(len(ls))) or len(ls) > 4:
+            raise NotImplementedError("the spherical-harmonics backward kernel covers l = 0..lmax with lmax <= 3")
+        n = xyz.shape[0]
+        g = g.reshape(n, -1).contiguous()
+        gx = torch.empty_like(xyz)
+        arr = (ctypes.c_int32 * len(ls))(*ls)
+        with torch.cuda.device(xyz.device):
+            _lib.check(
+                _lib.lib().e3x_sh_backward(
+                    arr, len(ls), int(bool(normalize)), _NORMALIZATION[normalization], _lib.ptr(xyz), _lib.ptr(g),
+                    _lib.ptr(gx), n, _lib.F32, _lib.stream_ptr(xyz.device),
+                )  # fmt: skip
+            )
+        return gx.reshape(batch + (3,)), None, None, None
 
 
 class SphericalHarmonics(torch.nn.Module):

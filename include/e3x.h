@@ -136,9 +136,15 @@ int e3x_tp_backward_w_x2(e3x_plan* plan, const void* x1, const void* x2, const v
 /* out[n, sum(2l+1 for l in ls)] = spherical harmonics of xyz[n, 3].  Replaces
  * SphericalHarmonics.forward (e3nn/o3/_spherical_harmonics.py:93-112) and the polynomial
  * chain _spherical_harmonics (:193-249 for l <= 3, recurrence of
- * _spherical_harmonics_generator.py:57-65 above).  max(ls) <= 8. */
+ * _spherical_harmonics_generator.py:57-65 above).  max(ls) <= 12. */
 int e3x_sh_forward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization, const void* xyz,
                    void* out, int64_t n, int32_t dtype, void* stream);
+
+/* grad_xyz[n, 3] from grad_out[n, (lmax+1)^2] for ls = 0..lmax, lmax <= 3: the backward pass of
+ * e3x_sh_forward (the reference differentiates the polynomial chain of
+ * e3nn/o3/_spherical_harmonics.py:93-112,193-249 by autograd). */
+int e3x_sh_backward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization, const void* xyz,
+                    const void* grad_out, void* grad_xyz, int64_t n, int32_t dtype, void* stream);
 
 /* Plain device copy dst[i] = src[i], n_bytes multiple of 16: the calibration kernel
  * for bandwidth counters (known traffic: n_bytes read + n_bytes written). */
