@@ -36,6 +36,7 @@ struct SubKernel {
   hipFunction_t fn_plain[kMaxDevices] = {nullptr};
   hipFunction_t fn_fused[kMaxDevices] = {nullptr};
   hipFunction_t fn_bwd_edge[kMaxDevices] = {nullptr};
+  hipFunction_t fn_dw[kMaxDevices] = {nullptr};
 };
 
 struct e3x_plan {
@@ -393,6 +394,10 @@ int load_functions(e3x_plan* P, int dev) {
       if (hipModuleGetFunction(&K->fn_bwd_edge[dev], mod, "e3x_uvu_bwd_edge") != hipSuccess)
         return fail(E3X_ERR_HIP, "kernel e3x_uvu_bwd_edge missing from " + K->hsaco);
     }
+    if (P->family == "uvw_small") {
+      if (hipModuleGetFunction(&K->fn_dw[dev], mod, "e3x_uvw_small_dw") != hipSuccess)
+        return fail(E3X_ERR_HIP, "kernel e3x_uvw_small_dw missing from " + K->hsaco);
+    }
     K->module[dev] = mod;
   }
   return E3X_OK;
@@ -637,5 +642,37 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
     if (err != hipSuccess)
       return fail(E3X_ERR_HIP, std::string("e3x_tp_backward_w_x2: launch failed: ") + hipGetErrorString(err));
   }
+  return E3X_OK;
+}
+
+extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2, const void* grad_out, void* grad_w,
+                                     int64_t Z, void* stream) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null plan");
+  if (P->family != "uvw_small")
+    return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: implemented for the uvw_small kernel family only, this plan is " + P->family);
+  if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: fp32 storage only");
+  if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: negative batch");
+  if (P->weight_numel == 0) return E3X_OK;
+  if (!grad_w) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  int dev, rc;
+  if ((rc = current_device(&dev))) return rc;
+  if (P->shared_weights && (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st))) return rc;
+  if (Z == 0) return E3X_OK;
+  if (!grad_out || (P->in1_dim && !x1) || (P->in2_dim && !x2)) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null pointer");
+  if ((rc = load_functions(P, dev))) return rc;
+  const long long wblocks = (P->weight_numel + 255) / 256;
+  // enough batch slices to fill the chip a few times over, at least 16 rows each
+  long long slices = (4096 + wblocks - 1) / wblocks;
+  if (slices > (Z + 15) / 16) slices = (Z + 15) / 16;
+  if (slices < 1) slices = 1;
+  if (slices > 65535) slices = 65535;
+  long long n_rows = Z, rows_per_slice = (Z + slices - 1) / slices;
+  slices = (Z + rows_per_slice - 1) / rows_per_slice;
+  void* args[] = {(void*)&x1, (void*)&x2, (void*)&grad_out, (void*)&grad_w, (void*)&n_rows, (void*)&rows_per_slice};
+  hipError_t err = hipModuleLaunchKernel(P->subs[0]->fn_dw[dev], (unsigned)wblocks, (unsigned)slices, 1, 256, 1, 1, 0, st,
+                                         args, nullptr);
+  if (err != hipSuccess)
+    return fail(E3X_ERR_HIP, std::string("e3x_tp_backward_w_uvw: launch failed: ") + hipGetErrorString(err));
   return E3X_OK;
 }

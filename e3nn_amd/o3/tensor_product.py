@@ -114,6 +114,18 @@ class _Plan:
             )
         return out
 
+    def backward_w_uvw(self, x1, x2, grad_out, shared_weights):
+        shape = (self.weight_numel,) if shared_weights else (x1.shape[0], self.weight_numel)
+        gw = torch.empty(shape, dtype=x1.dtype, device=x1.device)
+        with torch.cuda.device(x1.device):
+            _lib.check(
+                _lib.lib().e3x_tp_backward_w_uvw(
+                    self.handle, _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(grad_out), _lib.ptr(gw), x1.shape[0],
+                    _lib.stream_ptr(x1.device),
+                )
+            )
+        return gw
+
     def backward_w_x2(self, x1, x2, w, grad_out, src, dst, want_w, want_x2, num_edges):
         gw = torch.empty(num_edges, self.weight_numel, dtype=x1.dtype, device=x1.device) if want_w else None
         gx2 = torch.empty(num_edges, x2.shape[1], dtype=x1.dtype, device=x1.device) if want_x2 else None
@@ -172,10 +184,13 @@ class _TensorProductFn(torch.autograd.Function):
                 gw, g2 = tp._plan(x1.dtype).backward_w_x2(x1, x2, w, g, None, None, needw and tp.weight_numel > 0, need2, x1.shape[0])
         elif mode == "uvw":
             if needw and tp.weight_numel:
-                raise NotImplementedError(
-                    "the weight gradient of uvw tensor products has no kernel yet; call weight.requires_grad_(False) "
-                    "to differentiate with respect to the inputs only"
-                )
+                plan = tp._plan(x1.dtype)
+                if plan.family != "uvw_small" or x1.dtype != torch.float32:
+                    raise NotImplementedError(
+                        "the weight gradient of matrix-core / bf16 uvw tensor products has no kernel yet; call "
+                        "weight.requires_grad_(False) to differentiate with respect to the inputs only"
+                    )
+                gw = plan.backward_w_uvw(x1, x2, g, tp.shared_weights)
             if need1:
                 g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, _permuted_weights(tp, w, (2, 1, 0)))
             if need2:

@@ -133,6 +133,14 @@ int e3x_tp_backward_w_x2(e3x_plan* plan, const void* x1, const void* x2, const v
                          const void* src, const void* dst, int idx_bits, void* grad_w, void* grad_x2, int64_t E,
                          int64_t num_src_nodes, int64_t num_out_nodes, void* stream);
 
+/* Weight gradient of the `uvw` product: grad_w[weight_numel] (shared weights, summed over the batch with
+ * fp32 atomics, so the last bits depend on the order) or grad_w[Z, weight_numel] (per-sample weights), from
+ * x1[Z, in1_dim], x2[Z, in2_dim], grad_out[Z, out_dim].  The reference obtains it by autograd through
+ * einsum("uvw,ijk,zuvij->zwk") (e3nn/o3/_tensor_product/_codegen.py:148-165).  Implemented for plans of the
+ * "uvw_small" family in fp32 storage. */
+int e3x_tp_backward_w_uvw(e3x_plan* plan, const void* x1, const void* x2, const void* grad_out, void* grad_w,
+                          int64_t Z, void* stream);
+
 /* out[n, sum(2l+1 for l in ls)] = spherical harmonics of xyz[n, 3].  Replaces
  * SphericalHarmonics.forward (e3nn/o3/_spherical_harmonics.py:93-112) and the polynomial
  * chain _spherical_harmonics (:193-249 for l <= 3, recurrence of

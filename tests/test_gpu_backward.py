@@ -83,9 +83,37 @@ def test_uvw_input_gradients(maker, Z):
     assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
 
 
-def test_missing_backward_kernels_fail_loudly():
+@pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.cfg1, 4099),
+                                     (lambda: ks.golden_tp("fctp_per_sample_weights"), 5)])  # fmt: skip
+def test_uvw_weight_gradients(maker, Z):
+    tp = maker().to(DEV)
+    spec = oracle_spec(tp)
+    x1, x2 = seeded(Z, tp.irreps_in1.dim, seed=1), seeded(Z, tp.irreps_in2.dim, seed=2)
+    w = seeded(*((Z,) if not tp.shared_weights else ()), tp.weight_numel, seed=3) / 4
+    cot = seeded(Z, tp.irreps_out.dim, seed=4)
+    _, (r1, r2, rw) = _oracle_grads(lambda a, b, c: tp_forward_torch(spec, a, b, c), (x1, x2, w), cot)
+    a, b, c = (t.to(DEV).requires_grad_(True) for t in (x1, x2, w))
+    tp(a, b, c).backward(cot.to(DEV))
+    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
+    assert_close(c.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dw")
+    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dx1")
+    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
+    # the weights alone
+    c2 = w.to(DEV).requires_grad_(True)
+    tp(x1.to(DEV), x2.to(DEV), c2).backward(cot.to(DEV))
+    assert_close(c2.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dw alone")
+
+
+def test_internal_weights_train():
     tp = ks.cfg1().to(DEV)
-    x1, x2 = seeded(4, 64).to(DEV), seeded(4, 9).to(DEV)
+    x1, x2 = seeded(40, 64).to(DEV), seeded(40, 9).to(DEV)
+    tp(x1, x2).square().sum().backward()
+    assert tp.weight.grad is not None and tp.weight.grad.shape == tp.weight.shape and bool(tp.weight.grad.abs().sum() > 0)
+
+
+def test_missing_backward_kernels_fail_loudly():
+    tp = ks.mfma_small().to(DEV)
+    x1, x2 = seeded(4, tp.irreps_in1.dim).to(DEV), seeded(4, tp.irreps_in2.dim).to(DEV)
     out = tp(x1, x2)  # internal weights require a gradient
     with pytest.raises(NotImplementedError):
         out.sum().backward()
