@@ -10,6 +10,7 @@ extern const char* const kTplUvu;
 extern const char* const kTplUvwSmall;
 extern const char* const kTplUvwMfma;
 extern const char* const kTplUvwMfmaBf16;
+extern const char* const kTplUvwMfmaDw;
 
 std::string cache_dir();
 

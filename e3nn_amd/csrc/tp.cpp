@@ -2,7 +2,9 @@
 // tables that specialise the device templates, code-object loading and kernel launches.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <memory>
@@ -50,6 +52,10 @@ struct e3x_plan {
   int n_targets = 0;       // uvw_mfma: grid.y
   std::mutex mu;
   std::vector<std::unique_ptr<SubKernel>> subs;
+  // uvw_mfma: the weight-gradient kernel is a code object of its own, built on first use
+  std::unique_ptr<SubKernel> dw;
+  long long dw_tiles = 0;  // grid.x: the largest tile count of a path
+  int dw_paths = 0;        // grid.y
 };
 
 namespace {
@@ -377,6 +383,85 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   return E3X_OK;
 }
 
+// Tables of the matrix-core weight-gradient kernel: per path the M operand is the input with the smaller l.
+constexpr int kDwOuterBlock = 4;
+
+int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
+  std::ostringstream s, nzs, ps;
+  emit_header(s, P);
+  int n_nz = 0, n_path = 0, dkmax = 1, drmax = 1;
+  long long tiles = 0;
+  // the kernel reads 8 multiplicity indices of a row with 16-byte loads
+  for (const auto& p : P.paths)
+    if ((P.off1[p.in1] | P.off2[p.in2] | P.offo[p.out] | P.in1_dim | P.in2_dim | P.out_dim) & 3)
+      return fail(E3X_ERR_INVALID, "weight gradient on the matrix cores: irrep offsets and row lengths must be multiples of 4");
+  for (const auto& p : P.paths) {
+    const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2], &c = P.out[p.out];
+    const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1, d3 = 2 * c.l + 1;
+    const bool k_is_x2 = d2 < d1;
+    const auto& C = e3x::wigner_3j(a.l, b.l, c.l);
+    const int nz_beg = n_nz;
+    for (int i = 0; i < d1; ++i)
+      for (int j = 0; j < d2; ++j)
+        for (int k = 0; k < d3; ++k) {
+          const double cv = C[(i * d2 + j) * d3 + k] * p.pw;
+          if (cv != 0.0) {
+            nzs << "  {" << (k_is_x2 ? j : i) << ", " << (k_is_x2 ? i : j) << ", " << k << ", " << fstr(cv) << "},\n";
+            ++n_nz;
+          }
+        }
+    const long long W = c.mul;
+    const long long stride_u = (long long)b.mul * W, stride_v = W;  // W_p[u, v, w] at woff + (u * V + v) * W + w
+    const int dK = k_is_x2 ? d2 : d1, dR = k_is_x2 ? d1 : d2;
+    const int K = k_is_x2 ? b.mul : a.mul, O = k_is_x2 ? a.mul : b.mul;
+    dkmax = std::max(dkmax, dK);
+    drmax = std::max(drmax, dR);
+    ps << "  {" << (k_is_x2 ? "true" : "false") << ", " << (k_is_x2 ? P.off2[p.in2] : P.off1[p.in1]) << ", " << dK << ", "
+       << K << ", " << (k_is_x2 ? P.off1[p.in1] : P.off2[p.in2]) << ", " << dR << ", " << O << ", " << P.offo[p.out]
+       << ", " << d3 << ", " << W << ", " << p.woff << ", " << (k_is_x2 ? stride_v : stride_u) << ", "
+       << (k_is_x2 ? stride_u : stride_v) << ", " << nz_beg << ", " << n_nz << "},\n";
+    tiles = std::max(tiles, (long long)((K + 63) / 64) * (W / 64) * (O / kDwOuterBlock));
+    ++n_path;
+  }
+  s << "constexpr int WT = 64, OB = " << kDwOuterBlock << ", DKMAX = " << dkmax << ", DRMAX = " << drmax << ";\n";
+  s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
+    << nzs.str() << "};\n";
+  s << "struct DPath { bool k_is_x2; int koff, dK, K, roff, dR, O, goff, d3, W; long long wbase, wk_stride, wo_stride; "
+       "int nz_beg, nz_end; };\n";
+  s << "constexpr int N_DPATH = " << n_path << ";\nconstexpr DPath dpaths[N_DPATH] = {\n" << ps.str() << "};\n";
+  s << "}  // namespace cfg\n";
+  P.dw_tiles = tiles;
+  P.dw_paths = n_path;
+  *src = s.str() + e3x::kTplCommon + e3x::kTplUvwMfmaDw;
+  return E3X_OK;
+}
+
+// builds (or finds in the cache) the weight-gradient code object of a uvw_mfma plan
+int prepare_mfma_dw(e3x_plan* P) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  if (P->dw) return E3X_OK;
+  std::unique_ptr<SubKernel> K(new SubKernel);
+  std::string src;
+  int rc;
+  if ((rc = build_uvw_mfma_dw_source(*P, &src))) return rc;
+  if ((rc = e3x::get_code_object("uvw_mfma_dw", src, &K->key, &K->hsaco))) return rc;
+  P->dw = std::move(K);
+  return E3X_OK;
+}
+
+int load_dw_function(e3x_plan* P, int dev) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  SubKernel* K = P->dw.get();
+  if (K->module[dev]) return E3X_OK;
+  hipModule_t mod = nullptr;
+  hipError_t err = hipModuleLoad(&mod, K->hsaco.c_str());
+  if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + K->hsaco + ") failed: " + hipGetErrorString(err));
+  if (hipModuleGetFunction(&K->fn_dw[dev], mod, "e3x_uvw_mfma_dw") != hipSuccess)
+    return fail(E3X_ERR_HIP, "kernel e3x_uvw_mfma_dw missing from " + K->hsaco);
+  K->module[dev] = mod;
+  return E3X_OK;
+}
+
 int load_functions(e3x_plan* P, int dev) {
   std::lock_guard<std::mutex> lock(P->mu);
   for (auto& K : P->subs) {
@@ -645,11 +730,20 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
   return E3X_OK;
 }
 
+extern "C" int e3x_tp_plan_prepare_backward_w(e3x_plan* P) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: null plan");
+  if (P->family == "uvw_mfma") {
+    if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: fp32 storage only");
+    return prepare_mfma_dw(P);
+  }
+  return E3X_OK;  // the other families carry their gradient kernels in the forward code object
+}
+
 extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2, const void* grad_out, void* grad_w,
                                      int64_t Z, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null plan");
-  if (P->family != "uvw_small")
-    return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: implemented for the uvw_small kernel family only, this plan is " + P->family);
+  if (P->family != "uvw_small" && P->family != "uvw_mfma")
+    return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: the plan must be all-uvw");
   if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: fp32 storage only");
   if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: negative batch");
   if (P->weight_numel == 0) return E3X_OK;
@@ -657,9 +751,34 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   hipStream_t st = (hipStream_t)stream;
   int dev, rc;
   if ((rc = current_device(&dev))) return rc;
-  if (P->shared_weights && (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st))) return rc;
-  if (Z == 0) return E3X_OK;
+  const bool mfma = P->family == "uvw_mfma";
+  if (Z == 0) return P->shared_weights ? e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st) : E3X_OK;
   if (!grad_out || (P->in1_dim && !x1) || (P->in2_dim && !x2)) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null pointer");
+  long long n_rows = Z;
+  if (mfma) {
+    if (((uintptr_t)x1 | (uintptr_t)x2 | (uintptr_t)grad_out) & 15)
+      return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: x1, x2 and grad_out must be 16-byte aligned");
+    if ((rc = prepare_mfma_dw(P))) return rc;
+    if ((rc = load_dw_function(P, dev))) return rc;
+    // batch slices: enough workgroups for a few waves of the chip, at least 256 rows each
+    const long long wgs = P->dw_tiles * P->dw_paths;
+    long long slices = (2048 + wgs - 1) / wgs;
+    slices = std::min(slices, (long long)((Z + 255) / 256));
+    slices = std::max(1LL, std::min(slices, 1024LL));
+    long long rows_per_slice = (Z + slices - 1) / slices;
+    rows_per_slice = (rows_per_slice + 31) / 32 * 32;
+    slices = (Z + rows_per_slice - 1) / rows_per_slice;
+    int accumulate = slices > 1;
+    if (accumulate && (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st))) return rc;
+    void* args[] = {(void*)&x1, (void*)&x2, (void*)&grad_out, (void*)&grad_w, (void*)&n_rows, (void*)&rows_per_slice,
+                    (void*)&accumulate};
+    hipError_t err = hipModuleLaunchKernel(P->dw->fn_dw[dev], (unsigned)P->dw_tiles, (unsigned)P->dw_paths,
+                                           (unsigned)slices, 256, 1, 1, 0, st, args, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_backward_w_uvw: launch failed: ") + hipGetErrorString(err));
+    return E3X_OK;
+  }
+  if (P->shared_weights && (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st))) return rc;
   if ((rc = load_functions(P, dev))) return rc;
   const long long wblocks = (P->weight_numel + 255) / 256;
   // enough batch slices to fill the chip a few times over, at least 16 rows each
@@ -667,7 +786,7 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   if (slices > (Z + 15) / 16) slices = (Z + 15) / 16;
   if (slices < 1) slices = 1;
   if (slices > 65535) slices = 65535;
-  long long n_rows = Z, rows_per_slice = (Z + slices - 1) / slices;
+  long long rows_per_slice = (Z + slices - 1) / slices;
   slices = (Z + rows_per_slice - 1) / rows_per_slice;
   void* args[] = {(void*)&x1, (void*)&x2, (void*)&grad_out, (void*)&grad_w, (void*)&n_rows, (void*)&rows_per_slice};
   hipError_t err = hipModuleLaunchKernel(P->subs[0]->fn_dw[dev], (unsigned)wblocks, (unsigned)slices, 1, 256, 1, 1, 0, st,

@@ -117,6 +117,8 @@ class _Plan:
     def backward_w_uvw(self, x1, x2, grad_out, shared_weights):
         shape = (self.weight_numel,) if shared_weights else (x1.shape[0], self.weight_numel)
         gw = torch.empty(shape, dtype=x1.dtype, device=x1.device)
+        # the matrix-core kernel reads rows with 16-byte loads
+        x1, x2, grad_out = (t if t.data_ptr() % 16 == 0 else t.clone() for t in (x1, x2, grad_out))
         with torch.cuda.device(x1.device):
             _lib.check(
                 _lib.lib().e3x_tp_backward_w_uvw(
@@ -184,13 +186,12 @@ class _TensorProductFn(torch.autograd.Function):
                 gw, g2 = tp._plan(x1.dtype).backward_w_x2(x1, x2, w, g, None, None, needw and tp.weight_numel > 0, need2, x1.shape[0])
         elif mode == "uvw":
             if needw and tp.weight_numel:
-                plan = tp._plan(x1.dtype)
-                if plan.family != "uvw_small" or x1.dtype != torch.float32:
+                if x1.dtype != torch.float32:
                     raise NotImplementedError(
-                        "the weight gradient of matrix-core / bf16 uvw tensor products has no kernel yet; call "
+                        "the weight gradient of uvw tensor products has an fp32 kernel only; call "
                         "weight.requires_grad_(False) to differentiate with respect to the inputs only"
                     )
-                gw = plan.backward_w_uvw(x1, x2, g, tp.shared_weights)
+                gw = tp._plan(x1.dtype).backward_w_uvw(x1, x2, g, tp.shared_weights)
             if need1:
                 g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, _permuted_weights(tp, w, (2, 1, 0)))
             if need2:
@@ -413,6 +414,8 @@ class TensorProduct(torch.nn.Module):
         self._grad_plan("x1", dtype)
         if self._live_mode() == "uvw":
             self._grad_plan("x2", dtype)
+            if dtype == torch.float32 and self.weight_numel:
+                _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(self._plan(dtype).handle))
         return self
 
     def __getstate__(self):

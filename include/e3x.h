@@ -136,8 +136,11 @@ int e3x_tp_backward_w_x2(e3x_plan* plan, const void* x1, const void* x2, const v
 /* Weight gradient of the `uvw` product: grad_w[weight_numel] (shared weights, summed over the batch with
  * fp32 atomics, so the last bits depend on the order) or grad_w[Z, weight_numel] (per-sample weights), from
  * x1[Z, in1_dim], x2[Z, in2_dim], grad_out[Z, out_dim].  The reference obtains it by autograd through
- * einsum("uvw,ijk,zuvij->zwk") (e3nn/o3/_tensor_product/_codegen.py:148-165).  Implemented for plans of the
- * "uvw_small" family in fp32 storage. */
+ * einsum("uvw,ijk,zuvij->zwk") (e3nn/o3/_tensor_product/_codegen.py:148-165).  fp32 storage only.  Plans
+ * of the "uvw_mfma" family need x1, x2 and grad_out 16-byte aligned and build a second code object on first
+ * use; e3x_tp_plan_prepare_backward_w builds it ahead of time (no GPU needed), so that a later call finds
+ * it in the kernel cache. */
+int e3x_tp_plan_prepare_backward_w(e3x_plan* plan);
 int e3x_tp_backward_w_uvw(e3x_plan* plan, const void* x1, const void* x2, const void* grad_out, void* grad_w,
                           int64_t Z, void* stream);
 

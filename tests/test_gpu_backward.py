@@ -84,7 +84,8 @@ def test_uvw_input_gradients(maker, Z):
 
 
 @pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.cfg1, 4099),
-                                     (lambda: ks.golden_tp("fctp_per_sample_weights"), 5)])  # fmt: skip
+                                     (lambda: ks.golden_tp("fctp_per_sample_weights"), 5), (ks.mfma_small, 70),
+                                     (ks.mfma_small, 1500)])  # fmt: skip
 def test_uvw_weight_gradients(maker, Z):
     tp = maker().to(DEV)
     spec = oracle_spec(tp)
@@ -112,9 +113,12 @@ def test_internal_weights_train():
 
 
 def test_missing_backward_kernels_fail_loudly():
-    tp = ks.mfma_small().to(DEV)
+    # shared uvu weights have no gradient kernel: the call must raise, not fall back
+    tp = ks.golden_tp("uvu_shared_v2").to(DEV)
+    assert tp.shared_weights and tp.weight_numel
     x1, x2 = seeded(4, tp.irreps_in1.dim).to(DEV), seeded(4, tp.irreps_in2.dim).to(DEV)
-    out = tp(x1, x2)  # internal weights require a gradient
+    w = seeded(tp.weight_numel).to(DEV).requires_grad_(True)
+    out = tp(x1, x2, w)
     with pytest.raises(NotImplementedError):
         out.sum().backward()
 
