@@ -242,6 +242,53 @@ def bench_uvw(args, dev, dtype=torch.float32):
                          "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
 
 
+def bench_nequip_backward(args, dev, ctx):
+    """Forward + backward of the headline convolution: gradients with respect to node features, edge
+    attributes and per-edge weights, from a fixed cotangent."""
+    from e3nn_amd.nn import DstSortedEdges
+
+    tp = ctx["tp"]
+    edges = DstSortedEdges(ctx["src"], ctx["dst"], ctx["N"])
+    a, b, c = (ctx[k].clone().requires_grad_(True) for k in ("node_x", "attr", "w"))
+    cot = torch.randn(ctx["N"], tp.irreps_out.dim, device=dev)
+
+    def step():
+        a.grad = b.grad = c.grad = None
+        tp.forward_gather_scatter(a, b, c, edges=edges).backward(cot)
+
+    ms = event_time_ms(step, max(5, args.steps // 5), 2)
+    E = ctx["src"].shape[0]
+    return {"edges": E, "ms_forward_backward": ms, "edges_per_s": E / (ms * 1e-3)}
+
+
+def bench_uvw_backward(args, dev):
+    """Dense uvw (fp32), forward + backward with respect to both inputs and the shared weights, and the
+    weight-gradient kernel alone against the matrix-core peak."""
+    from tests import kernel_sets as ks
+
+    tp = ks.cfg5().to(dev)
+    Z = 65536
+    gen = torch.Generator().manual_seed(0)
+    with torch.no_grad():
+        tp.weight.copy_(torch.randn(tp.weight_numel, generator=gen) / 128.0)
+    x1 = torch.randn(Z, 1152, generator=gen).to(dev).requires_grad_(True)
+    x2 = torch.randn(Z, 1152, generator=gen).to(dev).requires_grad_(True)
+    cot = torch.randn(Z, 1152, generator=gen).to(dev)
+
+    def step():
+        x1.grad = x2.grad = tp.weight.grad = None
+        tp(x1, x2).backward(cot)
+
+    ms = event_time_ms(step, 2, 1)
+    plan = tp._plan(torch.float32)
+    a, b = x1.detach(), x2.detach()
+    ms_dw = event_time_ms(lambda: plan.backward_w_uvw(a, b, cot, True), 3, 1)
+    f_min = 2 * Z * 128**3 * 21
+    return {"rows": Z, "ms_forward_backward": ms, "ms_weight_gradient": ms_dw,
+            "roofline_weight_gradient": {"bound": "mfma", "achieved": f_min / (ms_dw * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
+                                         "unit": "TFLOP/s", "frac": f_min / (ms_dw * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}}  # fmt: skip
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -249,7 +296,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--locality-variants", action="store_true", help="also time the headline graph with sorted edges / Morton node ids")
-    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16,uvw,uvw_bf16 (default: all)")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16,uvw,uvw_bf16,nequip_bwd,uvw_bwd (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported (no collectives, no sharding)")
@@ -260,7 +307,7 @@ def main():
 
     neq, ctx = bench_nequip(args, dev)
     other = {"nequip_uvu": neq}
-    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_bf16", "uvw", "uvw_bf16"}
+    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_bf16", "uvw", "uvw_bf16", "nequip_bwd", "uvw_bwd"}
     if "copy" in want:
         other["copy_1GiB"] = bench_copy(args, dev)
     if "sh" in want:
@@ -273,6 +320,10 @@ def main():
         other["uvw_dense_fp32"] = bench_uvw(args, dev)
     if "uvw_bf16" in want:
         other["uvw_dense_bf16"] = bench_uvw(args, dev, torch.bfloat16)
+    if "nequip_bwd" in want:
+        other["nequip_uvu_forward_backward"] = bench_nequip_backward(args, dev, ctx)
+    if "uvw_bwd" in want:
+        other["uvw_dense_fp32_forward_backward"] = bench_uvw_backward(args, dev)
     line = {
         "metric": "per-edge uvu TP edges/sec (L=2, fused gather + tensor product + scatter)",
         "value": neq["edges_per_s"],
