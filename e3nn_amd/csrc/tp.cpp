@@ -39,6 +39,7 @@ struct SubKernel {
   hipFunction_t fn_fused[kMaxDevices] = {nullptr};
   hipFunction_t fn_bwd_edge[kMaxDevices] = {nullptr};
   hipFunction_t fn_dw[kMaxDevices] = {nullptr};
+  hipFunction_t fn_pack[kMaxDevices] = {nullptr};
 };
 
 struct e3x_plan {
@@ -310,6 +311,8 @@ bool uvw_mfma_eligible(const e3x_plan& P) {
   for (const auto& p : P.paths) {
     const int U = P.in1[p.in1].mul, V = P.in2[p.in2].mul, W = P.out[p.out].mul;
     if (U % 32 || V % 32 || W % 64 || U > 256 || V > 256 || P.out[p.out].l > 3) return false;
+    // the bf16 kernel reads 8 consecutive bf16 of a row with one 16-byte load
+    if (P.dtype == E3X_BF16 && ((P.off1[p.in1] | P.off2[p.in2] | P.in1_dim | P.in2_dim) & 7)) return false;
   }
   return true;
 }
@@ -358,7 +361,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
            << (k_is_x2 ? P.off2[p.in2] : P.off1[p.in1]) << ", "
            << (k_is_x2 ? d2 : d1) << ", " << (k_is_x2 ? b.mul : a.mul) << ", "
            << (k_is_x2 ? P.off1[p.in1] : P.off2[p.in2]) << ", " << (k_is_x2 ? d1 : d2) << ", "
-           << (k_is_x2 ? a.mul : b.mul) << ", " << p.woff << ", " << (k_is_x2 ? stride_v : stride_u) << ", "
+           << (k_is_x2 ? a.mul : b.mul) << ", " << W << ", " << p.woff << ", " << (k_is_x2 ? stride_v : stride_u) << ", "
            << (k_is_x2 ? stride_u : stride_v) << ", " << nz_beg << ", " << n_nz << "},\n";
       ++n_path;
     }
@@ -372,8 +375,8 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
     << nzs.str() << "};\n";
   s << "constexpr int DKA = " << dka << ";\n";
-  s << "struct MPath { bool synth, k_is_x2; int koff, dK, K, roff, dR, O; long long wbase, wk_stride, wo_stride; int nz_beg, "
-       "nz_end; };\n";
+  s << "struct MPath { bool synth, k_is_x2; int koff, dK, K, roff, dR, O, W; long long wbase, wk_stride, wo_stride; "
+       "int nz_beg, nz_end; };\n";
   s << "constexpr int N_MPATH = " << n_path << ";\nconstexpr MPath mpaths[N_MPATH] = {\n" << ps.str() << "};\n";
   s << "struct Target { int out_off, d3, w0, path_beg, path_end; };\n";
   s << "constexpr int N_TARGET = " << n_target << ";\nconstexpr Target targets[N_TARGET] = {\n" << ts.str() << "};\n";
@@ -478,6 +481,10 @@ int load_functions(e3x_plan* P, int dev) {
         return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused missing from " + K->hsaco);
       if (hipModuleGetFunction(&K->fn_bwd_edge[dev], mod, "e3x_uvu_bwd_edge") != hipSuccess)
         return fail(E3X_ERR_HIP, "kernel e3x_uvu_bwd_edge missing from " + K->hsaco);
+    }
+    if (P->family == "uvw_mfma" && P->dtype == E3X_BF16) {
+      if (hipModuleGetFunction(&K->fn_pack[dev], mod, "e3x_uvw_mfma_pack") != hipSuccess)
+        return fail(E3X_ERR_HIP, "kernel e3x_uvw_mfma_pack missing from " + K->hsaco);
     }
     if (P->family == "uvw_small") {
       if (hipModuleGetFunction(&K->fn_dw[dev], mod, "e3x_uvw_small_dw") != hipSuccess)
@@ -603,8 +610,19 @@ static int zero_output(e3x_plan* P, void* out, int64_t rows, hipStream_t st) {
   return e3x::fill_zero_bytes(out, bytes, st);
 }
 
+static bool needs_packed_weights(const e3x_plan* P) { return P->family == "uvw_mfma" && P->dtype == E3X_BF16; }
+
+extern "C" size_t e3x_tp_forward_workspace_bytes(const e3x_plan* P) {
+  return (P && needs_packed_weights(P)) ? (size_t)P->weight_numel * 2 : 0;
+}
+
 extern "C" int e3x_tp_forward(e3x_plan* P, const void* x1, const void* x2, const void* w, void* out, int64_t Z,
                               void* stream) {
+  return e3x_tp_forward_ws(P, x1, x2, w, out, Z, nullptr, 0, stream);
+}
+
+extern "C" int e3x_tp_forward_ws(e3x_plan* P, const void* x1, const void* x2, const void* w, void* out, int64_t Z,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_forward: null plan");
   if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_tp_forward: negative batch");
   if (Z == 0 || P->out_dim == 0) return E3X_OK;
@@ -619,6 +637,20 @@ extern "C" int e3x_tp_forward(e3x_plan* P, const void* x1, const void* x2, const
   }
   if ((rc = load_functions(P, dev))) return rc;
   long long n_rows = Z;
+  if (needs_packed_weights(P)) {
+    // the matrix-core kernel reads the weights repacked into octets of consecutive K indices
+    if (!workspace || workspace_bytes < (size_t)P->weight_numel * 2)
+      return fail(E3X_ERR_INVALID, "e3x_tp_forward: this plan needs e3x_tp_forward_ws with a workspace of "
+                                   "e3x_tp_forward_workspace_bytes(plan) bytes");
+    if (((uintptr_t)x1 | (uintptr_t)x2 | (uintptr_t)workspace) & 15)
+      return fail(E3X_ERR_INVALID, "e3x_tp_forward: x1, x2 and the workspace must be 16-byte aligned");
+    void* pargs[] = {(void*)&w, (void*)&workspace};
+    hipError_t err = hipModuleLaunchKernel(P->subs[0]->fn_pack[dev], (unsigned)(P->weight_numel / 8 / 256), 1, 1, 256, 1, 1,
+                                           0, st, pargs, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_forward: launch failed: ") + hipGetErrorString(err));
+    w = workspace;
+  }
   void* args[] = {(void*)&x1, (void*)&x2, (void*)&w, (void*)&out, (void*)&n_rows};
   for (auto& K : P->subs) {
     long long blocks;

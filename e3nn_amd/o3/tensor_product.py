@@ -93,10 +93,17 @@ class _Plan:
     def forward(self, x1, x2, w):
         Z = x1.shape[0]
         out = torch.empty(Z, self.out_dim, dtype=x1.dtype, device=x1.device)
+        ws_bytes = _lib.lib().e3x_tp_forward_workspace_bytes(self.handle)
+        ws = None
+        if ws_bytes:
+            # scratch for the weights repacked for the matrix cores; the kernel reads rows with 16-byte loads
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x1.device)
+            x1, x2 = (t if t.data_ptr() % 16 == 0 else t.clone() for t in (x1, x2))
         with torch.cuda.device(x1.device):
             _lib.check(
-                _lib.lib().e3x_tp_forward(
-                    self.handle, _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(w), _lib.ptr(out), Z, _lib.stream_ptr(x1.device)
+                _lib.lib().e3x_tp_forward_ws(
+                    self.handle, _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(w), _lib.ptr(out), Z,
+                    _lib.ptr(ws) if ws is not None else None, ws_bytes, _lib.stream_ptr(x1.device),
                 )
             )
         return out

@@ -94,6 +94,12 @@ int e3x_tp_plan_info(const e3x_plan* plan, int64_t* weight_numel, int64_t* in1_d
  * `out` is fully overwritten (output irreps no instruction reaches become 0). */
 int e3x_tp_forward(e3x_plan* plan, const void* x1, const void* x2, const void* w, void* out, int64_t Z,
                    void* stream);
+/* The same with caller-owned device scratch.  Plans of the "uvw_mfma" family in bf16 storage repack the
+ * weights for the matrix cores on every call and need e3x_tp_forward_workspace_bytes(plan) bytes (16-byte
+ * aligned, as x1 and x2 must be); every other plan needs none and e3x_tp_forward is enough. */
+size_t e3x_tp_forward_workspace_bytes(const e3x_plan* plan);
+int e3x_tp_forward_ws(e3x_plan* plan, const void* x1, const void* x2, const void* w, void* out, int64_t Z,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* Destination-sorted edge list for the fused scatter: stable sort of edge ids by dst.
  * rowptr[num_nodes+1], perm[E] are int32 device arrays owned by the caller;
