@@ -329,6 +329,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   emit_header(s, P);
   s << "constexpr int WT = " << wt << ", KMAX = " << kmax << ";\n";
   if (P.dtype == E3X_F32) s << "#define E3X_UVW_KC " << env_int("E3X_UVW_KC", 32) << "\n";
+  if (env_int("E3X_EXP", 0)) s << "#define E3X_EXP " << env_int("E3X_EXP", 0) << "\n";
   int n_nz = 0, n_path = 0, n_target = 0, dka = 1;
   for (size_t c = 0; c < P.out.size(); ++c) {
     std::ostringstream mine;
