@@ -242,6 +242,19 @@ def bench_uvw(args, dev, dtype=torch.float32):
                          "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
 
 
+def bench_library_gemm(args, dev):
+    """Context for the matrix-core rooflines: what the vendor GEMM (torch.matmul -> rocBLAS / hipBLASLt) reaches
+    on this GPU with N(0,1) data, 8192^3."""
+    out = {}
+    n = 8192
+    for name, dt in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+        a = torch.randn(n, n, device=dev).to(dt)
+        b = torch.randn(n, n, device=dev).to(dt)
+        ms = event_time_ms(lambda: a @ b, 5, 2)
+        out[name + "_tflops"] = 2 * n**3 / (ms * 1e-3) / 1e12
+    return out
+
+
 def bench_nequip_backward(args, dev, ctx):
     """Forward + backward of the headline convolution: gradients with respect to node features, edge
     attributes and per-edge weights, from a fixed cotangent."""
@@ -320,6 +333,8 @@ def main():
         other["uvw_dense_fp32"] = bench_uvw(args, dev)
     if "uvw_bf16" in want:
         other["uvw_dense_bf16"] = bench_uvw(args, dev, torch.bfloat16)
+    if "uvw" in want or "uvw_bf16" in want:
+        other["library_gemm_8192_randn"] = bench_library_gemm(args, dev)
     if "nequip_bwd" in want:
         other["nequip_uvu_forward_backward"] = bench_nequip_backward(args, dev, ctx)
     if "uvw_bwd" in want:

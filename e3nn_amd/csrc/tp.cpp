@@ -253,8 +253,6 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src) {
   bool prefetch = upl * (accregs + 2 * (x1regs + wregs)) + 2 * (int)P.in2_dim <= 96;
   prefetch = env_int("E3X_UVU_PREFETCH", prefetch ? 1 : 0) != 0;
   s << "constexpr bool PREFETCH = " << (prefetch ? "true" : "false") << ";\n";
-  if (env_int("E3X_EXPERIMENT_NO_MATH", 0)) s << "#define E3X_EXPERIMENT_NO_MATH 1\n";
-  if (env_int("E3X_NO_STREAM_HINT", 0)) s << "#define E3X_NO_STREAM_HINT 1\n";
   K.waves_per_block = env_int("E3X_UVU_WAVES_PER_BLOCK", 4);
   s << "#define E3X_WAVES_PER_BLOCK " << K.waves_per_block << "\n";
   s << "}  // namespace cfg\n";
@@ -329,8 +327,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   emit_header(s, P);
   s << "constexpr int WT = " << wt << ", KMAX = " << kmax << ";\n";
   if (P.dtype == E3X_F32) s << "#define E3X_UVW_KC " << env_int("E3X_UVW_KC", 32) << "\n";
-  if (env_int("E3X_EXP", 0)) s << "#define E3X_EXP " << env_int("E3X_EXP", 0) << "\n";
-  int n_nz = 0, n_path = 0, n_target = 0, dka = 1;
+  int n_nz = 0, n_path = 0, n_target = 0, dka = 1, drmax = 1;
   for (size_t c = 0; c < P.out.size(); ++c) {
     std::ostringstream mine;
     const int beg = n_path;
@@ -344,6 +341,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
       const bool synth = P.dtype == E3X_F32 && env_int("E3X_UVW_SYNTH", 1) && d3 < std::min(d1, d2);
       const bool k_is_x2 = !synth && d2 < d1;
       if (synth) dka = std::max(dka, d1);
+      drmax = std::max(drmax, k_is_x2 ? d1 : d2);
       const auto& C = e3x::wigner_3j(a.l, b.l, P.out[c].l);
       const int nz_beg = n_nz;
       for (int i = 0; i < d1; ++i)
@@ -375,7 +373,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   }
   s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
     << nzs.str() << "};\n";
-  s << "constexpr int DKA = " << dka << ";\n";
+  s << "constexpr int DKA = " << dka << ", DRMAX = " << drmax << ";\n";
   s << "struct MPath { bool synth, k_is_x2; int koff, dK, K, roff, dR, O, W; long long wbase, wk_stride, wo_stride; "
        "int nz_beg, nz_end; };\n";
   s << "constexpr int N_MPATH = " << n_path << ";\nconstexpr MPath mpaths[N_MPATH] = {\n" << ps.str() << "};\n";
@@ -574,7 +572,10 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
     std::unique_ptr<SubKernel> K(new SubKernel);
     K->path_ids = ids;
     std::string src;
-    if (P->family == "uvw_mfma") rc = build_uvw_mfma_source(*P, &src);
+    if (P->family == "uvw_mfma") {
+      rc = build_uvw_mfma_source(*P, &src);
+      K->waves_per_block = P->dtype == E3X_BF16 ? 8 : 4;
+    }
     else if (P->family == "uvw_small") rc = build_uvw_small_source(*P, *K, &src);
     else rc = build_uvu_source(*P, *K, &src);
     if (rc) return rc;
@@ -657,7 +658,8 @@ extern "C" int e3x_tp_forward_ws(e3x_plan* P, const void* x1, const void* x2, co
     long long blocks;
     unsigned grid_y = 1;
     if (P->family == "uvw_mfma") {
-      blocks = (Z + 63) / 64;
+      const int rows = 16 * K->waves_per_block;  // fp32: 4 waves, 64 rows; bf16: 8 waves, 128 rows
+      blocks = (Z + rows - 1) / rows;
       grid_y = (unsigned)P->n_targets;
     } else {
       const int groups = 64 / K->lanes;
@@ -704,7 +706,7 @@ extern "C" int e3x_tp_gather_scatter(e3x_plan* P, const void* node_x, const void
     blocks = (blocks + 7) / 8 * 8;  // the kernel deals contiguous eighths of the rows to the 8 XCDs
     if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
     hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1,
-                                           (unsigned)env_int("E3X_UVU_LDS_PAD", 0), st, args, nullptr);
+                                           0, st, args, nullptr);
     if (err != hipSuccess)
       return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
   }
