@@ -270,6 +270,9 @@ int build_uvw_small_source(e3x_plan& P, SubKernel& K, std::string* src) {
     max_mul = std::max(max_mul, P.out[p.out].mul);
   }
   K.lanes = max_mul > 32 ? 64 : pow2_at_least(max_mul, 16);
+  // long input rows: fewer rows per wavefront so that the staged rows fit in LDS (lanes beyond the output
+  // multiplicity idle)
+  while (K.lanes < 64 && (P.in1_dim + P.in2_dim) * 16 * (64 / K.lanes) > 65536) K.lanes *= 2;
   K.chunks = (max_mul + K.lanes - 1) / K.lanes;
   if ((P.in1_dim + P.in2_dim) * 16 * (64 / K.lanes) > 65536)
     return fail(E3X_ERR_INVALID, "uvw kernel: input rows too long for the LDS staging buffer");
@@ -308,9 +311,18 @@ bool uvw_mfma_eligible(const e3x_plan& P) {
   if (!P.shared_weights || P.paths.empty()) return false;
   for (const auto& p : P.paths) {
     const int U = P.in1[p.in1].mul, V = P.in2[p.in2].mul, W = P.out[p.out].mul;
-    if (U % 32 || V % 32 || W % 64 || U > 256 || V > 256 || P.out[p.out].l > 3) return false;
-    // the bf16 kernel reads 8 consecutive bf16 of a row with one 16-byte load
-    if (P.dtype == E3X_BF16 && ((P.off1[p.in1] | P.off2[p.in2] | P.in1_dim | P.in2_dim) & 7)) return false;
+    if (W % 64 || P.out[p.out].l > 3 || U < 1 || V < 1) return false;
+    const bool okU = U % 32 == 0 && U <= 256, okV = V % 32 == 0 && V <= 256;
+    if (P.dtype == E3X_BF16) {
+      // both multiplicities tile: the outer index runs in blocks of 8
+      if (!okU || !okV) return false;
+      // the bf16 kernel reads 8 consecutive bf16 of a row with one 16-byte load
+      if ((P.off1[p.in1] | P.off2[p.in2] | P.in1_dim | P.in2_dim) & 7) return false;
+    } else if (!okU && !okV) {
+      // fp32: one input's multiplicity is the GEMM K index (multiple of 32), the other's is a plain outer loop of
+      // any length -- e.g. node features x a few node attributes, or a linear map (second input "0e")
+      return false;
+    }
   }
   return true;
 }
@@ -319,13 +331,10 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   // 64 output channels per workgroup: 80 accumulator registers, two workgroups per CU (measured faster
   // than 128 channels at one workgroup per CU)
   int wt = env_int("E3X_UVW_WT", 64), kmax = 32;
-  for (const auto& p : P.paths) {
+  for (const auto& p : P.paths)
     if (P.out[p.out].mul % 128) wt = 64;
-    kmax = std::max(kmax, std::max(P.in1[p.in1].mul, P.in2[p.in2].mul));
-  }
   std::ostringstream s, nzs, ps, ts;
   emit_header(s, P);
-  s << "constexpr int WT = " << wt << ", KMAX = " << kmax << ";\n";
   if (P.dtype == E3X_F32) s << "#define E3X_UVW_KC " << env_int("E3X_UVW_KC", 32) << "\n";
   int n_nz = 0, n_path = 0, n_target = 0, dka = 1, drmax = 1;
   for (size_t c = 0; c < P.out.size(); ++c) {
@@ -338,8 +347,10 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
       // GEMM passes per outer index: 2l+1 of the K operand when accumulators are scaled, 2 l3 + 1 when the
       // operand is synthesised; take the cheapest
       // (the bf16 kernel scales accumulators only: its matrix passes are cheap next to the fp32 epilogue)
-      const bool synth = P.dtype == E3X_F32 && env_int("E3X_UVW_SYNTH", 1) && d3 < std::min(d1, d2);
-      const bool k_is_x2 = !synth && d2 < d1;
+      const bool okU = a.mul % 32 == 0 && a.mul <= 256, okV = b.mul % 32 == 0 && b.mul <= 256;
+      const bool synth = P.dtype == E3X_F32 && env_int("E3X_UVW_SYNTH", 1) && d3 < std::min(d1, d2) && okU;
+      const bool k_is_x2 = !synth && okV && (!okU || d2 < d1);
+      kmax = std::max(kmax, k_is_x2 ? b.mul : a.mul);
       if (synth) dka = std::max(dka, d1);
       drmax = std::max(drmax, k_is_x2 ? d1 : d2);
       const auto& C = e3x::wigner_3j(a.l, b.l, P.out[c].l);
@@ -371,6 +382,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
       ++n_target;
     }
   }
+  s << "constexpr int WT = " << wt << ", KMAX = " << kmax << ";\n";  // KMAX: the largest GEMM K extent
   s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
     << nzs.str() << "};\n";
   s << "constexpr int DKA = " << dka << ", DRMAX = " << drmax << ";\n";
@@ -386,21 +398,27 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
 }
 
 // Tables of the matrix-core weight-gradient kernel: per path the M operand is the input with the smaller l.
-constexpr int kDwOuterBlock = 4;
 
 int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
   std::ostringstream s, nzs, ps;
   emit_header(s, P);
   int n_nz = 0, n_path = 0, dkmax = 1, drmax = 1;
   long long tiles = 0;
-  // the kernel reads 8 multiplicity indices of a row with 16-byte loads
-  for (const auto& p : P.paths)
-    if ((P.off1[p.in1] | P.off2[p.in2] | P.offo[p.out] | P.in1_dim | P.in2_dim | P.out_dim) & 3)
+  // the kernel reads 8 multiplicity indices of the M operand and of the output gradient with 16-byte loads
+  for (const auto& p : P.paths) {
+    const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2];
+    const bool okU = a.mul % 32 == 0 && a.mul <= 256, okV = b.mul % 32 == 0 && b.mul <= 256;
+    const bool m_is_x2 = okV && (!okU || b.l < a.l);
+    const int moff = m_is_x2 ? P.off2[p.in2] : P.off1[p.in1];
+    const int64_t mdim = m_is_x2 ? P.in2_dim : P.in1_dim;
+    if ((moff | P.offo[p.out] | mdim | P.out_dim) & 3)
       return fail(E3X_ERR_INVALID, "weight gradient on the matrix cores: irrep offsets and row lengths must be multiples of 4");
+  }
   for (const auto& p : P.paths) {
     const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2], &c = P.out[p.out];
     const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1, d3 = 2 * c.l + 1;
-    const bool k_is_x2 = d2 < d1;
+    const bool okU = a.mul % 32 == 0 && a.mul <= 256, okV = b.mul % 32 == 0 && b.mul <= 256;
+    const bool k_is_x2 = okV && (!okU || d2 < d1);  // the M operand tiles by 32
     const auto& C = e3x::wigner_3j(a.l, b.l, c.l);
     const int nz_beg = n_nz;
     for (int i = 0; i < d1; ++i)
@@ -418,17 +436,18 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
     const int K = k_is_x2 ? b.mul : a.mul, O = k_is_x2 ? a.mul : b.mul;
     dkmax = std::max(dkmax, dK);
     drmax = std::max(drmax, dR);
+    const int ob = O % 4 == 0 ? 4 : (O % 2 == 0 ? 2 : 1);  // outer indices per workgroup
     ps << "  {" << (k_is_x2 ? "true" : "false") << ", " << (k_is_x2 ? P.off2[p.in2] : P.off1[p.in1]) << ", " << dK << ", "
-       << K << ", " << (k_is_x2 ? P.off1[p.in1] : P.off2[p.in2]) << ", " << dR << ", " << O << ", " << P.offo[p.out]
+       << K << ", " << (k_is_x2 ? P.off1[p.in1] : P.off2[p.in2]) << ", " << dR << ", " << O << ", " << ob << ", " << P.offo[p.out]
        << ", " << d3 << ", " << W << ", " << p.woff << ", " << (k_is_x2 ? stride_v : stride_u) << ", "
        << (k_is_x2 ? stride_u : stride_v) << ", " << nz_beg << ", " << n_nz << "},\n";
-    tiles = std::max(tiles, (long long)((K + 63) / 64) * (W / 64) * (O / kDwOuterBlock));
+    tiles = std::max(tiles, (long long)((K + 63) / 64) * (W / 64) * (O / ob));
     ++n_path;
   }
-  s << "constexpr int WT = 64, OB = " << kDwOuterBlock << ", DKMAX = " << dkmax << ", DRMAX = " << drmax << ";\n";
+  s << "constexpr int WT = 64, OBMAX = 4, DKMAX = " << dkmax << ", DRMAX = " << drmax << ";\n";
   s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
     << nzs.str() << "};\n";
-  s << "struct DPath { bool k_is_x2; int koff, dK, K, roff, dR, O, goff, d3, W; long long wbase, wk_stride, wo_stride; "
+  s << "struct DPath { bool k_is_x2; int koff, dK, K, roff, dR, O, OB, goff, d3, W; long long wbase, wk_stride, wo_stride; "
        "int nz_beg, nz_end; };\n";
   s << "constexpr int N_DPATH = " << n_path << ";\nconstexpr DPath dpaths[N_DPATH] = {\n" << ps.str() << "};\n";
   s << "}  // namespace cfg\n";
