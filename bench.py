@@ -198,13 +198,14 @@ def bench_sh(args, dev):
             "roofline_frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "bytes_per_launch": b}  # fmt: skip
 
 
-def bench_mace(args, dev, dtype=torch.float32):
+def bench_mace(args, dev, dtype=torch.float32, variant="A"):
+    """MACE-style uvu (L=3): variant A keeps 0e,1o,2e,3o outputs (23 paths), B every l <= 3 of either parity (34)."""
     from e3nn_amd.nn import DstSortedEdges
     from tests import kernel_sets as ks
 
     N, E = 20_000, 500_000
     gen = torch.Generator().manual_seed(0)
-    tp = ks.cfg4("A")
+    tp = ks.cfg4(variant)
     src = torch.randint(0, N, (E,), generator=gen, dtype=torch.int32).to(dev)
     dst = torch.randint(0, N, (E,), generator=gen, dtype=torch.int32).to(dev)
     node_x = torch.randn(N, tp.irreps_in1.dim, generator=gen).to(dev).to(dtype)
@@ -240,6 +241,35 @@ def bench_uvw(args, dev, dtype=torch.float32):
     return {"rows": Z, "ms": ms, "tflops_fmin": f_min / (ms * 1e-3) / 1e12, "tflops_fgemm_equiv": f_gemm / (ms * 1e-3) / 1e12,
             "roofline": {"bound": "mfma", "achieved": f_min / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
                          "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
+
+
+def bench_nequip_cube40(args, dev):
+    """The headline configuration as literally stated: 50 000 nodes in a 40 A cube, 5 A cutoff (degree ~354)."""
+    from e3nn_amd import o3
+    from e3nn_amd.nn import DstSortedEdges
+    from tests import kernel_sets as ks
+
+    N, side, cutoff = 50_000, 40.0, 5.0
+    pos, src, dst = radius_graph(N, side, cutoff)
+    E = src.shape[0]
+    gen = torch.Generator().manual_seed(0)
+    tp = ks.cfg3(merged=True)
+    node_x = torch.randn(N, tp.irreps_in1.dim, generator=gen).to(dev)
+    pos_t = torch.from_numpy(pos).float().to(dev)
+    src_t, dst_t = torch.from_numpy(src).to(dev), torch.from_numpy(dst).to(dev)
+    vec = pos_t[src_t] - pos_t[dst_t]
+    attr = o3.spherical_harmonics([0, 1, 2], vec, True, "component")
+    r = vec.norm(dim=1)
+    del vec, pos_t
+    w = torch.empty(E, tp.weight_numel, device=dev)
+    step = 2_000_000  # radial MLP in slices: its hidden activations are not kept
+    for a in range(0, E, step):
+        w[a : a + step] = radial_weights(r[a : a + step], cutoff, tp.weight_numel, torch.Generator().manual_seed(0), dev)
+    edges = DstSortedEdges(src_t, dst_t, N)
+    ms = event_time_ms(lambda: tp.forward_gather_scatter(node_x, attr, w, edges=edges), max(5, args.steps // 5), 2)
+    b = E * (4 * tp.weight_numel + 4 * 9 + 2 * 8) + N * 4 * (tp.irreps_in1.dim + tp.irreps_out.dim)
+    return {"edges": E, "nodes": N, "ms": ms, "edges_per_s": E / (ms * 1e-3), "achieved_gbs": b / (ms * 1e-3) / 1e9,
+            "roofline_frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "bytes_per_launch": b}  # fmt: skip
 
 
 def bench_library_gemm(args, dev):
@@ -309,7 +339,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--locality-variants", action="store_true", help="also time the headline graph with sorted edges / Morton node ids")
-    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_bf16,uvw,uvw_bf16,nequip_bwd,uvw_bwd (default: all)")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_b,mace_bf16,nequip40,uvw,uvw_bf16,nequip_bwd,uvw_bwd (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported (no collectives, no sharding)")
@@ -320,13 +350,17 @@ def main():
 
     neq, ctx = bench_nequip(args, dev)
     other = {"nequip_uvu": neq}
-    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_bf16", "uvw", "uvw_bf16", "nequip_bwd", "uvw_bwd"}
+    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_b", "mace_bf16", "nequip40", "uvw", "uvw_bf16", "nequip_bwd", "uvw_bwd"}
     if "copy" in want:
         other["copy_1GiB"] = bench_copy(args, dev)
     if "sh" in want:
         other["sh_lmax3_4M"] = bench_sh(args, dev)
     if "mace" in want:
         other["mace_uvu_fp32"] = bench_mace(args, dev)
+    if "mace_b" in want:
+        other["mace_uvu_fp32_variant_b"] = bench_mace(args, dev, variant="B")
+    if "nequip40" in want:
+        other["nequip_uvu_cube40"] = bench_nequip_cube40(args, dev)
     if "mace_bf16" in want:
         other["mace_uvu_bf16_storage"] = bench_mace(args, dev, torch.bfloat16)
     if "uvw" in want:
