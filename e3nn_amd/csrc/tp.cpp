@@ -311,7 +311,8 @@ bool uvw_mfma_eligible(const e3x_plan& P) {
   if (!P.shared_weights || P.paths.empty()) return false;
   for (const auto& p : P.paths) {
     const int U = P.in1[p.in1].mul, V = P.in2[p.in2].mul, W = P.out[p.out].mul;
-    if (W % 64 || P.out[p.out].l > 3 || U < 1 || V < 1) return false;
+    // fp32: 32-channel granularity (a half-filled last tile); bf16: whole 64-channel tiles
+    if (W % (P.dtype == E3X_BF16 ? 64 : 32) || P.out[p.out].l > 3 || U < 1 || V < 1) return false;
     const bool okU = U % 32 == 0 && U <= 256, okV = V % 32 == 0 && V <= 256;
     if (P.dtype == E3X_BF16) {
       // both multiplicities tile: the outer index runs in blocks of 8
@@ -378,7 +379,8 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
     if (n_path == beg) continue;
     ps << mine.str();
     for (int w0 = 0; w0 < P.out[c].mul; w0 += wt) {
-      ts << "  {" << P.offo[c] << ", " << 2 * P.out[c].l + 1 << ", " << w0 << ", " << beg << ", " << n_path << "},\n";
+      ts << "  {" << P.offo[c] << ", " << 2 * P.out[c].l + 1 << ", " << w0 << ", " << std::min(wt, P.out[c].mul - w0) << ", "
+         << beg << ", " << n_path << "},\n";
       ++n_target;
     }
   }
@@ -389,7 +391,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   s << "struct MPath { bool synth, k_is_x2; int koff, dK, K, roff, dR, O, W; long long wbase, wk_stride, wo_stride; "
        "int nz_beg, nz_end; };\n";
   s << "constexpr int N_MPATH = " << n_path << ";\nconstexpr MPath mpaths[N_MPATH] = {\n" << ps.str() << "};\n";
-  s << "struct Target { int out_off, d3, w0, path_beg, path_end; };\n";
+  s << "struct Target { int out_off, d3, w0, wn, path_beg, path_end; };\n";  // wn: channels in the tile (64, or 32 at the end)
   s << "constexpr int N_TARGET = " << n_target << ";\nconstexpr Target targets[N_TARGET] = {\n" << ts.str() << "};\n";
   s << "}  // namespace cfg\n";
   P.n_targets = n_target;
@@ -441,7 +443,7 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
        << K << ", " << (k_is_x2 ? P.off1[p.in1] : P.off2[p.in2]) << ", " << dR << ", " << O << ", " << ob << ", " << P.offo[p.out]
        << ", " << d3 << ", " << W << ", " << p.woff << ", " << (k_is_x2 ? stride_v : stride_u) << ", "
        << (k_is_x2 ? stride_u : stride_v) << ", " << nz_beg << ", " << n_nz << "},\n";
-    tiles = std::max(tiles, (long long)((K + 63) / 64) * (W / 64) * (O / ob));
+    tiles = std::max(tiles, (long long)((K + 63) / 64) * ((W + 63) / 64) * (O / ob));
     ++n_path;
   }
   s << "constexpr int WT = 64, OBMAX = 4, DKMAX = " << dkmax << ", DRMAX = " << drmax << ";\n";

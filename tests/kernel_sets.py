@@ -77,7 +77,13 @@ def node_fctp():
     # node-wise step of a convolution: features x a few scalar node attributes (one-hot species), the GEMM K index is
     # the feature multiplicity and the attribute index is a short outer loop (reference
     # e3nn/nn/models/v2106/points_convolution.py:56-58)
-    return o3.FullyConnectedTensorProduct("128x0e+64x1o+32x2e", "4x0e", "128x0e+64x1o+64x2e")
+    return o3.FullyConnectedTensorProduct("128x0e+64x1o+32x2e", "4x0e", "128x0e+64x1o+96x2e")
+
+
+def radial_layer():
+    # one dense layer of a radial network written as a tensor product of scalars: 64 -> 352 (= 5.5 tiles of 64
+    # channels: the last tile is half full), second input "0e"
+    return o3.FullyConnectedTensorProduct("64x0e", "0e", "352x0e")
 
 
 def scalar_exact():
@@ -103,6 +109,7 @@ def all_tensor_products():
         ("cfg5", cfg5(), (torch.float32, torch.bfloat16)),
         ("mfma_small", mfma_small(), (torch.float32,)),
         ("node_fctp", node_fctp(), (torch.float32,)),
+        ("radial_layer", radial_layer(), (torch.float32,)),
         ("scalar_exact", scalar_exact(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),
     ]
@@ -111,7 +118,7 @@ def all_tensor_products():
 
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
-                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "odd_mul"]  # fmt: skip
+                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "radial_layer", "odd_mul"]  # fmt: skip
 
 
 def prebuild(verbose=True):
