@@ -1,0 +1,75 @@
+"""Equivariant point convolution of the reference's ``v2106`` model family
+(``e3nn/nn/models/v2106/points_convolution.py:19-113``), every step on the HIP kernels of this package:
+
+    self-connection, lin1, lin2, alpha   FullyConnectedTensorProduct(features, node_attr)   uvw kernels
+    radial network                        FullyConnectedNet(edge_scalars)                     uvw + gate kernels
+    message                               scatter(tp(x[src], edge_attr, w), dst)              fused uvu kernel
+
+``node_features[edge_src]`` and the per-edge messages are never materialised.
+"""
+import torch
+
+from ..o3.irreps import Irrep, Irreps
+from ..o3.tensor_product import FullyConnectedTensorProduct, TensorProduct
+from .edges import DstSortedEdges
+from .fc import FullyConnectedNet
+
+
+class Convolution(torch.nn.Module):
+    r"""Same constructor and ``forward`` arguments as the reference; ``forward`` also accepts a prebuilt
+    ``edges=DstSortedEdges(...)`` so that the destination sort is paid once per graph instead of once per layer."""
+
+    def __init__(
+        self, irreps_node_input, irreps_node_attr, irreps_edge_attr, irreps_node_output, fc_neurons, num_neighbors
+    ) -> None:
+        super().__init__()
+        self.irreps_node_input = Irreps(irreps_node_input)
+        self.irreps_node_attr = Irreps(irreps_node_attr)
+        self.irreps_edge_attr = Irreps(irreps_edge_attr)
+        self.irreps_node_output = Irreps(irreps_node_output)
+        self.num_neighbors = num_neighbors
+
+        self.sc = FullyConnectedTensorProduct(self.irreps_node_input, self.irreps_node_attr, self.irreps_node_output)
+        self.lin1 = FullyConnectedTensorProduct(self.irreps_node_input, self.irreps_node_attr, self.irreps_node_input)
+
+        irreps_mid, instructions = [], []
+        for i, (mul, ir_in) in enumerate(self.irreps_node_input):
+            for j, (_, ir_edge) in enumerate(self.irreps_edge_attr):
+                for ir_out in ir_in * ir_edge:
+                    if ir_out in self.irreps_node_output or ir_out == Irrep(0, 1):
+                        k = len(irreps_mid)
+                        irreps_mid.append((mul, ir_out))
+                        instructions.append((i, j, k, "uvu", True))
+        irreps_mid = Irreps(irreps_mid)
+        irreps_mid, p, _ = irreps_mid.sort()
+        assert irreps_mid.dim > 0, (
+            f"irreps_node_input={self.irreps_node_input} time irreps_edge_attr={self.irreps_edge_attr} produces nothing "
+            f"in irreps_node_output={self.irreps_node_output}"
+        )
+        instructions = [(i_1, i_2, p[i_out], mode, train) for i_1, i_2, i_out, mode, train in instructions]
+        tp = TensorProduct(
+            self.irreps_node_input, self.irreps_edge_attr, irreps_mid, instructions, internal_weights=False, shared_weights=False
+        )
+        self.fc = FullyConnectedNet(list(fc_neurons) + [tp.weight_numel], torch.nn.functional.silu)
+        self.tp = tp
+        self.lin2 = FullyConnectedTensorProduct(irreps_mid, self.irreps_node_attr, self.irreps_node_output)
+        self.alpha = FullyConnectedTensorProduct(irreps_mid, self.irreps_node_attr, "0e")
+        with torch.no_grad():
+            self.alpha.weight.zero_()
+        assert (
+            self.alpha.output_mask[0] == 1.0
+        ), f"irreps_mid={irreps_mid} and irreps_node_attr={self.irreps_node_attr} are not able to generate scalars"
+
+    def forward(self, node_input, node_attr, edge_src, edge_dst, edge_attr, edge_scalars, edges=None) -> torch.Tensor:
+        weight = self.fc(edge_scalars)
+        node_self_connection = self.sc(node_input, node_attr)
+        node_features = self.lin1(node_input, node_attr)
+        if edges is None:
+            edges = DstSortedEdges(edge_src, edge_dst, node_input.shape[0])
+        node_features = self.tp.forward_gather_scatter(node_features, edge_attr, weight, edges=edges)
+        node_features = node_features.div(self.num_neighbors**0.5)
+        node_conv_out = self.lin2(node_features, node_attr)
+        alpha = self.alpha(node_features, node_attr)
+        m = self.sc.output_mask
+        alpha = (1 - m) + alpha * m
+        return node_self_connection + alpha * node_conv_out

@@ -1,0 +1,146 @@
+"""``o3.Linear``: the equivariant linear map of the reference (``e3nn/o3/_linear.py:27-260``), run as a ``uvw`` tensor
+product with a constant ``0e`` second input.
+
+For a path ``i_in -> i_out`` the reference computes ``alpha^(-1/2) * einsum("uw,zui->zwi", W, x)`` with ``alpha`` the
+fan-in (``_linear.py:152-165``).  The tensor product ``x (x) 1`` with instruction ``(i_in, 0, i_out, "uvw")`` has the
+Clebsch-Gordan tensor ``delta / sqrt(2l+1)`` and, under component normalisation, the path weight
+``sqrt((2l+1) / fan_in)``: the same map, with the same ``[mul_in, mul_out]`` weight blocks in the same order.  So the
+matrix-core ``uvw`` kernels (forward, input gradient, weight gradient) serve linear layers unchanged.
+"""
+from typing import List, NamedTuple, Optional, Tuple, Union
+
+import torch
+
+from .irreps import Irreps
+from .tensor_product import TensorProduct
+
+
+class Instruction(NamedTuple):
+    i_in: int
+    i_out: int
+    path_shape: tuple
+    path_weight: float
+
+
+class Linear(torch.nn.Module):
+    r"""Linear operation equivariant to :math:`O(3)`; same arguments as the reference's ``o3.Linear`` except ``f_in`` /
+    ``f_out`` (not implemented)."""
+
+    def __init__(
+        self,
+        irreps_in,
+        irreps_out,
+        *,
+        f_in: Optional[int] = None,
+        f_out: Optional[int] = None,
+        internal_weights: Optional[bool] = None,
+        shared_weights: Optional[bool] = None,
+        instructions: Optional[List[Tuple[int, int]]] = None,
+        biases: Union[bool, List[bool]] = False,
+        path_normalization: str = "element",
+        _optimize_einsums: Optional[bool] = None,
+    ) -> None:
+        super().__init__()
+        assert path_normalization in ["element", "path"]
+        if f_in is not None or f_out is not None:
+            raise NotImplementedError("Linear: f_in / f_out have no kernel")
+        irreps_in, irreps_out = Irreps(irreps_in), Irreps(irreps_out)
+        if instructions is None:
+            instructions = [
+                (i_in, i_out)
+                for i_in, (_, ir_in) in enumerate(irreps_in)
+                for i_out, (_, ir_out) in enumerate(irreps_out)
+                if ir_in == ir_out
+            ]
+        for i_in, i_out in instructions:
+            if not i_in < len(irreps_in):
+                raise IndexError(f"{i_in} is not a valid index for irreps_in")
+            if not i_out < len(irreps_out):
+                raise IndexError(f"{i_out} is not a valid index for irreps_out")
+            if irreps_in[i_in].ir != irreps_out[i_out].ir:
+                raise ValueError(f"{i_in} and {i_out} do not have the same irrep")
+
+        def alpha(i_in, i_out) -> float:
+            x = sum(irreps_in[a if path_normalization == "element" else i_in].mul for a, b in instructions if b == i_out)
+            return 1.0 if x == 0 else x
+
+        self.instructions = [
+            Instruction(i_in, i_out, (irreps_in[i_in].mul, irreps_out[i_out].mul), alpha(i_in, i_out) ** (-0.5))
+            for i_in, i_out in instructions
+        ]
+        if biases is None:
+            biases = len(irreps_out) * (False,)
+        if isinstance(biases, bool):
+            biases = [biases and ir.is_scalar() for _, ir in irreps_out]
+        assert len(biases) == len(irreps_out)
+        assert all(ir.is_scalar() or (not b) for b, (_, ir) in zip(biases, irreps_out))
+        self._bias_slices = [sl for b, sl in zip(biases, irreps_out.slices()) if b]
+        self.instructions += [
+            Instruction(-1, i_out, (mul_ir.dim,), 1.0) for i_out, (b, mul_ir) in enumerate(zip(biases, irreps_out)) if b
+        ]
+
+        if shared_weights is False and internal_weights is None:
+            internal_weights = False
+        if shared_weights is None:
+            shared_weights = True
+        if internal_weights is None:
+            internal_weights = True
+        assert shared_weights or not internal_weights
+        self.internal_weights, self.shared_weights = internal_weights, shared_weights
+        self.irreps_in, self.irreps_out = irreps_in, irreps_out
+
+        # the same map as a tensor product with "0e": the reference's own normalisation formula for TensorProduct
+        # (component / element or path) reproduces alpha^(-1/2) once the delta / sqrt(2l+1) of the 3j tensor is counted
+        self._tp = TensorProduct(
+            irreps_in, "0e", irreps_out, [(i, 0, o, "uvw", True) for i, o in instructions],
+            path_normalization=path_normalization, internal_weights=False, shared_weights=shared_weights,
+        )  # fmt: skip
+        self.weight_numel = self._tp.weight_numel
+        self.bias_numel = sum(sl.stop - sl.start for sl in self._bias_slices)
+        if internal_weights and self.weight_numel > 0:
+            self.weight = torch.nn.Parameter(torch.randn(self.weight_numel))
+        else:
+            self.register_buffer("weight", torch.Tensor())
+        if internal_weights and self.bias_numel > 0:
+            self.bias = torch.nn.Parameter(torch.zeros(self.bias_numel))
+        else:
+            self.register_buffer("bias", torch.Tensor())
+        self.register_buffer("output_mask", self._tp.output_mask.clone())
+
+    def __repr__(self) -> str:
+        return f"{self.__class__.__name__}({self.irreps_in} -> {self.irreps_out} | {self.weight_numel} weights)"
+
+    def forward(self, features, weight: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None):
+        if weight is None:
+            if self.weight_numel > 0 and not self.internal_weights:
+                raise RuntimeError("Weights must be provided when internal_weights = False")
+            weight = self.weight
+        if bias is None:
+            if self.bias_numel > 0 and not self.internal_weights:
+                raise RuntimeError("Biases must be provided when internal_weights = False")
+            bias = self.bias
+        ones = features.new_ones(features.shape[:-1] + (1,))
+        out = self._tp(features, ones, weight)
+        if self.bias_numel > 0:
+            off = 0
+            out = out.clone()
+            for sl in self._bias_slices:
+                n = sl.stop - sl.start
+                out[..., sl] += bias[..., off : off + n]
+                off += n
+        return out
+
+    def weight_view_for_instruction(self, instruction: int, weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+        weight = self.weight if weight is None else weight
+        ins = self.instructions[instruction]
+        if ins.i_in == -1:
+            raise ValueError(f"Instruction {instruction} is a bias")
+        off = sum(i.path_shape[0] * i.path_shape[1] for i in self.instructions[:instruction] if i.i_in != -1)
+        n = ins.path_shape[0] * ins.path_shape[1]
+        return weight.narrow(-1, off, n).view(weight.shape[:-1] + ins.path_shape)
+
+    def weight_views(self, weight: Optional[torch.Tensor] = None, yield_instruction: bool = False):
+        for i, ins in enumerate(self.instructions):
+            if ins.i_in != -1:
+                v = self.weight_view_for_instruction(i, weight)
+                yield (i, ins, v) if yield_instruction else v

@@ -21,7 +21,6 @@ from typing import List, Optional, Union
 import torch
 
 from .. import _lib, get_optimization_defaults
-from ..nn.edges import DstSortedEdges
 from .irreps import Irreps
 
 Instruction = namedtuple(
@@ -534,7 +533,7 @@ class TensorProduct(torch.nn.Module):
         edge_src: Optional[torch.Tensor] = None,
         edge_dst: Optional[torch.Tensor] = None,
         num_nodes: Optional[int] = None,
-        edges: Optional[DstSortedEdges] = None,
+        edges=None,
     ) -> torch.Tensor:
         """``scatter(self(node_x[edge_src], edge_attr, weight), edge_dst, num_nodes)`` in one kernel.
 
@@ -549,6 +548,8 @@ class TensorProduct(torch.nn.Module):
         torch._assert(edge_attr.ndim == 2 and edge_attr.shape[-1] == self._in2_dim, "Incorrect shape for edge_attr")
         self._check_device(node_x, edge_attr)
         if edges is None:
+            from ..nn.edges import DstSortedEdges  # here: e3nn_amd.nn imports this module
+
             edges = DstSortedEdges(edge_src, edge_dst, node_x.shape[0] if num_nodes is None else num_nodes, node_x.shape[0])
         torch._assert(edge_attr.shape[0] == edges.num_edges, "edge_attr must have one row per edge")
         torch._assert(edges.num_src_nodes == node_x.shape[0], "edge list was built for another node count")

@@ -66,6 +66,27 @@ typedef struct {
   int32_t dtype;          /* E3X_F32 / E3X_BF16 storage of x1, x2, w, out */
 } e3x_tp_desc;
 
+/* activation functions of e3x_gate_* */
+#define E3X_ACT_IDENTITY 0
+#define E3X_ACT_SILU 1
+#define E3X_ACT_TANH 2
+#define E3X_ACT_SIGMOID 3
+#define E3X_ACT_ABS 4
+#define E3X_ACT_RELU 5
+
+/* `count` scalar channels: out[offset_out + c] = cst * act(x[offset_in + c]) */
+typedef struct {
+  int32_t offset_in, offset_out, count, act;
+  float cst;
+} e3x_act_block;
+
+/* `mul` copies of an irrep of dimension `dim`, copy u gated by scalar u of a run of `mul` gate scalars:
+ * out[offset_out + u*dim + m] = cst * act(x[gate_offset_in + u]) * x[gated_offset_in + u*dim + m] */
+typedef struct {
+  int32_t gate_offset_in, gated_offset_in, offset_out, mul, dim, act;
+  float cst;
+} e3x_gate_block;
+
 typedef struct e3x_plan e3x_plan;
 
 const char* e3x_last_error(void);
@@ -162,6 +183,17 @@ int e3x_sh_forward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t n
  * e3nn/o3/_spherical_harmonics.py:93-112,193-249 by autograd). */
 int e3x_sh_backward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization, const void* xyz,
                     const void* grad_out, void* grad_xyz, int64_t n, int32_t dtype, void* stream);
+
+/* Gated non-linearity on rows x[Z, in_dim] -> out[Z, out_dim] (fp32), at most 16 blocks of each kind; columns of `out`
+ * that no block covers become 0.  Replaces nn.Gate.forward (e3nn/nn/_gate.py:121-144: Extract, Activation,
+ * ElementwiseTensorProduct, cat) and, with n_gates = 0, nn.Activation.forward (e3nn/nn/_activation.py:78-104);
+ * `cst` is the second-moment normalisation of e3nn/math/_normalize_activation.py:22-57.  e3x_gate_backward writes
+ * grad_x[Z, in_dim] from grad_out[Z, out_dim] (the reference differentiates the same graph by autograd). */
+int e3x_gate_forward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_block* gates, int32_t n_gates, const void* x,
+                     void* out, int64_t Z, int64_t in_dim, int64_t out_dim, int32_t dtype, void* stream);
+int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_block* gates, int32_t n_gates, const void* x,
+                      const void* grad_out, void* grad_x, int64_t Z, int64_t in_dim, int64_t out_dim, int32_t dtype,
+                      void* stream);
 
 /* Plain device copy dst[i] = src[i], n_bytes multiple of 16: the calibration kernel
  * for bandwidth counters (known traffic: n_bytes read + n_bytes written). */

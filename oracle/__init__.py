@@ -8,6 +8,8 @@ algorithm of the reference e3nn implementation for
 * TensorProduct normalisation + ``uvu`` / ``uvw`` contraction (tensor_product.py)
 * cartesian spherical harmonics             (spherical_harmonics.py)
 * edge gather + destination scatter-sum     (message_passing.py)
+* the node-wise blocks either side of the message: o3.Linear, nn.Activation, nn.Gate,
+  nn.FullyConnectedNet, the v2106 Convolution  (nn.py)
 * a multi-threaded torch-CPU einsum restatement used only as the timed CPU
   baseline                                   (torch_cpu.py)
 
@@ -29,4 +31,7 @@ Pin status (what independently fixes each function; see tests/test_oracle_*.py):
                          normalisations), scipy's complex harmonics, norm / parity /
                          zero-vector identities, the w3j recurrence.
 * gather / scatter ..... pinned: integer-valued payloads (bit-exact), golden output.
+* Linear / Activation / Gate / FullyConnectedNet / Convolution
+                         pinned: golden outputs from the reference (instruction tables,
+                         irreps, normalisation constants, outputs), Linear's closed form on scalars.
 """

@@ -16,6 +16,8 @@ expected outputs only:
                    irreps, output_mask) incl. the five benchmark configurations
 * tp_cases.npz     seeded inputs and outputs of small TensorProducts and of
                    gather -> TensorProduct -> scatter
+* nn_cases.npz/json  (``python tests/golden/make_golden.py nn``) o3.Linear, nn.Activation, nn.Gate,
+                   nn.FullyConnectedNet and the v2106 Convolution: parameters, inputs, outputs, irreps strings
 """
 import json
 import os
@@ -206,5 +208,84 @@ def main():
     print("wrote", sorted(os.listdir(HERE)))
 
 
+def main_nn(ref="/root/reference"):
+    """Node-wise blocks around the message: fixtures for the oracle's restatements in oracle/nn.py."""
+    o3 = import_reference(ref)
+    from e3nn import nn
+    from e3nn.nn.models.v2106.points_convolution import Convolution
+
+    g = torch.Generator().manual_seed(1234)
+    rn = lambda *shape: torch.randn(*shape, generator=g)  # noqa: E731
+    arrays, meta = {}, {}
+
+    for name, (a, b, kw) in {
+        "linear_mixed": ("4x0e+3x1o+2x0e", "5x0e+2x1o+3x1o+1x2e", {}),
+        "linear_path_norm": ("4x0e+3x1o+2x0e", "5x0e+2x1o", {"path_normalization": "path"}),
+        "linear_bias": ("6x0e+2x1e", "3x0e+2x1e+2x0e", {"biases": True}),
+    }.items():
+        lin = o3.Linear(a, b, **kw)
+        if lin.bias_numel:
+            with torch.no_grad():
+                lin.bias.copy_(rn(lin.bias_numel))
+        x = rn(7, lin.irreps_in.dim)
+        arrays[name + "/x"], arrays[name + "/w"], arrays[name + "/out"] = x.numpy(), lin.weight.detach().numpy(), lin(x).detach().numpy()
+        arrays[name + "/bias"] = lin.bias.detach().numpy()
+        meta[name] = {"irreps_in": a, "irreps_out": b, "kwargs": kw, "weight_numel": lin.weight_numel,
+                      "instructions": [[i.i_in, i.i_out, list(i.path_shape), i.path_weight] for i in lin.instructions]}  # fmt: skip
+
+    acts = {"silu": torch.nn.functional.silu, "tanh": torch.tanh, "sigmoid": torch.sigmoid, "abs": torch.abs, "relu": torch.relu}
+    from e3nn.math import normalize2mom
+    meta["cst"] = {k: normalize2mom(f).cst for k, f in acts.items()}
+
+    act = nn.Activation("5x0e+3x0o+2x1e+4x0o", [torch.nn.functional.silu, torch.tanh, None, torch.abs])
+    x = rn(6, act.irreps_in.dim)
+    arrays["activation/x"], arrays["activation/out"] = x.numpy(), act(x).numpy()
+    meta["activation"] = {"irreps_in": str(act.irreps_in), "acts": ["silu", "tanh", None, "abs"], "irreps_out": str(act.irreps_out)}
+
+    for name, (sc, a_s, ga, a_g, gd) in {
+        "gate_plain": ("6x0e", ["silu"], "5x0e", ["sigmoid"], "3x1o+2x2e"),
+        "gate_parity": ("4x0e+2x0o", ["silu", "tanh"], "3x0e+4x0o", ["sigmoid", "tanh"], "2x1o+3x1e+2x2e"),
+        "gate_only_scalars": ("7x0e", ["relu"], "", [], ""),
+    }.items():
+        gate = nn.Gate(sc, [acts[k] for k in a_s], ga, [acts[k] for k in a_g], gd)
+        x = rn(5, gate.irreps_in.dim)
+        arrays[name + "/x"], arrays[name + "/out"] = x.numpy(), gate(x).numpy()
+        meta[name] = {"args": [sc, a_s, ga, a_g, gd], "irreps_in": str(gate.irreps_in), "irreps_out": str(gate.irreps_out)}
+
+    fc = nn.FullyConnectedNet([3, 16, 8, 5], torch.nn.functional.silu)
+    x = rn(9, 3)
+    arrays["fc/x"], arrays["fc/out"] = x.numpy(), fc(x).detach().numpy()
+    for i in range(3):
+        arrays[f"fc/w{i}"] = getattr(fc, f"layer{i}").weight.detach().numpy()
+    meta["fc"] = {"hs": [3, 16, 8, 5], "act": "silu"}
+
+    conv = Convolution("4x0e+3x1o+2x1e", "2x0e", "0e+1o+2e", "5x0e+2x1o+3x2e", [3, 8], 4.0)
+    with torch.no_grad():
+        conv.alpha.weight.copy_(rn(conv.alpha.weight_numel))  # the reference zero-initialises it: exercise the path
+    N, E = 11, 40
+    node_input, node_attr = rn(N, conv.irreps_node_input.dim), rn(N, 2)
+    src, dst = torch.randint(0, N, (E,), generator=g), torch.randint(0, N, (E,), generator=g)
+    vec = rn(E, 3)
+    edge_attr = o3.spherical_harmonics([0, 1, 2], vec, True, "component")
+    edge_scalars = rn(E, 3)
+    out = conv(node_input, node_attr, src, dst, edge_attr, edge_scalars)
+    for k, v in dict(node_input=node_input, node_attr=node_attr, src=src, dst=dst, edge_attr=edge_attr,
+                     edge_scalars=edge_scalars, out=out.detach()).items():  # fmt: skip
+        arrays["conv/" + k] = v.numpy()
+    for k, v in conv.state_dict().items():
+        if k.endswith("weight") and v.numel():
+            arrays["conv/param/" + k] = v.numpy()
+    meta["conv"] = {"args": ["4x0e+3x1o+2x1e", "2x0e", "0e+1o+2e", "5x0e+2x1o+3x2e", [3, 8], 4.0],
+                    "irreps_mid": str(conv.tp.irreps_out), "tp_instructions": [[i.i_in1, i.i_in2, i.i_out] for i in conv.tp.instructions]}  # fmt: skip
+
+    np.savez_compressed(os.path.join(HERE, "nn_cases.npz"), **arrays)
+    with open(os.path.join(HERE, "nn_cases.json"), "w") as f:
+        json.dump(meta, f, separators=(",", ":"))
+    print("wrote nn_cases", len(arrays), "arrays")
+
+
 if __name__ == "__main__":
-    main()
+    if len(sys.argv) > 1 and sys.argv[1] == "nn":
+        main_nn(*sys.argv[2:])
+    else:
+        main()

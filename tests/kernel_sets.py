@@ -121,7 +121,47 @@ BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "u
                   "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "radial_layer", "odd_mul"]  # fmt: skip
 
 
+def nn_golden():
+    import numpy as np
+
+    with open(os.path.join(GOLDEN, "nn_cases.json")) as f:
+        meta = json.load(f)
+    return np.load(os.path.join(GOLDEN, "nn_cases.npz")), meta
+
+
+def nn_modules():
+    """(name, module) for the node-wise blocks the GPU tests run; every TensorProduct inside needs its kernels."""
+    from e3nn_amd import nn
+
+    _, meta = nn_golden()
+    out = []
+    for name in ("linear_mixed", "linear_path_norm", "linear_bias"):
+        m = meta[name]
+        out.append((name, o3.Linear(m["irreps_in"], m["irreps_out"], **m["kwargs"])))
+    out.append(("linear_wide", o3.Linear("128x0e+128x1o+64x2e", "128x0e+64x1o+32x1o")))
+    out.append(("fc_golden", nn.FullyConnectedNet(meta["fc"]["hs"], torch.nn.functional.silu)))
+    out.append(("fc_radial", nn.FullyConnectedNet([8, 64, 352], torch.nn.functional.silu)))
+    a = meta["conv"]["args"]
+    out.append(("conv_golden", nn.Convolution(a[0], a[1], a[2], a[3], a[4], a[5])))
+    out.append(("conv_wide", conv_wide()))
+    return out
+
+
+def conv_wide():
+    # one interaction block at NequIP-like width: 32 channels per irrep, 4 species, 8 radial basis functions
+    from e3nn_amd import nn
+
+    f = "32x0e+32x1o+32x2e"
+    return nn.Convolution(f, "4x0e", SH2, f, [8, 64], 37.5)
+
+
 def prebuild(verbose=True):
+    for name, mod in nn_modules():
+        for sub in mod.modules():
+            if isinstance(sub, o3.TensorProduct):
+                sub.compile_backward(torch.float32)
+        if verbose:
+            print(f"module {name}", flush=True)
     for name, tp, dtypes in all_tensor_products():
         for dt in dtypes:
             plan = tp._plan(dt)

@@ -1,0 +1,169 @@
+"""GPU parity of the node-wise blocks either side of the message (o3.Linear, nn.Activation, nn.Gate,
+nn.FullyConnectedNet, the v2106 Convolution): the modules on the HIP kernels against fixtures written from the
+reference and against the fp64 oracle (oracle/nn.py); gradients against central differences of the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from e3nn_amd import nn, o3
+from oracle import nn as onn
+from tests import kernel_sets as ks
+from tests.helpers import assert_close, seeded
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _t(a):
+    return torch.from_numpy(np.asarray(a)).float().to(DEV)
+
+
+@pytest.mark.parametrize("name", ["linear_mixed", "linear_path_norm", "linear_bias"])
+def test_linear_against_reference_fixture(name):
+    arr, meta = ks.nn_golden()
+    m = meta[name]
+    lin = o3.Linear(m["irreps_in"], m["irreps_out"], **m["kwargs"]).to(DEV)
+    assert lin.weight_numel == m["weight_numel"]
+    with torch.no_grad():
+        lin.weight.copy_(_t(arr[name + "/w"]))
+        if lin.bias_numel:
+            lin.bias.copy_(_t(arr[name + "/bias"]))
+    assert_close(lin(_t(arr[name + "/x"])), arr[name + "/out"], what=name)
+
+
+def test_linear_on_the_matrix_cores():
+    lin = dict(ks.nn_modules())["linear_wide"].to(DEV)
+    assert lin._tp._plan(torch.float32).family == "uvw_mfma"
+    x = seeded(300, lin.irreps_in.dim, seed=5)
+    ref = onn.linear_forward(str(lin.irreps_in), str(lin.irreps_out), x.numpy(), lin.weight.detach().cpu().numpy())
+    xd = x.to(DEV).requires_grad_(True)
+    out = lin(xd)
+    assert_close(out, ref, what="linear_wide")
+    # the map is linear in x and in w: <cot, L(x)> differentiates to L^T cot and to x (x) cot
+    cot = seeded(300, lin.irreps_out.dim, seed=6)
+    out.backward(cot.to(DEV))
+    ref_gx = onn.linear_forward(str(lin.irreps_in), str(lin.irreps_out), np.eye(lin.irreps_in.dim), lin.weight.detach().cpu().numpy())
+    assert_close(xd.grad, cot.numpy().astype(np.float64) @ ref_gx.T, atol=2e-4, what="d/dx")
+    w = lin.weight.detach().cpu().numpy().astype(np.float64)
+    rng = np.random.default_rng(0)
+    dw = rng.normal(size=w.shape)
+    fd = (onn.linear_forward(str(lin.irreps_in), str(lin.irreps_out), x.numpy(), dw) * cot.numpy()).sum()
+    assert float((lin.weight.grad.cpu().double().numpy() * dw).sum()) == pytest.approx(fd, rel=2e-4)
+
+
+def test_activation_and_gate_against_reference_fixtures():
+    arr, meta = ks.nn_golden()
+    acts = {"silu": torch.nn.functional.silu, "tanh": torch.tanh, "sigmoid": torch.sigmoid, "abs": torch.abs, "relu": torch.relu}
+    m = meta["activation"]
+    act = nn.Activation(m["irreps_in"], [acts[a] if a else None for a in m["acts"]])
+    assert str(act.irreps_out) == m["irreps_out"]
+    assert_close(act(_t(arr["activation/x"])), arr["activation/out"], what="activation")
+    for name in ("gate_plain", "gate_parity", "gate_only_scalars"):
+        sc, a_s, ga, a_g, gd = meta[name]["args"]
+        gate = nn.Gate(sc, [acts[k] for k in a_s], ga, [acts[k] for k in a_g], gd)
+        assert str(gate.irreps_in) == meta[name]["irreps_in"], name
+        assert str(gate.irreps_out.simplify()) == str(o3.Irreps(meta[name]["irreps_out"]).simplify()), name
+        assert_close(gate(_t(arr[name + "/x"])), arr[name + "/out"], what=name)
+
+
+def test_gate_gradient_against_central_differences():
+    args = ("16x0e+4x0o", ["silu", "tanh"], "8x0e+4x0o", ["sigmoid", "tanh"], "8x1o+4x2e")
+    gate = nn.Gate(args[0], args[1], args[2], args[3], args[4])
+    x = seeded(33, gate.irreps_in.dim, seed=3)
+    cot = seeded(33, gate.irreps_out.dim, seed=4)
+    xd = x.to(DEV).requires_grad_(True)
+    out = gate(xd)
+    ref, _, _ = onn.gate_forward(*args, x.numpy())
+    assert_close(out, ref, what="gate")
+    out.backward(cot.to(DEV))
+    rng = np.random.default_rng(1)
+    x64, c64 = x.numpy().astype(np.float64), cot.numpy().astype(np.float64)
+    for _ in range(3):
+        v = rng.normal(size=x64.shape)
+        eps = 1e-5
+        fd = ((onn.gate_forward(*args, x64 + eps * v)[0] - onn.gate_forward(*args, x64 - eps * v)[0]) * c64).sum() / (2 * eps)
+        assert float((xd.grad.cpu().double().numpy() * v).sum()) == pytest.approx(fd, rel=1e-4, abs=1e-4)
+
+
+def test_fully_connected_net():
+    arr, meta = ks.nn_golden()
+    fc = nn.FullyConnectedNet(meta["fc"]["hs"], torch.nn.functional.silu).to(DEV)
+    with torch.no_grad():
+        for i in range(3):
+            getattr(fc, f"layer{i}").weight.copy_(_t(arr[f"fc/w{i}"]))
+    assert_close(fc(_t(arr["fc/x"])), arr["fc/out"], what="fc fixture")
+    # radial-network shape: 8 -> 64 -> 352, the second layer on the matrix cores
+    fc = dict(ks.nn_modules())["fc_radial"].to(DEV)
+    assert fc.layer1._tp._plan(torch.float32).family == "uvw_mfma"
+    x = seeded(1000, 8, seed=8)
+    ws = [fc.layer0.weight.detach().cpu().numpy(), fc.layer1.weight.detach().cpu().numpy()]
+    xd = x.to(DEV).requires_grad_(True)
+    out = fc(xd)
+    assert_close(out, onn.fc_forward(ws, x.numpy(), "silu"), what="fc radial")
+    cot = seeded(1000, 352, seed=9)
+    out.backward(cot.to(DEV))
+    rng = np.random.default_rng(2)
+    x64, c64 = x.numpy().astype(np.float64), cot.numpy().astype(np.float64)
+    v = rng.normal(size=x64.shape)
+    eps = 1e-5
+    fd = ((onn.fc_forward(ws, x64 + eps * v) - onn.fc_forward(ws, x64 - eps * v)) * c64).sum() / (2 * eps)
+    assert float((xd.grad.cpu().double().numpy() * v).sum()) == pytest.approx(fd, rel=2e-4)
+    dw = rng.normal(size=ws[0].shape)
+    fd = ((onn.fc_forward([ws[0] + eps * dw, ws[1]], x64) - onn.fc_forward([ws[0] - eps * dw, ws[1]], x64)) * c64).sum() / (2 * eps)
+    assert float((fc.layer0.weight.grad.cpu().double().numpy() * dw).sum()) == pytest.approx(fd, rel=2e-4)
+
+
+def _conv_oracle(conv, args, params, node_input, node_attr, src, dst, edge_attr, edge_scalars):
+    return onn.convolution_forward(args[0], args[1], args[2], args[3], args[5], params, node_input, node_attr, src, dst,
+                                   edge_attr, edge_scalars)  # fmt: skip
+
+
+def test_convolution_against_reference_fixture():
+    arr, meta = ks.nn_golden()
+    a = meta["conv"]["args"]
+    conv = nn.Convolution(a[0], a[1], a[2], a[3], a[4], a[5]).to(DEV)
+    assert str(conv.tp.irreps_out) == meta["conv"]["irreps_mid"]
+    assert [[i.i_in1, i.i_in2, i.i_out] for i in conv.tp.instructions] == meta["conv"]["tp_instructions"]
+    sd = {k[len("conv/param/"):]: _t(arr[k]) for k in arr.files if k.startswith("conv/param/")}
+    missing = conv.load_state_dict(sd, strict=False)
+    assert not [k for k in missing.unexpected_keys], missing
+    own = conv.state_dict()
+    assert not [k for k in missing.missing_keys if k.endswith("weight") and "_tp" not in k and own[k].numel()], missing
+    out = conv(_t(arr["conv/node_input"]), _t(arr["conv/node_attr"]), torch.from_numpy(arr["conv/src"]).to(DEV),
+               torch.from_numpy(arr["conv/dst"]).to(DEV), _t(arr["conv/edge_attr"]), _t(arr["conv/edge_scalars"]))  # fmt: skip
+    assert_close(out, arr["conv/out"], atol=2e-4, what="convolution fixture")
+
+
+def test_convolution_block_forward_and_backward():
+    conv = ks.conv_wide().to(DEV)
+    with torch.no_grad():
+        conv.alpha.weight.normal_()
+    N, E = 150, 2500
+    g = torch.Generator().manual_seed(11)
+    src, dst = torch.randint(0, N, (E,), generator=g), torch.randint(0, N, (E,), generator=g)
+    node_input, node_attr = seeded(N, 288, seed=1), seeded(N, 4, seed=2)
+    vec = seeded(E, 3, seed=3)
+    edge_attr = o3.spherical_harmonics([0, 1, 2], vec.to(DEV), True, "component").cpu()
+    edge_scalars = seeded(E, 8, seed=4)
+    params = {k: v.detach().cpu().numpy().astype(np.float64) for k, v in conv.state_dict().items() if k.endswith("weight") and v.numel()}
+    a = ("32x0e+32x1o+32x2e", "4x0e", ks.SH2, "32x0e+32x1o+32x2e", [8, 64], 37.5)
+    run = lambda x, p=params: _conv_oracle(conv, a, p, x, node_attr.numpy(), src.numpy(), dst.numpy(), edge_attr.numpy(), edge_scalars.numpy())  # noqa: E731
+    xd = node_input.to(DEV).requires_grad_(True)
+    out = conv(xd, node_attr.to(DEV), src.to(DEV), dst.to(DEV), edge_attr.to(DEV), edge_scalars.to(DEV))
+    ref = run(node_input.numpy())
+    assert_close(out, ref, atol=1e-4 * max(1.0, float(np.abs(ref).max())), what="convolution block")
+    cot = seeded(N, 288, seed=5)
+    out.backward(cot.to(DEV))
+    rng = np.random.default_rng(3)
+    x64, c64 = node_input.numpy().astype(np.float64), cot.numpy().astype(np.float64)
+    v = rng.normal(size=x64.shape)
+    eps = 1e-5
+    fd = ((run(x64 + eps * v) - run(x64 - eps * v)) * c64).sum() / (2 * eps)
+    assert float((xd.grad.cpu().double().numpy() * v).sum()) == pytest.approx(fd, rel=5e-4)
+    for key, par in (("fc.layer0.weight", conv.fc.layer0.weight), ("lin1.weight", conv.lin1.weight), ("alpha.weight", conv.alpha.weight)):
+        dw = rng.normal(size=params[key].shape)
+        hi, lo = dict(params), dict(params)
+        hi[key], lo[key] = params[key] + eps * dw, params[key] - eps * dw
+        fd = ((run(x64, hi) - run(x64, lo)) * c64).sum() / (2 * eps)
+        got = float((par.grad.cpu().double().numpy().reshape(dw.shape) * dw).sum())
+        assert got == pytest.approx(fd, rel=5e-4, abs=1e-3), key

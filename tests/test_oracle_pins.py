@@ -293,3 +293,86 @@ def test_wigner_D_is_a_representation_and_w3j_is_invariant():
         lhs = otp.tp_forward(spec, x1 @ Da.T, x2 @ Db.T, w)
         rhs = otp.tp_forward(spec, x1, x2, w) @ Dc.T
         np.testing.assert_allclose(lhs, rhs, atol=1e-10)
+
+
+# ---- node-wise blocks either side of the message (oracle/nn.py) against fixtures written from the reference ----
+import json as _json
+import os as _os
+
+
+def _nn_golden():
+    here = _os.path.join(_os.path.dirname(_os.path.abspath(__file__)), "golden")
+    return np.load(_os.path.join(here, "nn_cases.npz")), _json.load(open(_os.path.join(here, "nn_cases.json")))
+
+
+@pytest.mark.parametrize("name", ["linear_mixed", "linear_path_norm", "linear_bias"])
+def test_linear_matches_reference(name):
+    from oracle import nn as onn
+
+    arr, meta = _nn_golden()
+    m = meta[name]
+    kw = m["kwargs"]
+    ins = onn.linear_instructions(m["irreps_in"], m["irreps_out"], None, kw.get("path_normalization", "element"))
+    ref_ins = [t for t in m["instructions"] if t[0] != -1]
+    assert [(a, b) for a, b, _, _ in ins] == [(t[0], t[1]) for t in ref_ins]
+    np.testing.assert_allclose([t[3] for t in ins], [t[3] for t in ref_ins], rtol=1e-14)
+    from oracle import irreps as oir
+
+    biases = [bool(kw.get("biases")) and l == 0 for _, l, _ in oir.parse(m["irreps_out"])] if kw.get("biases") else None
+    out = onn.linear_forward(m["irreps_in"], m["irreps_out"], arr[name + "/x"], arr[name + "/w"],
+                             path_normalization=kw.get("path_normalization", "element"), bias=arr[name + "/bias"], biases=biases)  # fmt: skip
+    np.testing.assert_allclose(out, arr[name + "/out"], rtol=1e-12, atol=1e-12)
+
+
+def test_linear_closed_form_on_scalars():
+    from oracle import nn as onn
+
+    rng = np.random.default_rng(0)
+    x, w = rng.normal(size=(5, 10)), rng.normal(size=30)
+    np.testing.assert_allclose(onn.linear_forward("10x0e", "3x0e", x, w), x @ w.reshape(10, 3) / np.sqrt(10), rtol=1e-13)
+
+
+def test_activation_constants_and_forward_match_reference():
+    from oracle import nn as onn
+
+    arr, meta = _nn_golden()
+    for k, v in meta["cst"].items():
+        assert onn.normalize2mom_const(k) == pytest.approx(v, rel=1e-13)
+    m = meta["activation"]
+    out, irreps_out = onn.activation_forward(m["irreps_in"], m["acts"], arr["activation/x"])
+    from oracle import irreps as oir
+
+    assert oir.to_str(irreps_out) == m["irreps_out"]
+    np.testing.assert_allclose(out, arr["activation/out"], rtol=1e-12, atol=1e-13)
+
+
+@pytest.mark.parametrize("name", ["gate_plain", "gate_parity", "gate_only_scalars"])
+def test_gate_matches_reference(name):
+    from oracle import irreps as oir
+    from oracle import nn as onn
+
+    arr, meta = _nn_golden()
+    m = meta[name]
+    out, irreps_in, irreps_out = onn.gate_forward(*m["args"], arr[name + "/x"])
+    assert oir.to_str(irreps_in) == m["irreps_in"]
+    assert oir.to_str(oir.simplify(irreps_out)) == str(m["irreps_out"]) or oir.to_str(irreps_out) == m["irreps_out"]
+    np.testing.assert_allclose(out, arr[name + "/out"], rtol=1e-12, atol=1e-13)
+
+
+def test_fully_connected_net_matches_reference():
+    from oracle import nn as onn
+
+    arr, meta = _nn_golden()
+    out = onn.fc_forward([arr[f"fc/w{i}"] for i in range(3)], arr["fc/x"], meta["fc"]["act"])
+    np.testing.assert_allclose(out, arr["fc/out"], rtol=1e-12, atol=1e-13)
+
+
+def test_convolution_matches_reference():
+    from oracle import nn as onn
+
+    arr, meta = _nn_golden()
+    a = meta["conv"]["args"]
+    params = {k[len("conv/param/"):]: arr[k] for k in arr.files if k.startswith("conv/param/")}
+    out = onn.convolution_forward(a[0], a[1], a[2], a[3], a[5], params, arr["conv/node_input"], arr["conv/node_attr"],
+                                  arr["conv/src"], arr["conv/dst"], arr["conv/edge_attr"], arr["conv/edge_scalars"])  # fmt: skip
+    np.testing.assert_allclose(out, arr["conv/out"], rtol=1e-11, atol=1e-12)
