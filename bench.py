@@ -272,6 +272,34 @@ def bench_nequip_cube40(args, dev):
             "roofline_frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "bytes_per_launch": b}  # fmt: skip
 
 
+def bench_convolution(args, dev, ctx):
+    """One whole interaction block (reference e3nn/nn/models/v2106/points_convolution.py:99-113) on the headline
+    graph: radial network 8 -> 64 -> 352, self-connection, lin1, fused message, lin2, alpha; 4 species."""
+    from e3nn_amd.nn import DstSortedEdges
+    from tests import kernel_sets as ks
+
+    conv = ks.conv_wide().to(dev)
+    N, E = ctx["N"], ctx["src"].shape[0]
+    gen = torch.Generator().manual_seed(0)
+    node_attr = torch.nn.functional.one_hot(torch.randint(0, 4, (N,), generator=gen), 4).float().to(dev)
+    edge_scalars = torch.randn(E, 8, generator=gen).to(dev)
+    edges = DstSortedEdges(ctx["src"], ctx["dst"], N)
+    x = ctx["node_x"].clone().requires_grad_(True)
+
+    def fwd():
+        with torch.no_grad():
+            return conv(x, node_attr, ctx["src"], ctx["dst"], ctx["attr"], edge_scalars, edges=edges)
+
+    def fwd_bwd():
+        x.grad = None
+        conv.zero_grad(set_to_none=True)
+        conv(x, node_attr, ctx["src"], ctx["dst"], ctx["attr"], edge_scalars, edges=edges).square().sum().backward()
+
+    ms_f = event_time_ms(fwd, max(5, args.steps // 5), 2)
+    ms_fb = event_time_ms(fwd_bwd, max(3, args.steps // 10), 1)
+    return {"edges": E, "nodes": N, "ms_forward": ms_f, "ms_forward_backward": ms_fb, "edges_per_s_forward": E / (ms_f * 1e-3)}
+
+
 def bench_library_gemm(args, dev):
     """Context for the matrix-core rooflines: what the vendor GEMM (torch.matmul -> rocBLAS / hipBLASLt) reaches
     on this GPU with N(0,1) data, 8192^3."""
@@ -339,7 +367,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--locality-variants", action="store_true", help="also time the headline graph with sorted edges / Morton node ids")
-    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_b,mace_bf16,nequip40,uvw,uvw_bf16,nequip_bwd,uvw_bwd (default: all)")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_b,mace_bf16,nequip40,uvw,uvw_bf16,conv,nequip_bwd,uvw_bwd (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported (no collectives, no sharding)")
@@ -350,7 +378,7 @@ def main():
 
     neq, ctx = bench_nequip(args, dev)
     other = {"nequip_uvu": neq}
-    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_b", "mace_bf16", "nequip40", "uvw", "uvw_bf16", "nequip_bwd", "uvw_bwd"}
+    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_b", "mace_bf16", "nequip40", "uvw", "uvw_bf16", "conv", "nequip_bwd", "uvw_bwd"}
     if "copy" in want:
         other["copy_1GiB"] = bench_copy(args, dev)
     if "sh" in want:
@@ -369,6 +397,8 @@ def main():
         other["uvw_dense_bf16"] = bench_uvw(args, dev, torch.bfloat16)
     if "uvw" in want or "uvw_bf16" in want:
         other["library_gemm_8192_randn"] = bench_library_gemm(args, dev)
+    if "conv" in want:
+        other["convolution_block"] = bench_convolution(args, dev, ctx)
     if "nequip_bwd" in want:
         other["nequip_uvu_forward_backward"] = bench_nequip_backward(args, dev, ctx)
     if "uvw_bwd" in want:

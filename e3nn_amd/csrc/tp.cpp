@@ -34,6 +34,7 @@ struct SubKernel {
   std::string key, hsaco;
   std::vector<int> path_ids;  // indices into e3x_plan::paths
   int lanes = 64, chunks = 1, upl = 1, waves_per_block = 4;
+  bool cached_weights = false;  // uvw_small: weights in registers, rows walked with a grid-sized stride
   hipModule_t module[kMaxDevices] = {nullptr};
   hipFunction_t fn_plain[kMaxDevices] = {nullptr};
   hipFunction_t fn_fused[kMaxDevices] = {nullptr};
@@ -290,15 +291,23 @@ int build_uvw_small_source(e3x_plan& P, SubKernel& K, std::string* src) {
   s << "};\nconstexpr int ACC_REGS = " << reg << ";\n";
   if (reg > 256) return fail(E3X_ERR_INVALID, "uvw kernel: more than 256 output components per multiplicity index");
   NzList L = emit_nz(P, K.path_ids);
-  s << "struct Path { int x1off, d1, U, x2off, d2, V, out, woff; int nz_beg, nz_end; };\n";
+  // shared weights of few (u, v) pairs live in registers, one per pair and lane (one chunk of output channels only)
+  long long pairs = 0;
+  for (const auto& p : P.paths) pairs += (long long)P.in1[p.in1].mul * P.in2[p.in2].mul;
+  const bool cached = P.shared_weights && K.chunks == 1 && pairs > 0 && pairs <= 64;
+  K.cached_weights = cached;
+  s << "constexpr int W_CACHE_REGS = " << (cached ? pairs : 0) << ";\n";
+  s << "struct Path { int x1off, d1, U, x2off, d2, V, out, woff, wreg; int nz_beg, nz_end; };\n";
   s << "constexpr int N_PATH = " << P.paths.size() << ";\nconstexpr Path paths[N_PATH > 0 ? N_PATH : 1] = {\n";
+  int wreg = 0;
   for (size_t i = 0; i < P.paths.size(); ++i) {
     const auto& p = P.paths[i];
     s << "  {" << P.off1[p.in1] << ", " << 2 * P.in1[p.in1].l + 1 << ", " << P.in1[p.in1].mul << ", " << P.off2[p.in2]
-      << ", " << 2 * P.in2[p.in2].l + 1 << ", " << P.in2[p.in2].mul << ", " << p.out << ", " << p.woff << ", "
-      << L.beg[i] << ", " << L.end[i] << "},\n";
+      << ", " << 2 * P.in2[p.in2].l + 1 << ", " << P.in2[p.in2].mul << ", " << p.out << ", " << p.woff << ", " << wreg
+      << ", " << L.beg[i] << ", " << L.end[i] << "},\n";
+    wreg += P.in1[p.in1].mul * P.in2[p.in2].mul;
   }
-  if (P.paths.empty()) s << "  {0, 1, 0, 0, 1, 0, 0, 0, 0, 0}\n";
+  if (P.paths.empty()) s << "  {0, 1, 0, 0, 1, 0, 0, 0, 0, 0, 0}\n";
   s << "};\n";
   emit_nz_table(s, L);
   s << "}  // namespace cfg\n";
@@ -307,13 +316,18 @@ int build_uvw_small_source(e3x_plan& P, SubKernel& K, std::string* src) {
 }
 
 // ---- uvw on the matrix cores ----------------------------------------------------------
+// largest GEMM K extent (multiplicity of the K operand) of the matrix-core kernels: the fp32 kernel keeps a
+// 64-row slice of the K operand in LDS (K * 256 bytes), the bf16 kernel keeps its K operand in registers
+int k_cap(int dtype) { return dtype == E3X_BF16 ? 256 : 512; }
+
 bool uvw_mfma_eligible(const e3x_plan& P) {
   if (!P.shared_weights || P.paths.empty()) return false;
   for (const auto& p : P.paths) {
     const int U = P.in1[p.in1].mul, V = P.in2[p.in2].mul, W = P.out[p.out].mul;
     // fp32: 32-channel granularity (a half-filled last tile); bf16: whole 64-channel tiles
     if (W % (P.dtype == E3X_BF16 ? 64 : 32) || P.out[p.out].l > 3 || U < 1 || V < 1) return false;
-    const bool okU = U % 32 == 0 && U <= 256, okV = V % 32 == 0 && V <= 256;
+    const int kcap = k_cap(P.dtype);
+    const bool okU = U % 32 == 0 && U <= kcap, okV = V % 32 == 0 && V <= kcap;
     if (P.dtype == E3X_BF16) {
       // both multiplicities tile: the outer index runs in blocks of 8
       if (!okU || !okV) return false;
@@ -348,7 +362,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
       // GEMM passes per outer index: 2l+1 of the K operand when accumulators are scaled, 2 l3 + 1 when the
       // operand is synthesised; take the cheapest
       // (the bf16 kernel scales accumulators only: its matrix passes are cheap next to the fp32 epilogue)
-      const bool okU = a.mul % 32 == 0 && a.mul <= 256, okV = b.mul % 32 == 0 && b.mul <= 256;
+      const bool okU = a.mul % 32 == 0 && a.mul <= k_cap(P.dtype), okV = b.mul % 32 == 0 && b.mul <= k_cap(P.dtype);
       const bool synth = P.dtype == E3X_F32 && env_int("E3X_UVW_SYNTH", 1) && d3 < std::min(d1, d2) && okU;
       const bool k_is_x2 = !synth && okV && (!okU || d2 < d1);
       kmax = std::max(kmax, k_is_x2 ? b.mul : a.mul);
@@ -409,7 +423,7 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
   // the kernel reads 8 multiplicity indices of the M operand and of the output gradient with 16-byte loads
   for (const auto& p : P.paths) {
     const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2];
-    const bool okU = a.mul % 32 == 0 && a.mul <= 256, okV = b.mul % 32 == 0 && b.mul <= 256;
+    const bool okU = a.mul % 32 == 0 && a.mul <= k_cap(P.dtype), okV = b.mul % 32 == 0 && b.mul <= k_cap(P.dtype);
     const bool m_is_x2 = okV && (!okU || b.l < a.l);
     const int moff = m_is_x2 ? P.off2[p.in2] : P.off1[p.in1];
     const int64_t mdim = m_is_x2 ? P.in2_dim : P.in1_dim;
@@ -419,7 +433,7 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
   for (const auto& p : P.paths) {
     const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2], &c = P.out[p.out];
     const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1, d3 = 2 * c.l + 1;
-    const bool okU = a.mul % 32 == 0 && a.mul <= 256, okV = b.mul % 32 == 0 && b.mul <= 256;
+    const bool okU = a.mul % 32 == 0 && a.mul <= k_cap(P.dtype), okV = b.mul % 32 == 0 && b.mul <= k_cap(P.dtype);
     const bool k_is_x2 = okV && (!okU || d2 < d1);  // the M operand tiles by 32
     const auto& C = e3x::wigner_3j(a.l, b.l, c.l);
     const int nz_beg = n_nz;
@@ -686,6 +700,7 @@ extern "C" int e3x_tp_forward_ws(e3x_plan* P, const void* x1, const void* x2, co
       const int groups = 64 / K->lanes;
       const long long items = (Z + groups - 1) / groups * K->chunks;
       blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
+      if (K->cached_weights) blocks = std::min(blocks, 256LL * 16);  // a few workgroups per CU, each walking many rows
     }
     if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_forward: batch too large for one launch");
     hipError_t err =
