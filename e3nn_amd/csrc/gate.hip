@@ -57,72 +57,98 @@ __device__ __forceinline__ void activation(int kind, float x, float& f, float& d
   }
 }
 
-// one thread per output element (row z, column c): consecutive threads write consecutive columns
-__global__ __launch_bounds__(256) void gate_fwd_kernel(Tables t, const float* __restrict__ x, float* __restrict__ out,
-                                                       long long n_rows, int in_dim, int out_dim) {
-  const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (id >= n_rows * out_dim) return;
-  const long long z = id / out_dim;
-  const int c = (int)(id - z * out_dim);
-  const float* row = x + z * in_dim;
-  float v = 0.f;
+// Thread (tx, ty) of a 64 x 4 block owns column 64 blockIdx.x + tx and walks rows 4 blockIdx.y + ty, + 4 gridDim.y, ...:
+// the block tables are searched once per thread, consecutive lanes touch consecutive columns of a row.
+constexpr int kCols = 64, kRows = 4;
+
+__global__ __launch_bounds__(kCols* kRows) void gate_fwd_kernel(Tables t, const float* __restrict__ x,
+                                                                float* __restrict__ out, long long n_rows, int in_dim,
+                                                                int out_dim) {
+  const int c = blockIdx.x * kCols + (threadIdx.x % kCols);
+  if (c >= out_dim) return;
+  int kind = -1, src = 0, gate = -1;  // kind < 0: no block covers this column
+  float cst = 0.f;
   for (int b = 0; b < t.n_act; ++b) {
     const e3x_act_block& a = t.act[b];
-    if (c >= a.offset_out && c < a.offset_out + a.count) {
-      float f, df;
-      activation(a.act, row[a.offset_in + (c - a.offset_out)], f, df);
-      v = a.cst * f;
-    }
+    if (c >= a.offset_out && c < a.offset_out + a.count) kind = a.act, cst = a.cst, src = a.offset_in + (c - a.offset_out);
   }
   for (int b = 0; b < t.n_gate; ++b) {
     const e3x_gate_block& g = t.gate[b];
     if (c >= g.offset_out && c < g.offset_out + g.mul * g.dim) {
-      const int rel = c - g.offset_out, u = rel / g.dim;
-      float f, df;
-      activation(g.act, row[g.gate_offset_in + u], f, df);
-      v = g.cst * f * row[g.gated_offset_in + rel];
+      const int rel = c - g.offset_out;
+      kind = g.act, cst = g.cst, src = g.gated_offset_in + rel, gate = g.gate_offset_in + rel / g.dim;
     }
   }
-  out[id] = v;
+  for (long long z = (long long)blockIdx.y * kRows + threadIdx.x / kCols; z < n_rows; z += (long long)gridDim.y * kRows) {
+    const float* row = x + z * in_dim;
+    float v = 0.f;
+    if (kind >= 0) {
+      float f, df;
+      activation(kind, row[gate >= 0 ? gate : src], f, df);
+      v = gate >= 0 ? cst * f * row[src] : cst * f;
+    }
+    out[z * out_dim + c] = v;
+  }
 }
 
-// one thread per input element: scalars and gated components take one term, a gate sums over its irrep's components
-__global__ __launch_bounds__(256) void gate_bwd_kernel(Tables t, const float* __restrict__ x,
-                                                       const float* __restrict__ gout, float* __restrict__ gx,
-                                                       long long n_rows, int in_dim, int out_dim) {
-  const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (id >= n_rows * in_dim) return;
-  const long long z = id / in_dim;
-  const int c = (int)(id - z * in_dim);
-  const float* row = x + z * in_dim;
-  const float* grow = gout + z * out_dim;
-  float v = 0.f;
+// the same walk over the input columns: a scalar or gated component takes one term, a gate sums over its irrep
+__global__ __launch_bounds__(kCols* kRows) void gate_bwd_kernel(Tables t, const float* __restrict__ x,
+                                                                const float* __restrict__ gout, float* __restrict__ gx,
+                                                                long long n_rows, int in_dim, int out_dim) {
+  const int c = blockIdx.x * kCols + (threadIdx.x % kCols);
+  if (c >= in_dim) return;
+  // roles of this input column (a column can play at most one role per block kind)
+  int a_kind = -1, a_out = 0;
+  float a_cst = 0.f;
+  int y_kind = -1, y_out = 0, y_gate = 0;  // gated component
+  float y_cst = 0.f;
+  int g_kind = -1, g_out = 0, g_src = 0, g_dim = 0;  // gate scalar
+  float g_cst = 0.f;
   for (int b = 0; b < t.n_act; ++b) {
     const e3x_act_block& a = t.act[b];
-    if (c >= a.offset_in && c < a.offset_in + a.count) {
-      float f, df;
-      activation(a.act, row[c], f, df);
-      v += a.cst * df * grow[a.offset_out + (c - a.offset_in)];
-    }
+    if (c >= a.offset_in && c < a.offset_in + a.count) a_kind = a.act, a_cst = a.cst, a_out = a.offset_out + (c - a.offset_in);
   }
   for (int b = 0; b < t.n_gate; ++b) {
     const e3x_gate_block& g = t.gate[b];
     if (c >= g.gated_offset_in && c < g.gated_offset_in + g.mul * g.dim) {
-      const int rel = c - g.gated_offset_in, u = rel / g.dim;
-      float f, df;
-      activation(g.act, row[g.gate_offset_in + u], f, df);
-      v += g.cst * f * grow[g.offset_out + rel];
+      const int rel = c - g.gated_offset_in;
+      y_kind = g.act, y_cst = g.cst, y_out = g.offset_out + rel, y_gate = g.gate_offset_in + rel / g.dim;
     }
     if (c >= g.gate_offset_in && c < g.gate_offset_in + g.mul) {
       const int u = c - g.gate_offset_in;
-      float f, df;
-      activation(g.act, row[c], f, df);
-      float s = 0.f;
-      for (int m = 0; m < g.dim; ++m) s += grow[g.offset_out + u * g.dim + m] * row[g.gated_offset_in + u * g.dim + m];
-      v += g.cst * df * s;
+      g_kind = g.act, g_cst = g.cst, g_out = g.offset_out + u * g.dim, g_src = g.gated_offset_in + u * g.dim, g_dim = g.dim;
     }
   }
-  gx[id] = v;
+  for (long long z = (long long)blockIdx.y * kRows + threadIdx.x / kCols; z < n_rows; z += (long long)gridDim.y * kRows) {
+    const float* row = x + z * in_dim;
+    const float* grow = gout + z * out_dim;
+    float v = 0.f, f, df;
+    if (a_kind >= 0) {
+      activation(a_kind, row[c], f, df);
+      v += a_cst * df * grow[a_out];
+    }
+    if (y_kind >= 0) {
+      activation(y_kind, row[y_gate], f, df);
+      v += y_cst * f * grow[y_out];
+    }
+    if (g_kind >= 0) {
+      activation(g_kind, row[c], f, df);
+      float s = 0.f;
+      for (int m = 0; m < g_dim; ++m) s += grow[g_out + m] * row[g_src + m];
+      v += g_cst * df * s;
+    }
+    gx[z * in_dim + c] = v;
+  }
+}
+
+// grid of the column-walk kernels: all column blocks, enough row blocks for a few workgroups per CU
+dim3 walk_grid(int64_t Z, int64_t dim) {
+  const long long cb = (dim + kCols - 1) / kCols;
+  long long rb = (Z + kRows - 1) / kRows;
+  const long long want = (256LL * 16 + cb - 1) / cb;
+  if (rb > want) rb = want;
+  if (rb > 65535) rb = 65535;
+  return dim3((unsigned)cb, (unsigned)rb);
 }
 
 int fill_tables(const char* who, const e3x_act_block* acts, int n_acts, const e3x_gate_block* gates, int n_gates,
@@ -165,9 +191,7 @@ extern "C" int e3x_gate_forward(const e3x_act_block* acts, int32_t n_acts, const
   if (Z < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: negative batch");
   if (Z == 0 || out_dim == 0) return E3X_OK;
   if (!x || !out) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: null pointer");
-  const long long n = Z * out_dim, blocks = (n + 255) / 256;
-  if (blocks >= (1LL << 31)) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: too many elements for one launch");
-  hipLaunchKernelGGL(gate_fwd_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, t, (const float*)x,
+  hipLaunchKernelGGL(gate_fwd_kernel, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
                      (float*)out, (long long)Z, (int)in_dim, (int)out_dim);
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_forward: kernel launch failed");
   return E3X_OK;
@@ -183,9 +207,7 @@ extern "C" int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, cons
   if (Z < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: negative batch");
   if (Z == 0 || in_dim == 0) return E3X_OK;
   if (!x || !grad_out || !grad_x) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: null pointer");
-  const long long n = Z * in_dim, blocks = (n + 255) / 256;
-  if (blocks >= (1LL << 31)) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: too many elements for one launch");
-  hipLaunchKernelGGL(gate_bwd_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, t, (const float*)x,
+  hipLaunchKernelGGL(gate_bwd_kernel, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
                      (const float*)grad_out, (float*)grad_x, (long long)Z, (int)in_dim, (int)out_dim);
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward: kernel launch failed");
   return E3X_OK;

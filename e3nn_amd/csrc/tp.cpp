@@ -696,6 +696,12 @@ extern "C" int e3x_tp_forward_ws(e3x_plan* P, const void* x1, const void* x2, co
       const int rows = 16 * K->waves_per_block;  // fp32: 4 waves, 64 rows; bf16: 8 waves, 128 rows
       blocks = (Z + rows - 1) / rows;
       grid_y = (unsigned)P->n_targets;
+      // weights that fit in one L2 with room to spare: order the workgroups by row tile (fp32 kernel)
+      if (P->dtype == E3X_F32 && P->n_targets > 1 && P->weight_numel * 4 <= (1 << 20) &&
+          blocks * P->n_targets < (1LL << 31)) {
+        blocks = (blocks + 7) / 8 * 8 * P->n_targets;  // row tiles padded to the 8 XCDs
+        grid_y = 1;
+      }
     } else {
       const int groups = 64 / K->lanes;
       const long long items = (Z + groups - 1) / groups * K->chunks;
