@@ -265,10 +265,11 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src) {
 int build_uvw_small_source(e3x_plan& P, SubKernel& K, std::string* src) {
   int max_mul = 1;
   std::vector<char> usedo(P.out.size(), 0);
+  bool all_uvw = true;
   for (const auto& p : P.paths) {
-    if (!p.has_w) return fail(E3X_ERR_INVALID, "uvw instruction must have weights");
     usedo[p.out] = 1;
     max_mul = std::max(max_mul, P.out[p.out].mul);
+    all_uvw = all_uvw && p.mode == E3X_MODE_UVW;
   }
   K.lanes = max_mul > 32 ? 64 : pow2_at_least(max_mul, 16);
   // long input rows: fewer rows per wavefront so that the staged rows fit in LDS (lanes beyond the output
@@ -294,20 +295,20 @@ int build_uvw_small_source(e3x_plan& P, SubKernel& K, std::string* src) {
   // shared weights of few (u, v) pairs live in registers, one per pair and lane (one chunk of output channels only)
   long long pairs = 0;
   for (const auto& p : P.paths) pairs += (long long)P.in1[p.in1].mul * P.in2[p.in2].mul;
-  const bool cached = P.shared_weights && K.chunks == 1 && pairs > 0 && pairs <= 64;
+  const bool cached = all_uvw && P.shared_weights && K.chunks == 1 && pairs > 0 && pairs <= 64;
   K.cached_weights = cached;
   s << "constexpr int W_CACHE_REGS = " << (cached ? pairs : 0) << ";\n";
-  s << "struct Path { int x1off, d1, U, x2off, d2, V, out, woff, wreg; int nz_beg, nz_end; };\n";
+  s << "struct Path { int x1off, d1, U, x2off, d2, V, out, woff, wreg, mode; bool has_w; int nz_beg, nz_end; };\n";
   s << "constexpr int N_PATH = " << P.paths.size() << ";\nconstexpr Path paths[N_PATH > 0 ? N_PATH : 1] = {\n";
   int wreg = 0;
   for (size_t i = 0; i < P.paths.size(); ++i) {
     const auto& p = P.paths[i];
     s << "  {" << P.off1[p.in1] << ", " << 2 * P.in1[p.in1].l + 1 << ", " << P.in1[p.in1].mul << ", " << P.off2[p.in2]
       << ", " << 2 * P.in2[p.in2].l + 1 << ", " << P.in2[p.in2].mul << ", " << p.out << ", " << p.woff << ", " << wreg
-      << ", " << L.beg[i] << ", " << L.end[i] << "},\n";
+      << ", " << p.mode << ", " << (p.has_w ? "true" : "false") << ", " << L.beg[i] << ", " << L.end[i] << "},\n";
     wreg += P.in1[p.in1].mul * P.in2[p.in2].mul;
   }
-  if (P.paths.empty()) s << "  {0, 1, 0, 0, 1, 0, 0, 0, 0, 0, 0}\n";
+  if (P.paths.empty()) s << "  {0, 1, 0, 0, 1, 0, 0, 0, 0, 0, false, 0, 0}\n";
   s << "};\n";
   emit_nz_table(s, L);
   s << "}  // namespace cfg\n";
@@ -561,7 +562,7 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
   if ((rc = take(d->in2, d->n_in2, P->in2, P->off2, P->in2_dim))) return rc;
   if ((rc = take(d->out, d->n_out, P->out, P->offo, P->out_dim))) return rc;
 
-  int n_uvu = 0, n_uvw = 0;
+  int n_uvu = 0, n_uvw = 0, n_other = 0;
   std::vector<char> reached(P->out.size(), 0);
   int64_t woff = 0;
   for (int t = 0; t < d->n_ins; ++t) {
@@ -572,15 +573,31 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
     // selection rules (reference _tensor_product.py:294-295)
     if (a.p * b.p != c.p || c.l < std::abs(a.l - b.l) || c.l > a.l + b.l)
       return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: instruction violates the selection rules");
-    if (I.mode != E3X_MODE_UVU && I.mode != E3X_MODE_UVW)
-      return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: only the uvu and uvw connection modes are implemented");
-    if (I.mode == E3X_MODE_UVW && !I.has_weight) return fail(E3X_ERR_INVALID, "uvw instruction must have weights");
-    const int64_t n_w = I.mode == E3X_MODE_UVU ? (int64_t)a.mul * b.mul : (int64_t)a.mul * b.mul * c.mul;
+    if (I.mode < E3X_MODE_UVW || I.mode > E3X_MODE_U_LT_VW)
+      return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: unknown connection mode");
+    // weight block shapes and multiplicity constraints of the connection modes (reference _tensor_product.py:236-262)
+    const int64_t U = a.mul, V = b.mul, W = c.mul;
+    int64_t n_w = 0;
+    bool shape_ok = true, need_w = false;
+    switch (I.mode) {
+      case E3X_MODE_UVW: n_w = U * V * W, need_w = true; break;
+      case E3X_MODE_UVU: n_w = U * V, shape_ok = U == W; break;
+      case E3X_MODE_UVV: n_w = U * V, shape_ok = V == W; break;
+      case E3X_MODE_UUW: n_w = U * W, shape_ok = U == V && (I.has_weight || W == 1); break;
+      case E3X_MODE_UUU: n_w = U, shape_ok = U == V && V == W; break;
+      case E3X_MODE_UVUV: n_w = U * V, shape_ok = W == U * V; break;
+      case E3X_MODE_UVU_LT_V: n_w = U * (U - 1) / 2, shape_ok = U == V && W == U * (U - 1) / 2; break;
+      default: n_w = U * (U - 1) / 2 * W, shape_ok = U == V, need_w = true; break;
+    }
+    if (!shape_ok) return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: multiplicities do not fit the connection mode");
+    if (need_w && !I.has_weight) return fail(E3X_ERR_INVALID, "uvw and u<vw instructions must have weights");
     const bool empty = a.mul == 0 || b.mul == 0 || c.mul == 0;  // dropped, reference _codegen.py:51
     if (!empty) {
       PathInfo p{I.i_in1, I.i_in2, I.i_out, I.mode, I.has_weight ? 1 : 0, I.path_weight, (int)woff};
       P->paths.push_back(p);
-      (I.mode == E3X_MODE_UVU ? n_uvu : n_uvw)++;
+      if (I.mode == E3X_MODE_UVU) ++n_uvu;
+      else if (I.mode == E3X_MODE_UVW) ++n_uvw;
+      else ++n_other;
       reached[I.i_out] = 1;
     }
     if (I.has_weight && !empty) woff += n_w;
@@ -589,13 +606,16 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
   P->weight_numel = woff;
   for (size_t c = 0; c < P->out.size(); ++c)
     if (!reached[c] && dim_of(P->out[c]) > 0) P->zero_fill = true;
-  if (n_uvu && n_uvw)
-    return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: mixing uvu and uvw instructions in one plan is not implemented");
+  // all-uvu and all-uvw instruction sets have their own kernel families; every other set (the six remaining
+  // connection modes, or a mixture) takes the general vector-ALU kernel
+  const bool general = n_other > 0 || (n_uvu > 0 && n_uvw > 0);
+  if (general && d->dtype != E3X_F32)
+    return fail(E3X_ERR_INVALID, "e3x_tp_plan_create: connection modes other than uvu / uvw are fp32 only");
 
   const char* force_small = std::getenv("E3X_UVW_FORCE_VALU");
   std::vector<std::vector<int>> parts;
-  if (n_uvw) {
-    P->family = (uvw_mfma_eligible(*P) && !(force_small && force_small[0] == '1')) ? "uvw_mfma" : "uvw_small";
+  if (n_uvw || general) {
+    P->family = (!general && uvw_mfma_eligible(*P) && !(force_small && force_small[0] == '1')) ? "uvw_mfma" : "uvw_small";
     std::vector<int> all(P->paths.size());
     for (size_t i = 0; i < all.size(); ++i) all[i] = (int)i;
     parts.push_back(all);

@@ -28,7 +28,7 @@ Instruction = namedtuple(
 )
 
 _MODES = ["uvw", "uvu", "uvv", "uuw", "uuu", "uvuv", "uvu<v", "u<vw"]
-_KERNEL_MODES = {"uvw": _lib.MODE_UVW, "uvu": _lib.MODE_UVU}
+_KERNEL_MODES = {"uvw": 0, "uvu": 1, "uvv": 2, "uuw": 3, "uuu": 4, "uvuv": 5, "uvu<v": 6, "u<vw": 7}  # E3X_MODE_*
 _DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}
 
 
@@ -202,6 +202,10 @@ class _TensorProductFn(torch.autograd.Function):
                 g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, _permuted_weights(tp, w, (2, 1, 0)))
             if need2:
                 g2 = tp._grad_plan("x2", x1.dtype).forward(x1, g, _permuted_weights(tp, w, (0, 2, 1)))
+        elif mode == "general":
+            raise NotImplementedError(
+                "tensor products with connection modes other than pure uvu / pure uvw have a forward kernel only"
+            )
         else:
             g1, g2 = torch.zeros_like(x1), torch.zeros_like(x2)
             gw = torch.zeros_like(w) if needw else None
@@ -333,17 +337,10 @@ class TensorProduct(torch.nn.Module):
         self._compile_left_right = compile_left_right
 
         for t in self.instructions:
-            if t.connection_mode not in _KERNEL_MODES:
-                raise NotImplementedError(
-                    f"connection mode '{t.connection_mode}' has no HIP kernel; implemented modes: uvu, uvw"
-                )
             if t.connection_mode == "uvu":
                 assert i1[t.i_in1].mul == io[t.i_out].mul
-            if t.connection_mode == "uvw":
+            if t.connection_mode in ("uvw", "u<vw"):
                 assert t.has_weight
-        live = {t.connection_mode for t in self.instructions if 0 not in t.path_shape}
-        if len(live) > 1:
-            raise NotImplementedError("mixing uvu and uvw instructions in one TensorProduct has no HIP kernel")
 
         self.weight_numel = sum(prod(t.path_shape) for t in self.instructions if t.has_weight)
         if internal_weights and self.weight_numel > 0:
@@ -371,8 +368,11 @@ class TensorProduct(torch.nn.Module):
         return [(t.i_in1, t.i_in2, t.i_out, t.connection_mode, t.has_weight, t.path_weight) for t in self.instructions]
 
     def _live_mode(self):
+        """"uvu" / "uvw" for the two families with backward kernels, "general" for anything else, None if empty."""
         live = {t.connection_mode for t in self.instructions if 0 not in t.path_shape}
-        return next(iter(live)) if live else None
+        if not live:
+            return None
+        return next(iter(live)) if len(live) == 1 and live <= {"uvu", "uvw"} else "general"
 
     def _plan(self, dtype: torch.dtype) -> _Plan:
         if dtype not in _DTYPES:
@@ -417,6 +417,8 @@ class TensorProduct(torch.nn.Module):
     def compile_backward(self, dtype: torch.dtype = torch.float32) -> "TensorProduct":
         """Also builds the transposed plans the backward pass uses."""
         self._plan(dtype)
+        if self._live_mode() == "general":
+            return self  # forward kernel only
         self._grad_plan("x1", dtype)
         if self._live_mode() == "uvw":
             self._grad_plan("x2", dtype)

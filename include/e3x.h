@@ -35,6 +35,12 @@ extern "C" {
 /* connection modes (reference _tensor_product.py:245-254) */
 #define E3X_MODE_UVW 0
 #define E3X_MODE_UVU 1
+#define E3X_MODE_UVV 2
+#define E3X_MODE_UUW 3
+#define E3X_MODE_UUU 4
+#define E3X_MODE_UVUV 5
+#define E3X_MODE_UVU_LT_V 6 /* "uvu<v" */
+#define E3X_MODE_U_LT_VW 7  /* "u<vw" */
 
 /* spherical-harmonics output normalisation (reference _spherical_harmonics.py:103-110) */
 #define E3X_NORM_INTEGRAL 0

@@ -20,7 +20,7 @@ GOLDEN_GPU_CASES = [
     "fctp_cfg1", "fctp_small_cfg5_like", "fctp_per_sample_weights", "fctp_norm_path",
     "uvu_merged_cfg3_like_mul4", "uvu_builder_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2",
     "uvu_builderB_cfg4_like_mul2", "uvu_shared_v2", "uvu_mixed_weightless", "empty_path_and_missing_output",
-    "conv_small",
+    "modes_uuu_uvuv_uuw_uvv", "modes_triangular", "conv_small",
 ]  # fmt: skip
 
 
@@ -86,6 +86,13 @@ def radial_layer():
     return o3.FullyConnectedTensorProduct("64x0e", "0e", "352x0e")
 
 
+def mixed_modes():
+    # uvu and uvw paths into the same output irrep plus an elementwise and an unweighted path: the general kernel
+    ins = [(0, 0, 0, "uvu", True), (1, 1, 0, "uvw", True), (1, 0, 1, "uvu", False), (1, 1, 2, "uvv", True),
+           (0, 0, 3, "uuu", True), (1, 2, 4, "uuw", False)]  # fmt: skip
+    return o3.TensorProduct("4x0e+4x1o", "4x0e+3x1o+4x1e", "4x0e+4x1o+3x1e+4x0e+1x0o", ins, shared_weights=False)
+
+
 def scalar_exact():
     # 1x1 Clebsch-Gordan, path weight 1: products and sums of small integers are exact in fp32
     return message_tensor_product("32x0e", "0e", irreps_out="32x0e")
@@ -110,6 +117,7 @@ def all_tensor_products():
         ("mfma_small", mfma_small(), (torch.float32,)),
         ("node_fctp", node_fctp(), (torch.float32,)),
         ("radial_layer", radial_layer(), (torch.float32,)),
+        ("mixed_modes", mixed_modes(), (torch.float32,)),
         ("scalar_exact", scalar_exact(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),
     ]

@@ -41,6 +41,18 @@ def test_matches_reference_golden(golden_tp, name):
             assert (tp.output_mask[sl] == flag).all()
 
 
+def test_general_connection_modes_against_oracle():
+    # uvu + uvw + uvv + uuu + uuw (unweighted) in one instruction set, per-sample weights
+    tp = ks.mixed_modes()
+    x1, x2 = seeded(37, tp.irreps_in1.dim, seed=1), seeded(37, tp.irreps_in2.dim, seed=2)
+    w = seeded(37, tp.weight_numel, seed=3)
+    out = tp(x1.to(DEV), x2.to(DEV), w.to(DEV))
+    ref = otp.tp_forward(oracle_spec(tp), x1.numpy(), x2.numpy(), w.numpy())
+    assert_close(out, ref, what="mixed modes")
+    with pytest.raises(NotImplementedError):  # forward kernel only
+        tp(x1.to(DEV).requires_grad_(True), x2.to(DEV), w.to(DEV)).sum().backward()
+
+
 def test_cfg1_full_size_against_oracle():
     # FCTP('16x0e+16x1o', '0e+1o+2e' -> '16x0e+16x1o+16x2e'), batch 4096, x2 = SH(lmax 2) of unit vectors, seed 0
     g = torch.Generator().manual_seed(0)

@@ -131,8 +131,11 @@ def test_module_state_and_api_details():
         o3.TensorProduct("1o", "1o", "3e", [(0, 0, 0, "uvu", True)])
     with pytest.raises(AssertionError):
         o3.TensorProduct("1o", "1o", "1e", [(0, 0, 0, "uvu", True)], internal_weights=True, shared_weights=False)
+    # every connection mode of the reference builds a plan (the general vector-ALU kernel family)
+    tp = o3.TensorProduct("2x1o", "2x1o", "2x1e", [(0, 0, 0, "uuu", True)])
+    assert tp.weight_numel == 2 and tp._plan(torch.float32).family == "uvw_small"
     with pytest.raises(NotImplementedError):
-        o3.TensorProduct("2x1o", "2x1o", "2x1e", [(0, 0, 0, "uuu", True)])
+        o3.TensorProduct("2x1o", "2x1o", "2x1e", [(0, 0, 0, "uuu", True)], compile_right=True)
     set_optimization_defaults(specialized_code=False)
     assert get_optimization_defaults()["specialized_code"] is False
     set_optimization_defaults(specialized_code=True)
