@@ -780,8 +780,8 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
                                     int64_t E, int64_t num_src_nodes, int64_t num_out_nodes, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: null plan");
   if (P->family != "uvu") return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: the plan must be all-uvu");
-  if (P->shared_weights && P->weight_numel && grad_w)
-    return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: the gradient of shared weights is not implemented");
+  if (P->shared_weights && P->weight_numel && grad_w && P->dtype != E3X_F32)
+    return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: the gradient of shared weights is fp32 only");
   if (idx_bits != 32 && idx_bits != 64) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: idx_bits must be 32 or 64");
   if (E < 0 || num_src_nodes < 0 || num_out_nodes < 0) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: negative size");
   if ((src == nullptr) != (dst == nullptr))
@@ -809,7 +809,9 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
     if ((rc = e3x::fill_zero_bytes(grad_x2, (size_t)E * P->in2_dim * esz, st))) return rc;
   }
   // weights of paths with an unused multiplicity tail and unweighted paths are never written: start from zero
-  if (grad_w && P->weight_numel && (rc = e3x::fill_zero_bytes(grad_w, (size_t)E * P->weight_numel * esz, st))) return rc;
+  if (grad_w && P->weight_numel &&
+      (rc = e3x::fill_zero_bytes(grad_w, (size_t)(P->shared_weights ? 1 : E) * P->weight_numel * esz, st)))
+    return rc;
   int idx64 = idx_bits == 64;
   long long n_edges = E, n_src = num_src_nodes;
   void* args[] = {(void*)&x1,  (void*)&x2,     (void*)&w,       (void*)&grad_out,  (void*)&src,     (void*)&dst,

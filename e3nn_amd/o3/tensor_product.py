@@ -76,6 +76,7 @@ class _Plan:
         handle = _lib.c_void_p()
         _lib.check(L.e3x_tp_plan_create(ctypes.byref(desc), ctypes.byref(handle)))
         self.handle = handle
+        self.shared_weights = bool(shared_weights)
         wn, fam, key = ctypes.c_int64(), ctypes.c_char_p(), ctypes.c_char_p()
         _lib.check(L.e3x_tp_plan_info(handle, ctypes.byref(wn), None, None, None, ctypes.byref(fam), ctypes.byref(key)))
         self.weight_numel, self.family, self.key = wn.value, fam.value.decode(), key.value.decode()
@@ -135,7 +136,8 @@ class _Plan:
         return gw
 
     def backward_w_x2(self, x1, x2, w, grad_out, src, dst, want_w, want_x2, num_edges):
-        gw = torch.empty(num_edges, self.weight_numel, dtype=x1.dtype, device=x1.device) if want_w else None
+        gw_shape = (self.weight_numel,) if self.shared_weights else (num_edges, self.weight_numel)
+        gw = torch.empty(gw_shape, dtype=x1.dtype, device=x1.device) if want_w else None
         gx2 = torch.empty(num_edges, x2.shape[1], dtype=x1.dtype, device=x1.device) if want_x2 else None
         bits = src.element_size() * 8 if src is not None else 64
         with torch.cuda.device(x1.device):
@@ -187,8 +189,8 @@ class _TensorProductFn(torch.autograd.Function):
             if need1:
                 g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, w)
             if need2 or (needw and tp.weight_numel):
-                if tp.shared_weights and needw and tp.weight_numel:
-                    raise NotImplementedError("the gradient of shared uvu weights has no kernel")
+                if tp.shared_weights and needw and tp.weight_numel and x1.dtype != torch.float32:
+                    raise NotImplementedError("the gradient of shared uvu weights has an fp32 kernel only")
                 gw, g2 = tp._plan(x1.dtype).backward_w_x2(x1, x2, w, g, None, None, needw and tp.weight_numel > 0, need2, x1.shape[0])
         elif mode == "uvw":
             if needw and tp.weight_numel:
@@ -243,8 +245,8 @@ class TensorProduct(torch.nn.Module):
     r"""Tensor product with parametrised paths (see the reference docstring, ``_tensor_product.py:25-194``).
 
     ``instructions`` is a list of ``(i_in1, i_in2, i_out, mode, has_weight[, path_weight])``.
-    Only the ``uvu`` and ``uvw`` connection modes have kernels; other modes raise
-    ``NotImplementedError`` at construction.
+    All-``uvu`` and all-``uvw`` instruction sets have dedicated kernels with a backward pass; every other
+    connection mode (and mixtures) runs forward on the general vector-ALU kernel.
     """
 
     def __init__(

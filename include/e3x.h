@@ -156,12 +156,13 @@ int e3x_tp_gather_scatter(e3x_plan* plan, const void* node_x, const void* edge_a
 
 /* Gradients of the `uvu` product (plain: src = dst = NULL, row e of every table; fused: the edge lists
  * of e3x_tp_gather_scatter, unsorted) with respect to the per-sample weights and the second input:
- *   grad_w[E, weight_numel], grad_x2[E, in2_dim]  from  grad_out[num_out_nodes, out_dim].
+ *   grad_w[E, weight_numel] (shared weights: one [weight_numel] vector summed over the edges with fp32 atomics),
+ *   grad_x2[E, in2_dim]  from  grad_out[num_out_nodes, out_dim].
  * Either output may be NULL.  The reference obtains these by autograd through the einsums of
  * e3nn/o3/_tensor_product/_codegen.py:166-187.  The gradient with respect to the first input is the
  * forward entry point applied to a transposed plan (inputs grad_out and x2, output irreps_in1, same
  * weights) with source and destination exchanged; no separate entry point is needed for it.
- * Only for all-`uvu` plans with per-sample weights; bf16 storage only for plans of a single kernel. */
+ * Only for all-`uvu` plans; bf16 storage only for per-sample weights and plans of a single kernel. */
 int e3x_tp_backward_w_x2(e3x_plan* plan, const void* x1, const void* x2, const void* w, const void* grad_out,
                          const void* src, const void* dst, int idx_bits, void* grad_w, void* grad_x2, int64_t E,
                          int64_t num_src_nodes, int64_t num_out_nodes, void* stream);

@@ -112,13 +112,27 @@ def test_internal_weights_train():
     assert tp.weight.grad is not None and tp.weight.grad.shape == tp.weight.shape and bool(tp.weight.grad.abs().sum() > 0)
 
 
-def test_missing_backward_kernels_fail_loudly():
-    # shared uvu weights have no gradient kernel: the call must raise, not fall back
+def test_shared_uvu_weight_gradient():
     tp = ks.golden_tp("uvu_shared_v2").to(DEV)
     assert tp.shared_weights and tp.weight_numel
-    x1, x2 = seeded(4, tp.irreps_in1.dim).to(DEV), seeded(4, tp.irreps_in2.dim).to(DEV)
-    w = seeded(tp.weight_numel).to(DEV).requires_grad_(True)
-    out = tp(x1, x2, w)
+    spec = oracle_spec(tp)
+    Z = 300
+    x1, x2, w = seeded(Z, tp.irreps_in1.dim, seed=1), seeded(Z, tp.irreps_in2.dim, seed=2), seeded(tp.weight_numel, seed=3)
+    cot = seeded(Z, tp.irreps_out.dim, seed=4)
+    _, (r1, r2, rw) = _oracle_grads(lambda a, b, c: tp_forward_torch(spec, a, b, c), (x1, x2, w), cot)
+    a, b, c = (t.to(DEV).requires_grad_(True) for t in (x1, x2, w))
+    tp(a, b, c).backward(cot.to(DEV))
+    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
+    assert_close(c.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dw (shared)")
+    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dx1")
+    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
+
+
+def test_missing_backward_kernels_fail_loudly():
+    # connection modes outside pure uvu / pure uvw have a forward kernel only: the call must raise, not fall back
+    tp = ks.mixed_modes()
+    x1 = seeded(4, tp.irreps_in1.dim).to(DEV).requires_grad_(True)
+    out = tp(x1, seeded(4, tp.irreps_in2.dim).to(DEV), seeded(4, tp.weight_numel).to(DEV))
     with pytest.raises(NotImplementedError):
         out.sum().backward()
 
