@@ -4,6 +4,7 @@
 // hand-written device template.  The code object is compiled once with the system HIP
 // compiler and kept under the cache directory, keyed by a hash of the full source text
 // and the compiler flags, so identical instruction sets never compile twice.
+#include <atomic>
 #include <dlfcn.h>
 #include <fcntl.h>
 #include <spawn.h>
@@ -77,10 +78,13 @@ int get_code_object(const std::string& family, const std::string& source, std::s
       return fail(E3X_ERR_COMPILE, "kernel " + std::string(key) + " is not in the cache (" + dir +
                                        ") and E3X_NO_JIT=1 forbids compiling it");
   ::mkdir(dir.c_str(), 0755);
-  const std::string src_path = base + ".hip", log_path = base + ".log";
-  char tmp_name[64];
-  std::snprintf(tmp_name, sizeof(tmp_name), ".tmp%d.hsaco", (int)getpid());
-  const std::string tmp_path = base + tmp_name;
+  // Threads and processes may build the same kernel at the same time: each works on files of its own and moves
+  // the results into place at the end (rename is atomic; the contents are identical whoever wins).
+  static std::atomic<unsigned> serial{0};
+  char tag[64];
+  std::snprintf(tag, sizeof(tag), ".tmp%d_%u", (int)getpid(), serial.fetch_add(1));
+  const std::string final_src = base + ".hip";
+  const std::string src_path = base + tag + ".hip", log_path = base + tag + ".log", tmp_path = base + tag + ".hsaco";
   {
     std::ofstream f(src_path);
     if (!f) return fail(E3X_ERR_COMPILE, "cannot write " + src_path);
@@ -114,11 +118,15 @@ int get_code_object(const std::string& family, const std::string& source, std::s
     ss << lf.rdbuf();
     std::string log = ss.str();
     if (log.size() > 2000) log = log.substr(0, 2000) + "...";
-    return fail(E3X_ERR_COMPILE, "compiling " + src_path + " failed:\n" + log);
+    std::rename(src_path.c_str(), final_src.c_str());  // keep the source that failed next to its key
+    std::remove(log_path.c_str());
+    std::remove(tmp_path.c_str());
+    return fail(E3X_ERR_COMPILE, "compiling " + final_src + " failed:\n" + log);
   }
+  std::rename(src_path.c_str(), final_src.c_str());
+  std::remove(log_path.c_str());
   if (std::rename(tmp_path.c_str(), path_out->c_str()) != 0)
     return fail(E3X_ERR_COMPILE, "cannot move the code object into the cache");
-  std::remove(log_path.c_str());
   return E3X_OK;
 }
 

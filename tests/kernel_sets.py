@@ -163,17 +163,27 @@ def conv_wide():
     return nn.Convolution(f, "4x0e", SH2, f, [8, 64], 37.5)
 
 
-def prebuild(verbose=True):
+def prebuild(verbose=True, workers=6):
+    """Builds every kernel the tests and the benchmark use.  Plan creation spends its time in the HIP compiler (a child
+    process, the calling thread waits with the GIL released), so a few threads build several kernels at once."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    jobs = []
     for name, mod in nn_modules():
         for sub in mod.modules():
             if isinstance(sub, o3.TensorProduct):
-                sub.compile_backward(torch.float32)
-        if verbose:
-            print(f"module {name}", flush=True)
+                jobs.append((f"module {name}", sub, (torch.float32,), True))
     for name, tp, dtypes in all_tensor_products():
-        for dt in dtypes:
-            plan = tp._plan(dt)
-            if verbose:
-                print(f"kernel {name:32s} {str(dt):16s} {plan.key}", flush=True)
-        if name in BACKWARD_CASES:
+        jobs.append((f"kernel {name}", tp, dtypes, name in BACKWARD_CASES))
+
+    def build(job):
+        name, tp, dtypes, backward = job
+        keys = [tp._plan(dt).key for dt in dtypes]
+        if backward:
             tp.compile_backward(torch.float32)
+        return name, keys
+
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        for name, keys in pool.map(build, jobs):
+            if verbose:
+                print(f"{name:40s} {' '.join(keys)}", flush=True)
