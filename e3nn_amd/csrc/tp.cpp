@@ -808,9 +808,11 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
       return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: grad_x2 in bf16 storage needs a single-kernel plan");
     if ((rc = e3x::fill_zero_bytes(grad_x2, (size_t)E * P->in2_dim * esz, st))) return rc;
   }
-  // weights of paths with an unused multiplicity tail and unweighted paths are never written: start from zero
-  if (grad_w && P->weight_numel &&
-      (rc = e3x::fill_zero_bytes(grad_w, (size_t)(P->shared_weights ? 1 : E) * P->weight_numel * esz, st)))
+  // Per-sample weights: every weighted path belongs to exactly one kernel of the plan and every multiplicity index
+  // to exactly one lane, so each element of grad_w[E, weight_numel] is stored exactly once -- no zero fill (it would
+  // be a second pass over the largest tensor of the call).  Shared weights are accumulated with atomics from zero.
+  if (grad_w && P->weight_numel && P->shared_weights &&
+      (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * esz, st)))
     return rc;
   int idx64 = idx_bits == 64;
   long long n_edges = E, n_src = num_src_nodes;

@@ -32,6 +32,10 @@ def test_uvu_plain_gradients(maker, Z):
     ref_out, (r1, r2, rw) = _oracle_grads(lambda a, b, c: tp_forward_torch(spec, a, b, c), (x1, x2, w), cot)
     a, b, c = (t.to(DEV).requires_grad_(True) for t in (x1, x2, w))
     out = tp(a, b, c)
+    # the weight gradient is written without a zero fill: hand the allocator a NaN-filled block of its size first,
+    # so that an element the kernel skipped would show
+    junk = torch.full((Z, tp.weight_numel), float("nan"), device=DEV)
+    del junk
     out.backward(cot.to(DEV))
     scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
     assert_close(out, ref_out.numpy(), atol=1e-4 * scale(ref_out))
@@ -53,6 +57,8 @@ def test_fused_message_gradients(maker, N, E, idx):
     a, b, c = (t.to(DEV).requires_grad_(True) for t in (node_x, attr, w))
     edges = DstSortedEdges(src.to(idx).to(DEV), dst.to(idx).to(DEV), N)
     out = tp.forward_gather_scatter(a, b, c, edges=edges)
+    junk = torch.full((E, tp.weight_numel), float("nan"), device=DEV)  # see test_uvu_plain_gradients
+    del junk
     out.backward(cot.to(DEV))
     scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
     assert_close(out, ref_out.numpy(), atol=1e-4 * scale(ref_out))
