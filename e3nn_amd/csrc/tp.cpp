@@ -881,7 +881,10 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   }
   if (P->shared_weights && (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st))) return rc;
   if ((rc = load_functions(P, dev))) return rc;
-  const long long wblocks = (P->weight_numel + 255) / 256;
+  // one thread per (path, v, w) column of the weight blocks
+  long long cols = 0;
+  for (const auto& q : P->paths) cols += (long long)P->in2[q.in2].mul * P->out[q.out].mul;
+  const long long wblocks = (cols + 255) / 256;
   // enough batch slices to fill the chip a few times over, at least 16 rows each
   long long slices = (4096 + wblocks - 1) / wblocks;
   if (slices > (Z + 15) / 16) slices = (Z + 15) / 16;
