@@ -80,6 +80,11 @@ def node_fctp():
     return o3.FullyConnectedTensorProduct("128x0e+64x1o+32x2e", "4x0e", "128x0e+64x1o+96x2e")
 
 
+def wide_k():
+    # GEMM K extents above 128 (256 and 160): the K operand is resident in LDS in blocks of 128, restaged per outer index
+    return o3.FullyConnectedTensorProduct("256x0e+160x1o", "32x0e+32x1o", "64x0e+64x1o")
+
+
 def radial_layer():
     # one dense layer of a radial network written as a tensor product of scalars: 64 -> 352 (= 5.5 tiles of 64
     # channels: the last tile is half full), second input "0e"
@@ -117,6 +122,7 @@ def all_tensor_products():
         ("mfma_small", mfma_small(), (torch.float32,)),
         ("node_fctp", node_fctp(), (torch.float32,)),
         ("radial_layer", radial_layer(), (torch.float32,)),
+        ("wide_k", wide_k(), (torch.float32,)),
         ("mixed_modes", mixed_modes(), (torch.float32,)),
         ("scalar_exact", scalar_exact(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),

@@ -167,7 +167,7 @@ def _fan_in_weights(tp, seed=0):
     return w
 
 
-@pytest.mark.parametrize("maker,Z", [(ks.mfma_small, 150), (ks.cfg5, 70), (ks.node_fctp, 333), (ks.radial_layer, 1000)])
+@pytest.mark.parametrize("maker,Z", [(ks.mfma_small, 150), (ks.cfg5, 70), (ks.node_fctp, 333), (ks.radial_layer, 1000), (ks.wide_k, 130)])
 def test_uvw_matrix_core_kernel_against_oracle(maker, Z):
     tp = maker().to(DEV)
     assert tp._plan(torch.float32).family == "uvw_mfma"
