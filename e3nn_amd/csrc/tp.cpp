@@ -352,6 +352,8 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   std::ostringstream s, nzs, ps, ts;
   emit_header(s, P);
   if (P.dtype == E3X_F32) s << "#define E3X_UVW_KC " << env_int("E3X_UVW_KC", 32) << "\n";
+  if (env_int("E3X_UVW_KS", 0)) s << "#define E3X_UVW_KS " << env_int("E3X_UVW_KS", 0) << "\n";
+  if (env_int("E3X_UVW_WPE", 0)) s << "#define E3X_UVW_WPE " << env_int("E3X_UVW_WPE", 0) << "\n";
   int n_nz = 0, n_path = 0, n_target = 0, dka = 1, drmax = 1;
   for (size_t c = 0; c < P.out.size(); ++c) {
     std::ostringstream mine;
