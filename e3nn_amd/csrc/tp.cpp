@@ -869,7 +869,7 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
     slices = std::min(slices, (long long)((Z + 255) / 256));
     slices = std::max(1LL, std::min(slices, 1024LL));
     long long rows_per_slice = (Z + slices - 1) / slices;
-    rows_per_slice = (rows_per_slice + 31) / 32 * 32;
+    rows_per_slice = (rows_per_slice + 23) / 24 * 24;  // whole chunks of the kernel
     slices = (Z + rows_per_slice - 1) / rows_per_slice;
     int accumulate = slices > 1;
     if (accumulate && (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st))) return rc;
