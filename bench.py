@@ -300,6 +300,32 @@ def bench_convolution(args, dev, ctx):
     return {"edges": E, "nodes": N, "ms_forward": ms_f, "ms_forward_backward": ms_fb, "edges_per_s_forward": E / (ms_f * 1e-3)}
 
 
+def bench_radial_network(args, dev, ctx):
+    """The radial network of the block above, 8 -> 64 -> 352 with SiLU (reference e3nn/nn/_fc.py:38-48,70-88), on all
+    edges of the headline graph: as ONE kernel (no gradient wanted) and layer by layer (the path that has a backward)."""
+    from e3nn_amd.nn import FullyConnectedNet
+
+    E = ctx["src"].shape[0]
+    net = FullyConnectedNet([8, 64, 352], torch.nn.functional.silu).to(dev)
+    x = torch.randn(E, 8, generator=torch.Generator().manual_seed(0)).to(dev)
+
+    def one_kernel():
+        with torch.no_grad():
+            return net(x)
+
+    def layered():
+        return net(x)  # parameters require a gradient: tensor-product and gate kernels, one pair per layer
+
+    assert net.fused_plan().handle is not None
+    ms1 = event_time_ms(one_kernel, max(5, args.steps // 2), 3)
+    msl = event_time_ms(layered, max(5, args.steps // 5), 2)
+    flop = 2.0 * E * (8 * 64 + 64 * 352)
+    out_bytes = E * (8 + 352) * 4
+    return {"edges": E, "ms_one_kernel": ms1, "ms_layer_by_layer": msl, "tflops_one_kernel": flop / (ms1 * 1e-3) / 1e12,
+            "frac_fp32_mfma_peak": flop / (ms1 * 1e-3) / 1e12 / 157.3, "hbm_gbs_one_kernel": out_bytes / (ms1 * 1e-3) / 1e9,
+            "frac_hbm_peak": out_bytes / (ms1 * 1e-3) / 1e9 / HBM_PEAK_GBS}  # fmt: skip
+
+
 def bench_library_gemm(args, dev):
     """Context for the matrix-core rooflines: what the vendor GEMM (torch.matmul -> rocBLAS / hipBLASLt) reaches
     on this GPU with N(0,1) data, 8192^3."""
@@ -367,7 +393,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--locality-variants", action="store_true", help="also time the headline graph with sorted edges / Morton node ids")
-    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_b,mace_bf16,nequip40,uvw,uvw_bf16,conv,nequip_bwd,uvw_bwd (default: all)")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_b,mace_bf16,nequip40,uvw,uvw_bf16,conv,radial,nequip_bwd,uvw_bwd (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported (no collectives, no sharding)")
@@ -378,7 +404,7 @@ def main():
 
     neq, ctx = bench_nequip(args, dev)
     other = {"nequip_uvu": neq}
-    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_b", "mace_bf16", "nequip40", "uvw", "uvw_bf16", "conv", "nequip_bwd", "uvw_bwd"}
+    want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_b", "mace_bf16", "nequip40", "uvw", "uvw_bf16", "conv", "radial", "nequip_bwd", "uvw_bwd"}
     if "copy" in want:
         other["copy_1GiB"] = bench_copy(args, dev)
     if "sh" in want:
@@ -399,6 +425,8 @@ def main():
         other["library_gemm_8192_randn"] = bench_library_gemm(args, dev)
     if "conv" in want:
         other["convolution_block"] = bench_convolution(args, dev, ctx)
+    if "radial" in want:
+        other["radial_network_8_64_352"] = bench_radial_network(args, dev, ctx)
     if "nequip_bwd" in want:
         other["nequip_uvu_forward_backward"] = bench_nequip_backward(args, dev, ctx)
     if "uvw_bwd" in want:

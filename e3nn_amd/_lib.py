@@ -15,6 +15,7 @@ F32, BF16 = 0, 1
 MODE_UVW, MODE_UVU = 0, 1
 NORM_INTEGRAL, NORM_COMPONENT, NORM_NORM = 0, 1, 2
 ERR_INDEX = -4
+ERR_INVALID = -1
 
 c_void_p, c_int, c_int32, c_int64, c_size_t = ctypes.c_void_p, ctypes.c_int, ctypes.c_int32, ctypes.c_int64, ctypes.c_size_t
 
@@ -60,6 +61,12 @@ _SIGNATURES = {
                                c_int32, c_void_p]),
     "e3x_sh_backward": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
                                 c_int32, c_void_p]),
+    "e3x_fc_plan_create": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, ctypes.c_double, c_int32, ctypes.c_double,
+                                   ctypes.c_double, c_int32, ctypes.POINTER(c_void_p)]),
+    "e3x_fc_plan_destroy": (c_int, [c_void_p]),
+    "e3x_fc_workspace_bytes": (c_size_t, [c_void_p]),
+    "e3x_fc_plan_key": (ctypes.c_char_p, [c_void_p]),
+    "e3x_fc_forward": (c_int, [c_void_p, c_void_p, ctypes.POINTER(c_void_p), c_void_p, c_int64, c_void_p, c_size_t, c_void_p]),
     "e3x_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
 }  # fmt: skip
 

@@ -1,0 +1,182 @@
+// Fused fully-connected network of scalars (the radial network of a convolution): plan creation,
+// emission of the constexpr tables that specialise templates/fc_mfma.inc, code-object loading, launches.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <memory>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "e3x_internal.h"
+#include "jit.h"
+
+namespace {
+constexpr int kMaxDevices = 64;
+constexpr int kMaxLayers = 8;
+// LDS the packed weights may take (the CU has 160 KB; leave room for the runtime's own use)
+constexpr int64_t kMaxPackedBytes = 150 * 1024;
+// widest hidden layer: its activations (RS x width / 2 registers) and the next layer's live together
+constexpr int kMaxHidden = 128;
+}  // namespace
+
+struct e3x_fc_plan {
+  std::vector<int> hs, hp;
+  int n_layers = 0, rows_per_wg = 0;
+  int64_t packed_numel = 0;
+  std::string key, hsaco;
+  std::mutex mu;
+  hipModule_t module[kMaxDevices] = {nullptr};
+  hipFunction_t fn_pack[kMaxDevices] = {nullptr};
+  hipFunction_t fn_fwd[kMaxDevices] = {nullptr};
+  int n_cu[kMaxDevices] = {0};
+};
+
+namespace {
+
+using e3x::fail;
+
+std::string fstr(double v) {
+  char buf[64];
+  std::snprintf(buf, sizeof(buf), "%.9ef", v);
+  return buf;
+}
+
+int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+int load_functions(e3x_fc_plan* P, int dev) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  if (P->module[dev]) return E3X_OK;
+  hipModule_t mod = nullptr;
+  hipError_t err = hipModuleLoad(&mod, P->hsaco.c_str());
+  if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + P->hsaco + ") failed: " + hipGetErrorString(err));
+  if (hipModuleGetFunction(&P->fn_pack[dev], mod, "e3x_fc_pack") != hipSuccess ||
+      hipModuleGetFunction(&P->fn_fwd[dev], mod, "e3x_fc_forward_k") != hipSuccess)
+    return fail(E3X_ERR_HIP, "kernels missing from " + P->hsaco);
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+  P->n_cu[dev] = n;
+  P->module[dev] = mod;
+  return E3X_OK;
+}
+
+}  // namespace
+
+extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act,
+                                  double variance_in, double variance_out, int32_t dtype, e3x_fc_plan** out) {
+  if (!hs || !out) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: null argument");
+  if (dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: only fp32 storage is implemented");
+  if (n_hs < 2 || n_hs - 1 > kMaxLayers) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: 1 to 8 layers");
+  if (act < E3X_ACT_IDENTITY || act > E3X_ACT_RELU) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: unknown activation");
+  if (!(variance_in > 0) || !(variance_out > 0)) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: variances must be positive");
+  const int NL = n_hs - 1;
+  std::unique_ptr<e3x_fc_plan> P(new e3x_fc_plan);
+  P->n_layers = NL;
+  for (int i = 0; i <= NL; ++i) {
+    if (hs[i] < 1 || hs[i] > (1 << 20)) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: bad layer width");
+    P->hs.push_back(hs[i]);
+    P->hp.push_back(round_up(hs[i], i == 0 ? 8 : 32));
+    if (i < NL && P->hp[i] > kMaxHidden)
+      return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: input and hidden widths are limited to 128 in the fused kernel");
+  }
+  for (int l = 0; l < NL; ++l) P->packed_numel += (int64_t)P->hp[l] * P->hp[l + 1];
+  if (P->packed_numel * 4 > kMaxPackedBytes)
+    return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: the weights of the network do not fit the LDS of a compute unit");
+
+  // e3nn/nn/_fc.py:70-88: every layer but the last is followed by act (unit second moment: cst * act) and has
+  // var_out = 1; the last has var_out = variance_out and act only with out_act.  _fc.py:38-48: with act,
+  // act(x @ W / sqrt(h_in var_in)) * sqrt(var_out); without, x @ W / sqrt(h_in var_in / var_out).
+  std::vector<double> wscale(NL);
+  std::vector<int> acts(NL);
+  double post_prev = 1.0, var_in = variance_in, out_post = 1.0;
+  for (int l = 0; l < NL; ++l) {
+    const bool last = l == NL - 1;
+    const double var_out = last ? variance_out : 1.0;
+    const bool has_act = act != E3X_ACT_IDENTITY && (!last || out_act);  // E3X_ACT_IDENTITY: act=None
+    acts[l] = has_act ? act : E3X_ACT_IDENTITY;
+    double post;
+    if (has_act) {
+      wscale[l] = post_prev / std::sqrt((double)hs[l] * var_in);
+      post = act_cst * std::sqrt(var_out);
+    } else {
+      wscale[l] = post_prev / std::sqrt((double)hs[l] * var_in / var_out);
+      post = 1.0;
+    }
+    if (last) out_post = post;
+    post_prev = post;
+    var_in = var_out;
+  }
+
+  // a wave carries 32 rs rows: the input and output activations of a hidden layer are live together
+  // (rs (hp[l] + hp[l+1]) / 2 registers) next to rs accumulator tiles of 16
+  int live = P->hp[NL - 1] / 2;
+  for (int l = 0; l + 1 < NL; ++l) live = std::max(live, (P->hp[l] + P->hp[l + 1]) / 2);
+  const int rs = 2 * live + 32 + 24 <= 224 ? 2 : 1;
+  P->rows_per_wg = 8 * 32 * rs;
+  std::ostringstream s;
+  s << "// generated: one fully-connected network\n#include <stdint.h>\nnamespace cfg {\n";
+  s << "constexpr int NL = " << NL << ";\nconstexpr int H[NL + 1] = {";
+  for (int i = 0; i <= NL; ++i) s << (i ? ", " : "") << P->hs[i];
+  s << "};\nconstexpr int HP[NL + 1] = {";
+  for (int i = 0; i <= NL; ++i) s << (i ? ", " : "") << P->hp[i];
+  s << "};\nconstexpr int ACT[NL] = {";
+  for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << acts[l];
+  s << "};\nconstexpr float WSCALE[NL] = {";
+  for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << fstr(wscale[l]);
+  s << "};\nconstexpr float OUT_POST = " << fstr(out_post) << ";\n";
+  s << "constexpr int RS = " << rs << ";\n}  // namespace cfg\n";
+  const std::string src = s.str() + e3x::kTplCommon + e3x::kTplFcMfma;
+  int rc = e3x::get_code_object("fc_mfma", src, &P->key, &P->hsaco);
+  if (rc) return rc;
+  *out = P.release();
+  return E3X_OK;
+}
+
+extern "C" int e3x_fc_plan_destroy(e3x_fc_plan* plan) {
+  delete plan;  // code objects stay loaded for the life of the process
+  return E3X_OK;
+}
+
+extern "C" size_t e3x_fc_workspace_bytes(const e3x_fc_plan* P) { return P ? (size_t)P->packed_numel * 4 : 0; }
+
+extern "C" const char* e3x_fc_plan_key(const e3x_fc_plan* P) { return P ? P->key.c_str() : ""; }
+
+extern "C" int e3x_fc_forward(e3x_fc_plan* P, const void* x, const void* const* weights, void* out, int64_t Z,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_fc_forward: null plan");
+  if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_fc_forward: negative batch");
+  if (Z == 0) return E3X_OK;
+  if (!x || !out || !weights || !workspace) return fail(E3X_ERR_INVALID, "e3x_fc_forward: null pointer");
+  if (workspace_bytes < (size_t)P->packed_numel * 4) return fail(E3X_ERR_INVALID, "e3x_fc_forward: workspace too small");
+  if (((uintptr_t)workspace & 15) || ((uintptr_t)x & 15))
+    return fail(E3X_ERR_INVALID, "e3x_fc_forward: x and workspace must be 16-byte aligned");
+  struct {
+    const void* w[8];
+  } ptrs = {};
+  for (int l = 0; l < P->n_layers; ++l) {
+    if (!weights[l]) return fail(E3X_ERR_INVALID, "e3x_fc_forward: null weight pointer");
+    ptrs.w[l] = weights[l];
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(E3X_ERR_HIP, "hipGetDevice failed");
+  int rc = load_functions(P, dev);
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  {
+    void* args[] = {&ptrs, &workspace};
+    hipError_t err = hipModuleLaunchKernel(P->fn_pack[dev], (unsigned)((P->packed_numel + 255) / 256), 1, 1, 256, 1, 1, 0, st,
+                                           args, nullptr);
+    if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_fc_forward: pack launch failed: ") + hipGetErrorString(err));
+  }
+  long long n_rows = Z;
+  long long tiles = (Z + P->rows_per_wg - 1) / P->rows_per_wg;
+  long long blocks = tiles < P->n_cu[dev] ? tiles : P->n_cu[dev];  // one persistent workgroup per compute unit
+  void* args[] = {&x, &workspace, &out, &n_rows};
+  hipError_t err = hipModuleLaunchKernel(P->fn_fwd[dev], (unsigned)blocks, 1, 1, 512, 1, 1, 0, st, args, nullptr);
+  if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_fc_forward: launch failed: ") + hipGetErrorString(err));
+  return E3X_OK;
+}

@@ -1,12 +1,20 @@
 """``nn.FullyConnectedNet`` (``e3nn/nn/_fc.py:9-88``): dense layers ``x @ W / sqrt(h_in)`` with a second-moment
-normalised activation.  A dense layer of scalars is the ``uvw`` tensor product ``h_in x0e (x) 0e -> h_out x0e``, so each
-layer runs on the tensor-product kernels (matrix cores when h_in and h_out are multiples of 32) and the activation on
-the gate kernel; parameter names and shapes (``layer{i}.weight [h_in, h_out]``) are the reference's.
+normalised activation; parameter names and shapes (``layer{i}.weight [h_in, h_out]``) are the reference's.
+
+Two device paths, both HIP kernels of this package:
+
+* no gradient wanted (inference, or nothing upstream requires one): the whole network runs as ONE kernel that
+  keeps the hidden activations in registers (``e3x_fc_forward``);
+* otherwise each layer is the ``uvw`` tensor product ``h_in x0e (x) 0e -> h_out x0e`` (matrix cores when h_in and
+  h_out are multiples of 32) followed by the gate kernel, which have backward passes.
 """
+import ctypes
+
 import torch
 
+from .. import _lib
 from ..o3.tensor_product import TensorProduct
-from .activation import Activation, activation_name
+from .activation import _KINDS, Activation, activation_name, second_moment_constant
 
 
 class _Layer(torch.nn.Module):
@@ -40,6 +48,53 @@ class _Layer(torch.nn.Module):
         return x
 
 
+class _FusedPlan:
+    """Handle of a fused-network plan of the library; ``None`` handle when the network is outside its limits."""
+
+    def __init__(self, hs, act_name, out_act, variance_in, variance_out) -> None:
+        self.handle = None
+        self.key = None
+        self.reason = None
+        self._args = (list(hs), act_name, out_act, variance_in, variance_out)
+        L = _lib.lib()
+        arr = (ctypes.c_int32 * len(hs))(*hs)
+        h = ctypes.c_void_p()
+        rc = L.e3x_fc_plan_create(
+            arr, len(hs), _KINDS[act_name], second_moment_constant(act_name), int(bool(out_act)), float(variance_in),
+            float(variance_out), 0, ctypes.byref(h),
+        )  # fmt: skip
+        if rc == _lib.ERR_INVALID:
+            self.reason = L.e3x_last_error().decode()  # outside the fused kernel's limits: layer by layer instead
+            return
+        _lib.check(rc)
+        self.handle = h
+        self.key = L.e3x_fc_plan_key(h).decode()
+        self.workspace_bytes = L.e3x_fc_workspace_bytes(h)
+
+    def __reduce__(self):  # copies and pickles rebuild the plan from its arguments
+        return (_FusedPlan, self._args)
+
+    def __del__(self):
+        if getattr(self, "handle", None) is not None:
+            try:
+                _lib.lib().e3x_fc_plan_destroy(self.handle)
+            except Exception:
+                pass
+
+    def forward(self, x, weights):
+        L = _lib.lib()
+        Z = x.shape[0]
+        out = torch.empty((Z, weights[-1].shape[1]), device=x.device, dtype=torch.float32)
+        ws = torch.empty(self.workspace_bytes, device=x.device, dtype=torch.uint8)
+        ptrs = (ctypes.c_void_p * len(weights))(*[w.data_ptr() for w in weights])
+        with torch.cuda.device(x.device):
+            _lib.check(
+                L.e3x_fc_forward(self.handle, _lib.ptr(x), ptrs, _lib.ptr(out), Z, _lib.ptr(ws), self.workspace_bytes,
+                                 _lib.stream_ptr(x.device))
+            )  # fmt: skip
+        return out
+
+
 class FullyConnectedNet(torch.nn.Sequential):
     r"""Fully-connected network ``hs[0] -> hs[1] -> ... -> hs[-1]``; ``act`` is normalised to unit second moment."""
 
@@ -56,6 +111,31 @@ class FullyConnectedNet(torch.nn.Sequential):
                 a = act
             setattr(self, f"layer{i}", _Layer(h1, h2, a, var_in, var_out))
             var_in = var_out
+        self._fused_args = (self.hs, activation_name(act), out_act, variance_in, variance_out)
+        self._fused = None
 
     def __repr__(self) -> str:
         return f"{self.__class__.__name__}{self.hs}"
+
+    def fused_plan(self):
+        """The one-kernel plan of this network (built on first use); its ``handle`` is None outside the kernel's limits."""
+        if self._fused is None:
+            self._fused = _FusedPlan(*self._fused_args) if len(self.hs) >= 2 else False
+        return self._fused
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        layers = list(self)
+        wants_grad = torch.is_grad_enabled() and (x.requires_grad or any(l.weight.requires_grad for l in layers))
+        if layers and not wants_grad and x.is_cuda and x.dtype == torch.float32 and x.shape[-1] == self.hs[0]:
+            plan = self.fused_plan()
+            if plan and plan.handle is not None:
+                lead = x.shape[:-1]
+                x2 = x.reshape(-1, self.hs[0]).contiguous()
+                if x2.data_ptr() % 16:
+                    x2 = x2.clone()
+                ws = [l.weight.detach().contiguous() for l in layers]
+                if all(w.is_cuda and w.dtype == torch.float32 for w in ws):
+                    return plan.forward(x2, ws).reshape(lead + (self.hs[-1],))
+        for layer in layers:
+            x = layer(x)
+        return x

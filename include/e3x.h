@@ -202,6 +202,29 @@ int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_
                       const void* grad_out, void* grad_x, int64_t Z, int64_t in_dim, int64_t out_dim, int32_t dtype,
                       void* stream);
 
+/* Fully-connected network of scalars hs[0] -> hs[1] -> ... -> hs[n_hs-1] in ONE kernel (fp32, matrix cores):
+ *   layer l:  x <- act(x @ W_l / sqrt(hs[l] var_in)) * act_cst * sqrt(var_out)      (with activation)
+ *             x <- x @ W_l / sqrt(hs[l] var_in / var_out)                           (without)
+ * Replaces nn.FullyConnectedNet.forward (e3nn/nn/_fc.py:38-48 for a layer, :70-88 for which layers carry the
+ * activation and which variances: every layer but the last has the activation and var_out = 1, the last has
+ * var_out = variance_out and the activation only with out_act != 0).  `act` is an E3X_ACT_* code
+ * (E3X_ACT_IDENTITY for the reference's act=None) and `act_cst` its second-moment normalisation
+ * (e3nn/math/_normalize_activation.py:22-57).  The hidden activations never leave the registers.
+ * Limits (E3X_ERR_INVALID beyond them): 1..8 layers, hs[0] and the hidden widths <= 128, the zero-padded weights
+ * (widths rounded up to 32; hs[0] to 8) <= 150 KB in total.
+ * e3x_fc_forward: x[Z, hs[0]] -> out[Z, hs[n_hs-1]]; `weights` is a HOST array of n_hs-1 device pointers,
+ * weights[l] = W_l[hs[l], hs[l+1]] row-major (the reference's `layer{l}.weight`); `workspace` is device memory of
+ * e3x_fc_workspace_bytes(plan) bytes, 16-byte aligned like x, that the call overwrites. */
+typedef struct e3x_fc_plan e3x_fc_plan;
+int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act, double variance_in,
+                       double variance_out, int32_t dtype, e3x_fc_plan** out);
+int e3x_fc_plan_destroy(e3x_fc_plan* plan);
+size_t e3x_fc_workspace_bytes(const e3x_fc_plan* plan);
+/* name of the plan's code object in the kernel cache */
+const char* e3x_fc_plan_key(const e3x_fc_plan* plan);
+int e3x_fc_forward(e3x_fc_plan* plan, const void* x, const void* const* weights, void* out, int64_t Z, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
 /* Plain device copy dst[i] = src[i], n_bytes multiple of 16: the calibration kernel
  * for bandwidth counters (known traffic: n_bytes read + n_bytes written). */
 int e3x_copy_bytes(const void* src, void* dst, size_t n_bytes, void* stream);

@@ -161,6 +161,25 @@ def nn_modules():
     return out
 
 
+# (hs, act, out_act, variance_in, variance_out) of the networks the one-kernel path is tested on: the radial network of
+# the benchmark block; three layers with a 96-wide output; widths that are multiples of nothing (scalar input loads,
+# zero-padded hidden layer, a partial last column tile); one layer with an output activation and variances; no activation
+FUSED_FC_CASES = [
+    ([8, 64, 352], "silu", False, 1, 1),
+    ([8, 64, 64, 96], "tanh", False, 1, 1),
+    ([5, 100, 50], "silu", False, 1, 1),
+    ([16, 40], "sigmoid", True, 2, 3),
+    ([12, 32, 32], None, False, 1, 2),
+    ([128, 128, 128, 8], "relu", True, 1, 1),
+]
+
+
+def fused_fc_nets():
+    from e3nn_amd import nn
+
+    return [nn.FullyConnectedNet(hs, act, variance_in=vi, variance_out=vo, out_act=oa) for hs, act, oa, vi, vo in FUSED_FC_CASES]
+
+
 def conv_wide():
     # one interaction block at NequIP-like width: 32 channels per irrep, 4 species, 8 radial basis functions
     from e3nn_amd import nn
@@ -174,16 +193,23 @@ def prebuild(verbose=True, workers=6):
     process, the calling thread waits with the GIL released), so a few threads build several kernels at once."""
     from concurrent.futures import ThreadPoolExecutor
 
+    from e3nn_amd import nn
+
     jobs = []
-    for name, mod in nn_modules():
+    for name, mod in nn_modules() + [(f"fused_fc{i}", net) for i, net in enumerate(fused_fc_nets())]:
         for sub in mod.modules():
             if isinstance(sub, o3.TensorProduct):
                 jobs.append((f"module {name}", sub, (torch.float32,), True))
+            if isinstance(sub, nn.FullyConnectedNet):
+                jobs.append((f"module {name} (one kernel)", sub, None, False))
     for name, tp, dtypes in all_tensor_products():
         jobs.append((f"kernel {name}", tp, dtypes, name in BACKWARD_CASES))
 
     def build(job):
         name, tp, dtypes, backward = job
+        if dtypes is None:
+            plan = tp.fused_plan()
+            return name, [plan.key or "(layer by layer: " + plan.reason + ")"]
         keys = [tp._plan(dt).key for dt in dtypes]
         if backward:
             tp.compile_backward(torch.float32)

@@ -85,6 +85,33 @@ def test_gate_gradient_against_central_differences():
         assert float((xd.grad.cpu().double().numpy() * v).sum()) == pytest.approx(fd, rel=1e-4, abs=1e-4)
 
 
+@pytest.mark.parametrize("case", range(len(ks.FUSED_FC_CASES)))
+def test_fully_connected_net_one_kernel(case):
+    """Without a gradient the whole network is one kernel: against the oracle and against the layer-by-layer kernels,
+    on batch sizes around the 64-row wave tile and the 512-row workgroup tile."""
+    hs, act, out_act, vi, vo = ks.FUSED_FC_CASES[case]
+    net = ks.fused_fc_nets()[case].to(DEV)
+    assert net.fused_plan().handle is not None, net.fused_plan().reason
+    ws = [getattr(net, f"layer{i}").weight.detach().cpu().numpy() for i in range(len(hs) - 1)]
+    for Z in (0, 1, 63, 513, 20011):
+        x = seeded(max(Z, 1), hs[0], seed=100 + case)[:Z]
+        with torch.no_grad():
+            out = net(x.to(DEV))
+        assert out.shape == (Z, hs[-1])
+        if Z == 0:
+            continue
+        want = onn.fc_forward(ws, x.numpy(), act, variance_in=vi, variance_out=vo, out_act=out_act)
+        assert_close(out, want, what=f"one-kernel fc {hs} Z={Z}")
+        layered = net(x.to(DEV).requires_grad_(True)).detach()
+        assert_close(out, layered.cpu().numpy(), what=f"one-kernel fc vs layers {hs} Z={Z}")
+    # leading batch dimensions and a view that is not 16-byte aligned
+    x = seeded(7 * 11 * hs[0] + 1, 1, seed=5).reshape(-1)[1:].reshape(7, 11, hs[0])
+    with torch.no_grad():
+        out = net(x.to(DEV)[:, 1:])
+    want = onn.fc_forward(ws, x[:, 1:].numpy().reshape(-1, hs[0]), act, variance_in=vi, variance_out=vo, out_act=out_act)
+    assert_close(out.reshape(-1, hs[-1]), want, what="one-kernel fc, batch dims")
+
+
 def test_fully_connected_net():
     arr, meta = ks.nn_golden()
     fc = nn.FullyConnectedNet(meta["fc"]["hs"], torch.nn.functional.silu).to(DEV)
