@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <memory>
 #include <mutex>
 #include <sstream>
@@ -20,13 +21,14 @@ constexpr int kMaxDevices = 64;
 constexpr int kMaxLayers = 8;
 // LDS the packed weights may take (the CU has 160 KB; leave room for the runtime's own use)
 constexpr int64_t kMaxPackedBytes = 150 * 1024;
-// widest hidden layer: its activations (RS x width / 2 registers) and the next layer's live together
-constexpr int kMaxHidden = 128;
+// registers of a lane that may hold activations (of 256 at two waves per SIMD): the input and output of a hidden
+// layer, width / 2 registers each per 32 rows, are live together
+constexpr int kMaxLiveRegs = 192;
 }  // namespace
 
 struct e3x_fc_plan {
   std::vector<int> hs, hp;
-  int n_layers = 0, rows_per_wg = 0;
+  int n_layers = 0, rows_per_wg = 0, waves = 8;
   int64_t packed_numel = 0;
   std::string key, hsaco;
   std::mutex mu;
@@ -80,8 +82,6 @@ extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, 
     if (hs[i] < 1 || hs[i] > (1 << 20)) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: bad layer width");
     P->hs.push_back(hs[i]);
     P->hp.push_back(round_up(hs[i], i == 0 ? 8 : 32));
-    if (i < NL && P->hp[i] > kMaxHidden)
-      return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: input and hidden widths are limited to 128 in the fused kernel");
   }
   for (int l = 0; l < NL; ++l) P->packed_numel += (int64_t)P->hp[l] * P->hp[l + 1];
   if (P->packed_numel * 4 > kMaxPackedBytes)
@@ -115,8 +115,16 @@ extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, 
   // (rs (hp[l] + hp[l+1]) / 2 registers) next to rs accumulator tiles of 16
   int live = P->hp[NL - 1] / 2;
   for (int l = 0; l + 1 < NL; ++l) live = std::max(live, (P->hp[l] + P->hp[l + 1]) / 2);
-  const int rs = 2 * live + 32 + 24 <= 224 ? 2 : 1;
-  P->rows_per_wg = 8 * 32 * rs;
+  if (live > kMaxLiveRegs)
+    return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: layers too wide for the fused kernel (input or hidden width above 384, "
+                                 "or two consecutive ones above 384 in total)");
+  int rs = 2 * live + 32 + 24 <= 224 ? 2 : 1;
+  int waves = 8;
+  if (const char* v = std::getenv("E3X_FC_RS")) rs = std::atoi(v);
+  if (const char* v = std::getenv("E3X_FC_WAVES")) waves = std::atoi(v);
+  if ((rs != 1 && rs != 2) || waves < 1 || waves > 16) return fail(E3X_ERR_INVALID, "E3X_FC_RS must be 1 or 2, E3X_FC_WAVES 1..16");
+  P->waves = waves;
+  P->rows_per_wg = waves * 32 * rs;
   std::ostringstream s;
   s << "// generated: one fully-connected network\n#include <stdint.h>\nnamespace cfg {\n";
   s << "constexpr int NL = " << NL << ";\nconstexpr int H[NL + 1] = {";
@@ -128,7 +136,8 @@ extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, 
   s << "};\nconstexpr float WSCALE[NL] = {";
   for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << fstr(wscale[l]);
   s << "};\nconstexpr float OUT_POST = " << fstr(out_post) << ";\n";
-  s << "constexpr int RS = " << rs << ";\n}  // namespace cfg\n";
+  if (const char* v = std::getenv("E3X_FC_EXP")) s << "#define E3X_FC_EXP " << std::atoi(v) << "\n";
+  s << "constexpr int RS = " << rs << ", WAVES = " << waves << ";\n}  // namespace cfg\n";
   const std::string src = s.str() + e3x::kTplCommon + e3x::kTplFcMfma;
   int rc = e3x::get_code_object("fc_mfma", src, &P->key, &P->hsaco);
   if (rc) return rc;
@@ -176,7 +185,7 @@ extern "C" int e3x_fc_forward(e3x_fc_plan* P, const void* x, const void* const* 
   long long tiles = (Z + P->rows_per_wg - 1) / P->rows_per_wg;
   long long blocks = tiles < P->n_cu[dev] ? tiles : P->n_cu[dev];  // one persistent workgroup per compute unit
   void* args[] = {&x, &workspace, &out, &n_rows};
-  hipError_t err = hipModuleLaunchKernel(P->fn_fwd[dev], (unsigned)blocks, 1, 1, 512, 1, 1, 0, st, args, nullptr);
+  hipError_t err = hipModuleLaunchKernel(P->fn_fwd[dev], (unsigned)blocks, 1, 1, 64 * P->waves, 1, 1, 0, st, args, nullptr);
   if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_fc_forward: launch failed: ") + hipGetErrorString(err));
   return E3X_OK;
 }

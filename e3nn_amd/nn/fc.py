@@ -5,8 +5,10 @@ Two device paths, both HIP kernels of this package:
 
 * no gradient wanted (inference, or nothing upstream requires one): the whole network runs as ONE kernel that
   keeps the hidden activations in registers (``e3x_fc_forward``);
-* otherwise each layer is the ``uvw`` tensor product ``h_in x0e (x) 0e -> h_out x0e`` (matrix cores when h_in and
-  h_out are multiples of 32) followed by the gate kernel, which have backward passes.
+* otherwise the network runs layer by layer and keeps what the backward pass needs.  A dense layer is the same
+  kernel specialised to one layer, forward (``x @ W``) and for the input gradient (``g @ W^T``); the weight gradient
+  is that of the ``uvw`` tensor product ``h_in x0e (x) 0e -> h_out x0e``; the activation is the gate kernel.
+  Layers outside the one-kernel limits run on the tensor-product kernels throughout.
 """
 import ctypes
 
@@ -15,6 +17,34 @@ import torch
 from .. import _lib
 from ..o3.tensor_product import TensorProduct
 from .activation import _KINDS, Activation, activation_name, second_moment_constant
+
+
+class _DenseFn(torch.autograd.Function):
+    """``x @ W * s`` of one layer on the one-layer specialisations of the fused kernel (s is folded in by the plans)."""
+
+    @staticmethod
+    def forward(ctx, x, w, layer):
+        ctx.layer = layer
+        ctx.save_for_backward(x, w)
+        return layer._fwd.forward(x, [w.contiguous()])
+
+    @staticmethod
+    def backward(ctx, g):
+        x, w = ctx.saved_tensors
+        layer = ctx.layer
+        g = g.contiguous()
+        if g.data_ptr() % 16:
+            g = g.clone()
+        gx = gw = None
+        if ctx.needs_input_grad[0]:
+            # g @ W^T * s through the plan [h_out -> h_in], whose own factor is 1 / sqrt(h_out)
+            wt = (w.t() * (layer._scale * layer.h_out**0.5)).contiguous()
+            gx = layer._bwd.forward(g, [wt])
+        if ctx.needs_input_grad[1]:
+            ones = x.new_ones(x.shape[0], 1)
+            gw = layer._tp._plan(torch.float32).backward_w_uvw(x, ones, g, True).reshape(layer.h_in, layer.h_out)
+            gw = gw * (layer._scale * layer.h_in**0.5)  # the tensor product's path weight is 1 / sqrt(h_in)
+        return gx, gw, None
 
 
 class _Layer(torch.nn.Module):
@@ -28,11 +58,37 @@ class _Layer(torch.nn.Module):
             f"{h_in}x0e", "0e", f"{h_out}x0e", [(0, 0, 0, "uvw", True)], internal_weights=False, shared_weights=True
         )
         self.act = None if act is None else Activation(f"{h_out}x0e", [self._act_name])
+        # _fc.py:41-48: x @ W / sqrt(h_in var_in) before an activation, x @ W / sqrt(h_in var_in / var_out) without
+        self._scale = (h_in * var_in) ** -0.5 if act is not None else (h_in * var_in / var_out) ** -0.5
+        self._fwd = self._bwd = None
 
     def __repr__(self) -> str:
         return f"Layer({self.h_in}->{self.h_out}, act={self._act_name})"
 
+    def dense_plans(self):
+        """One-layer plans of the fused kernel for ``x @ W`` and ``g @ W^T`` (built on first use); False outside its limits."""
+        if self._fwd is None:
+            var_ratio = self.var_in if self.act is not None else self.var_in / self.var_out
+            fwd = _FusedPlan([self.h_in, self.h_out], "identity", False, var_ratio, 1)
+            bwd = _FusedPlan([self.h_out, self.h_in], "identity", False, 1, 1)
+            if fwd.handle is None or bwd.handle is None:
+                self._fwd = self._bwd = False
+            else:
+                self._fwd, self._bwd = fwd, bwd
+        return self._fwd, self._bwd
+
     def forward(self, x: torch.Tensor):
+        if x.is_cuda and x.dtype == torch.float32 and self.weight.dtype == torch.float32 and self.dense_plans()[0]:
+            lead = x.shape[:-1]
+            x2 = x.reshape(-1, self.h_in).contiguous()
+            if x2.data_ptr() % 16:
+                x2 = x2.clone()
+            y = _DenseFn.apply(x2, self.weight, self).reshape(lead + (self.h_out,))
+            if self.act is not None:
+                y = self.act(y)
+                if self.var_out != 1:
+                    y = y * self.var_out**0.5
+            return y
         ones = x.new_ones(x.shape[:-1] + (1,))
         if self.act is not None:
             x = self._tp(x, ones, self.weight.reshape(-1))

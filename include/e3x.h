@@ -210,8 +210,8 @@ int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_
  * var_out = variance_out and the activation only with out_act != 0).  `act` is an E3X_ACT_* code
  * (E3X_ACT_IDENTITY for the reference's act=None) and `act_cst` its second-moment normalisation
  * (e3nn/math/_normalize_activation.py:22-57).  The hidden activations never leave the registers.
- * Limits (E3X_ERR_INVALID beyond them): 1..8 layers, hs[0] and the hidden widths <= 128, the zero-padded weights
- * (widths rounded up to 32; hs[0] to 8) <= 150 KB in total.
+ * Limits (E3X_ERR_INVALID beyond them): 1..8 layers; with widths rounded up to 32 (hs[0] to 8), the input of the last
+ * layer <= 384, the input plus the output of every other layer <= 384, and all weights together <= 150 KB.
  * e3x_fc_forward: x[Z, hs[0]] -> out[Z, hs[n_hs-1]]; `weights` is a HOST array of n_hs-1 device pointers,
  * weights[l] = W_l[hs[l], hs[l+1]] row-major (the reference's `layer{l}.weight`); `workspace` is device memory of
  * e3x_fc_workspace_bytes(plan) bytes, 16-byte aligned like x, that the call overwrites. */

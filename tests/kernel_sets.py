@@ -155,6 +155,8 @@ def nn_modules():
     out.append(("linear_wide", o3.Linear("128x0e+128x1o+64x2e", "128x0e+64x1o+32x1o")))
     out.append(("fc_golden", nn.FullyConnectedNet(meta["fc"]["hs"], torch.nn.functional.silu)))
     out.append(("fc_radial", nn.FullyConnectedNet([8, 64, 352], torch.nn.functional.silu)))
+    # a hidden layer too wide for the one-kernel path and its one-layer specialisations: tensor-product kernels throughout
+    out.append(("fc_wide_hidden", nn.FullyConnectedNet([8, 512, 16], torch.nn.functional.silu)))
     a = meta["conv"]["args"]
     out.append(("conv_golden", nn.Convolution(a[0], a[1], a[2], a[3], a[4], a[5])))
     out.append(("conv_wide", conv_wide()))
@@ -209,7 +211,11 @@ def prebuild(verbose=True, workers=6):
         name, tp, dtypes, backward = job
         if dtypes is None:
             plan = tp.fused_plan()
-            return name, [plan.key or "(layer by layer: " + plan.reason + ")"]
+            keys = [plan.key or "(layer by layer: " + plan.reason + ")"]
+            for layer in tp:
+                fwd, bwd = layer.dense_plans()
+                keys += [fwd.key, bwd.key] if fwd else ["(tensor-product kernels)"]
+            return name, keys
         keys = [tp._plan(dt).key for dt in dtypes]
         if backward:
             tp.compile_backward(torch.float32)

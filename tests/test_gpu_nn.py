@@ -112,6 +112,29 @@ def test_fully_connected_net_one_kernel(case):
     assert_close(out.reshape(-1, hs[-1]), want, what="one-kernel fc, batch dims")
 
 
+def test_fully_connected_net_wide_hidden_layer():
+    """Outside the limits of the fused kernel every layer runs on the tensor-product kernels, forward and backward."""
+    fc = dict(ks.nn_modules())["fc_wide_hidden"].to(DEV)
+    assert fc.fused_plan().handle is None and not fc.layer0.dense_plans()[0]
+    x = seeded(300, 8, seed=21)
+    ws = [fc.layer0.weight.detach().cpu().numpy(), fc.layer1.weight.detach().cpu().numpy()]
+    with torch.no_grad():
+        assert_close(fc(x.to(DEV)), onn.fc_forward(ws, x.numpy(), "silu"), what="wide fc, no grad")
+    xd = x.to(DEV).requires_grad_(True)
+    out = fc(xd)
+    assert_close(out, onn.fc_forward(ws, x.numpy(), "silu"), what="wide fc")
+    cot = seeded(300, 16, seed=22)
+    out.backward(cot.to(DEV))
+    rng = np.random.default_rng(3)
+    x64, c64 = x.numpy().astype(np.float64), cot.numpy().astype(np.float64)
+    v, eps = rng.normal(size=x64.shape), 1e-5
+    fd = ((onn.fc_forward(ws, x64 + eps * v) - onn.fc_forward(ws, x64 - eps * v)) * c64).sum() / (2 * eps)
+    assert float((xd.grad.cpu().double().numpy() * v).sum()) == pytest.approx(fd, rel=2e-4)
+    dw = rng.normal(size=ws[1].shape)
+    fd = ((onn.fc_forward([ws[0], ws[1] + eps * dw], x64) - onn.fc_forward([ws[0], ws[1] - eps * dw], x64)) * c64).sum() / (2 * eps)
+    assert float((fc.layer1.weight.grad.cpu().double().numpy() * dw).sum()) == pytest.approx(fd, rel=2e-4)
+
+
 def test_fully_connected_net():
     arr, meta = ks.nn_golden()
     fc = nn.FullyConnectedNet(meta["fc"]["hs"], torch.nn.functional.silu).to(DEV)
@@ -138,6 +161,10 @@ def test_fully_connected_net():
     dw = rng.normal(size=ws[0].shape)
     fd = ((onn.fc_forward([ws[0] + eps * dw, ws[1]], x64) - onn.fc_forward([ws[0] - eps * dw, ws[1]], x64)) * c64).sum() / (2 * eps)
     assert float((fc.layer0.weight.grad.cpu().double().numpy() * dw).sum()) == pytest.approx(fd, rel=2e-4)
+    dw = rng.normal(size=ws[1].shape)
+    fd = ((onn.fc_forward([ws[0], ws[1] + eps * dw], x64) - onn.fc_forward([ws[0], ws[1] - eps * dw], x64)) * c64).sum() / (2 * eps)
+    assert float((fc.layer1.weight.grad.cpu().double().numpy() * dw).sum()) == pytest.approx(fd, rel=2e-4)
+    assert fc.layer1.dense_plans()[0], "the dense layers of the radial network run on the one-layer kernels"
 
 
 def _conv_oracle(conv, args, params, node_input, node_attr, src, dst, edge_attr, edge_scalars):
