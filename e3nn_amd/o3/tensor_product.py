@@ -205,9 +205,7 @@ class _TensorProductFn(torch.autograd.Function):
             if need2:
                 g2 = tp._grad_plan("x2", x1.dtype).forward(x1, g, _permuted_weights(tp, w, (0, 2, 1)))
         elif mode == "general":
-            raise NotImplementedError(
-                "tensor products with connection modes other than pure uvu / pure uvw have a forward kernel only"
-            )
+            raise AssertionError("general connection modes are differentiated through TensorProduct._dense_equivalent")
         else:
             g1, g2 = torch.zeros_like(x1), torch.zeros_like(x2)
             gw = torch.zeros_like(w) if needw else None
@@ -276,8 +274,7 @@ class TensorProduct(torch.nn.Module):
         path_normalization = "element" if path_normalization is None else path_normalization
         assert irrep_normalization in ["component", "norm", "none"]
         assert path_normalization in ["element", "path", "none"]
-        if compile_right:
-            raise NotImplementedError("TensorProduct.right() has no kernel; construct with compile_right=False")
+        self._compile_right = compile_right  # right() runs on the forward kernel: nothing extra to build
 
         self.irreps_in1 = Irreps(irreps_in1)
         self.irreps_in2 = Irreps(irreps_in2)
@@ -416,11 +413,75 @@ class TensorProduct(torch.nn.Module):
         self._plan(dtype)
         return self
 
+    def _dense_equivalent(self):
+        """``(tp, expand)`` for instruction sets outside pure ``uvu`` / pure ``uvw``: the same bilinear map written as
+        a pure ``uvw`` product whose weight blocks ``[U, V, W]`` are zero except where the connection mode couples
+        the indices (``uvu``: ``D[u, v, u] = w[u, v]``, ``uuu``: ``D[u, u, u] = w[u]``, ``u<vw``: ``D[u, v, w] = w[p(u, v), w]``
+        for ``u < v`` ...), with the path weights carried over unchanged.  ``expand(w)`` builds the dense weights
+        from the structured ones by a differentiable ``index_copy``.  It costs U V W instead of U V products per path,
+        but every gradient of the ``uvw`` family has a kernel; the forward pass without gradients keeps the
+        mode-specific kernel."""
+        cached = self._plans.get("dense")
+        if cached is not None:
+            return cached
+        i1, i2, io = self.irreps_in1, self.irreps_in2, self.irreps_out
+        ins, blocks = [], []  # blocks: (weighted, numel of the structured block, positions in the dense block, dense numel)
+        for t in self.instructions:
+            U, V, W = i1[t.i_in1].mul, i2[t.i_in2].mul, io[t.i_out].mul
+            ins.append((t.i_in1, t.i_in2, t.i_out, "uvw", True, t.path_weight**2))
+            u, v = torch.meshgrid(torch.arange(U), torch.arange(V), indexing="ij")
+            u, v = u.reshape(-1), v.reshape(-1)
+            m = t.connection_mode
+            if m == "uvw":
+                pos = torch.arange(U * V * W)
+            elif m == "uvu":
+                pos = (u * V + v) * W + u
+            elif m == "uvv":
+                pos = (u * V + v) * W + v
+            elif m == "uuw":
+                a = torch.arange(U)
+                base = (a * V + a) * W
+                pos = (base[:, None] + torch.arange(W)[None, :]).reshape(-1) if t.has_weight else base
+            elif m == "uuu":
+                a = torch.arange(U)
+                pos = (a * V + a) * W + a
+            elif m == "uvuv":
+                pos = (u * V + v) * W + (u * V + v)
+            else:
+                pu, pv = torch.triu_indices(U, V, 1)
+                pair = (pu * V + pv) * W
+                if m == "uvu<v":
+                    pos = pair + torch.arange(pair.numel())
+                else:  # u<vw
+                    pos = (pair[:, None] + torch.arange(W)[None, :]).reshape(-1)
+            blocks.append((t.has_weight, prod(t.path_shape) if t.has_weight else pos.numel(), pos, U * V * W))
+        shared = self.shared_weights or self.weight_numel == 0
+        tp = TensorProduct(
+            i1, i2, io, ins, irrep_normalization="none", path_normalization="none", internal_weights=False, shared_weights=shared
+        )
+
+        def expand(w, like):
+            batch = () if shared else w.shape[:-1]
+            out, off = [], 0
+            for weighted, n, pos, dense in blocks:
+                pos = pos.to(like.device)
+                if weighted:
+                    vals = w.narrow(-1, off, n)
+                    off += n
+                else:
+                    vals = like.new_ones(batch + (n,))
+                out.append(like.new_zeros(batch + (dense,)).index_copy(-1, pos, vals.to(like.dtype)))
+            return torch.cat(out, dim=-1) if out else like.new_empty(batch + (0,))
+
+        self._plans["dense"] = (tp, expand)
+        return tp, expand
+
     def compile_backward(self, dtype: torch.dtype = torch.float32) -> "TensorProduct":
         """Also builds the transposed plans the backward pass uses."""
         self._plan(dtype)
         if self._live_mode() == "general":
-            return self  # forward kernel only
+            self._dense_equivalent()[0].compile_backward(dtype)
+            return self
         self._grad_plan("x1", dtype)
         if self._live_mode() == "uvw":
             self._grad_plan("x2", dtype)
@@ -496,7 +557,24 @@ class TensorProduct(torch.nn.Module):
 
     # ------------------------------------------------------------------ evaluation
     def right(self, y, weight=None):
-        raise NotImplementedError("TensorProduct.right() has no HIP kernel")
+        r"""Partially evaluate :math:`w x \otimes y`: the matrices ``[..., irreps_in1.dim, irreps_out.dim]`` with
+        ``forward(x, y, w) == x @ right(y, w)`` (reference ``_tensor_product.py:447-486``).  There is no kernel of its
+        own: row ``a`` of the result is the tensor product of the ``a``-th basis vector with ``y``, so one forward
+        launch on ``irreps_in1.dim`` rows per sample gives the whole matrix (and its gradients)."""
+        torch._assert(self._compile_right, "`right` method is not compiled, set `compile_right` to True when creating the TensorProduct")
+        torch._assert(y.shape[-1] == self._in2_dim, "Incorrect last dimension for y")
+        w = self._get_weights(weight)
+        self._check_device(y)
+        if self.shared_weights or self.weight_numel == 0:
+            batch = tuple(y.shape[:-1])
+        else:
+            batch = tuple(torch.broadcast_shapes(y.shape[:-1], w.shape[:-1]))
+        d1 = self._in1_dim
+        eye = torch.eye(d1, dtype=y.dtype, device=y.device).expand(batch + (d1, d1))
+        yb = y.expand(batch + (-1,)).unsqueeze(-2).expand(batch + (d1, self._in2_dim))
+        if not (self.shared_weights or self.weight_numel == 0):
+            w = w.expand(batch + (-1,)).unsqueeze(-2).expand(batch + (d1, self.weight_numel))
+        return self.forward(eye, yb, w if self.weight_numel else None)
 
     def _check_device(self, *tensors):
         for t in tensors:
@@ -526,7 +604,11 @@ class TensorProduct(torch.nn.Module):
             wf = w.to(x1.dtype).contiguous()
         else:
             wf = w.expand(batch + (-1,)).reshape(-1, self.weight_numel).to(x1.dtype).contiguous()
-        out = _TensorProductFn.apply(x1, x2, wf, self)
+        if self._live_mode() == "general" and torch.is_grad_enabled() and (x1.requires_grad or x2.requires_grad or wf.requires_grad):
+            dense_tp, expand = self._dense_equivalent()
+            out = _TensorProductFn.apply(x1, x2, expand(wf, x1), dense_tp)
+        else:
+            out = _TensorProductFn.apply(x1, x2, wf, self)
         return out.reshape(batch + (self.irreps_out.dim,))
 
     def forward_gather_scatter(

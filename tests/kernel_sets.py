@@ -29,7 +29,7 @@ def golden_meta():
         return json.load(f)
 
 
-def tp_from_meta(m):
+def tp_from_meta(m, **extra):
     upw = m.get("user_path_weights", [1.0] * len(m["instructions"]))
     ins = [tuple(t[:5]) + (pw,) for t, pw in zip(m["instructions"], upw)]
     kw = {}
@@ -37,15 +37,15 @@ def tp_from_meta(m):
         kw = dict(irrep_normalization=m["irrep_normalization"], path_normalization=m["path_normalization"])
     return o3.TensorProduct(
         m["irreps_in1"], m["irreps_in2"], m["irreps_out"], ins,
-        internal_weights=m["internal_weights"], shared_weights=m["shared_weights"], **kw,
+        internal_weights=m["internal_weights"], shared_weights=m["shared_weights"], **kw, **extra,
     )  # fmt: skip
 
 
-def golden_tp(name, meta=None):
+def golden_tp(name, meta=None, **extra):
     m = dict((meta or golden_meta())[name])
     if name == "fctp_norm_path":
         m.update(irrep_normalization="norm", path_normalization="path")
-    return tp_from_meta(m)
+    return tp_from_meta(m, **extra)
 
 
 def cfg1():
@@ -91,11 +91,11 @@ def radial_layer():
     return o3.FullyConnectedTensorProduct("64x0e", "0e", "352x0e")
 
 
-def mixed_modes():
+def mixed_modes(**extra):
     # uvu and uvw paths into the same output irrep plus an elementwise and an unweighted path: the general kernel
     ins = [(0, 0, 0, "uvu", True), (1, 1, 0, "uvw", True), (1, 0, 1, "uvu", False), (1, 1, 2, "uvv", True),
            (0, 0, 3, "uuu", True), (1, 2, 4, "uuw", False)]  # fmt: skip
-    return o3.TensorProduct("4x0e+4x1o", "4x0e+3x1o+4x1e", "4x0e+4x1o+3x1e+4x0e+1x0o", ins, shared_weights=False)
+    return o3.TensorProduct("4x0e+4x1o", "4x0e+3x1o+4x1e", "4x0e+4x1o+3x1e+4x0e+1x0o", ins, shared_weights=False, **extra)
 
 
 def scalar_exact():
@@ -132,7 +132,8 @@ def all_tensor_products():
 
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
-                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "radial_layer", "odd_mul"]  # fmt: skip
+                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "radial_layer", "odd_mul",
+                  "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
 
 
 def nn_golden():

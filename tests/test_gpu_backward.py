@@ -134,13 +134,62 @@ def test_shared_uvu_weight_gradient():
     assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
 
 
-def test_missing_backward_kernels_fail_loudly():
-    # connection modes outside pure uvu / pure uvw have a forward kernel only: the call must raise, not fall back
-    tp = ks.mixed_modes()
-    x1 = seeded(4, tp.irreps_in1.dim).to(DEV).requires_grad_(True)
-    out = tp(x1, seeded(4, tp.irreps_in2.dim).to(DEV), seeded(4, tp.weight_numel).to(DEV))
-    with pytest.raises(NotImplementedError):
-        out.sum().backward()
+@pytest.mark.parametrize("maker", [ks.mixed_modes, lambda: ks.golden_tp("modes_uuu_uvuv_uuw_uvv"), lambda: ks.golden_tp("modes_triangular")])
+def test_general_mode_gradients(maker):
+    """Connection modes outside pure uvu / pure uvw are differentiated through the equivalent uvw product with structured
+    weights.  The map is trilinear, so central differences of the float64 oracle along a direction are exact."""
+    from oracle import tensor_product as otp
+
+    tp = maker().to(DEV)
+    assert tp._live_mode() == "general"
+    spec = oracle_spec(tp)
+    Z = 37
+    wshape = (tp.weight_numel,) if tp.shared_weights else (Z, tp.weight_numel)
+    x1, x2, w = seeded(Z, tp.irreps_in1.dim, seed=1), seeded(Z, tp.irreps_in2.dim, seed=2), seeded(*wshape, seed=3)
+    cot = seeded(Z, tp.irreps_out.dim, seed=4)
+    a, b, c = (t.to(DEV).requires_grad_(True) for t in (x1, x2, w))
+    out = tp(a, b, c)
+    f = lambda p, q, r: otp.tp_forward(spec, p, q, r if tp.weight_numel else None)  # noqa: E731
+    n1, n2, nw = (t.numpy().astype(np.float64) for t in (x1, x2, w))
+    assert_close(out, f(n1, n2, nw), what="forward through the dense equivalent")
+    with torch.no_grad():
+        assert_close(tp(a, b, c), f(n1, n2, nw), what="forward, mode-specific kernel")
+    out.backward(cot.to(DEV))
+    rng = np.random.default_rng(5)
+    c64 = cot.numpy().astype(np.float64)
+    for got, which in ((a.grad, 0), (b.grad, 1), (c.grad, 2)):
+        if which == 2 and not tp.weight_numel:
+            continue
+        for _ in range(3):
+            args = [n1, n2, nw]
+            v = rng.normal(size=args[which].shape)
+            plus, minus = list(args), list(args)
+            plus[which], minus[which] = args[which] + v, args[which] - v
+            want = ((f(*plus) - f(*minus)) * c64).sum() / 2
+            assert float((got.cpu().double().numpy() * v).sum()) == pytest.approx(want, rel=2e-4, abs=1e-3)
+
+
+@pytest.mark.parametrize("maker", [lambda **kw: ks.golden_tp("fctp_small_cfg5_like", **kw), lambda **kw: ks.golden_tp("uvu_merged_cfg3_like_mul4", **kw), ks.mixed_modes])
+def test_right(maker):
+    """right(y, w) is the matrix with forward(x, y, w) == x @ right(y, w) (the reference's own test of right(),
+    tests/o3/tensor_product_test.py, checks this identity); the forward side is the oracle's."""
+    from oracle import tensor_product as otp
+
+    with pytest.raises(AssertionError):  # as in the reference, right() is there only when asked for at construction
+        maker().right(seeded(1, maker().irreps_in2.dim).to(DEV))
+    tp = maker(compile_right=True).to(DEV)
+    spec = oracle_spec(tp)
+    Z = 5
+    wshape = (tp.weight_numel,) if tp.shared_weights else (Z, tp.weight_numel)
+    x1, x2, w = seeded(Z, tp.irreps_in1.dim, seed=1), seeded(Z, tp.irreps_in2.dim, seed=2), seeded(*wshape, seed=3)
+    with torch.no_grad():
+        r = tp.right(x2.to(DEV), w.to(DEV) if tp.weight_numel else None)
+    assert r.shape == (Z, tp.irreps_in1.dim, tp.irreps_out.dim)
+    got = torch.einsum("zik,zi->zk", r.cpu().double(), x1.double())
+    want = otp.tp_forward(spec, *(t.numpy().astype(np.float64) for t in (x1, x2)), w.numpy().astype(np.float64) if tp.weight_numel else None)
+    assert_close(got, want, what="x @ right(y, w)")
+    # rows of the operator that belong to an input irrep no instruction reads are zero
+    assert torch.isfinite(r).all()
 
 
 @pytest.mark.parametrize("lmax", [1, 2, 3])

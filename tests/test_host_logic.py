@@ -134,8 +134,7 @@ def test_module_state_and_api_details():
     # every connection mode of the reference builds a plan (the general vector-ALU kernel family)
     tp = o3.TensorProduct("2x1o", "2x1o", "2x1e", [(0, 0, 0, "uuu", True)])
     assert tp.weight_numel == 2 and tp._plan(torch.float32).family == "uvw_small"
-    with pytest.raises(NotImplementedError):
-        o3.TensorProduct("2x1o", "2x1o", "2x1e", [(0, 0, 0, "uuu", True)], compile_right=True)
+    assert o3.TensorProduct("2x1o", "2x1o", "2x1e", [(0, 0, 0, "uuu", True)], compile_right=True)._compile_right
     set_optimization_defaults(specialized_code=False)
     assert get_optimization_defaults()["specialized_code"] is False
     set_optimization_defaults(specialized_code=True)
@@ -155,3 +154,25 @@ def test_plan_creation_needs_no_gpu_and_reports_family():
     assert L.e3x_tp_plan_create(ctypes.byref(bad), ctypes.byref(h)) == -1  # 1o x 1o -> 1o violates parity
     assert b"selection" in L.e3x_last_error()
     assert L.e3x_csr_workspace_bytes(1000, 10) > 3 * 4000
+
+
+@pytest.mark.parametrize("name", ["mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"])
+def test_dense_uvw_equivalent_of_general_modes(name):
+    """Gradients of connection modes outside pure uvu / pure uvw go through a pure-uvw product with structured weights:
+    on the oracle, that product with the expanded weights is the same map as the original instruction set."""
+    from oracle import tensor_product as otp
+    from tests import kernel_sets as ks
+    from tests.helpers import oracle_spec, seeded
+
+    tp = ks.mixed_modes() if name == "mixed_modes" else ks.golden_tp(name)
+    dense_tp, expand = tp._dense_equivalent()
+    assert all(t.connection_mode == "uvw" for t in dense_tp.instructions)
+    Z = 6
+    wshape = (tp.weight_numel,) if tp.shared_weights else (Z, tp.weight_numel)
+    x1, x2, w = seeded(Z, tp.irreps_in1.dim, seed=1), seeded(Z, tp.irreps_in2.dim, seed=2), seeded(*wshape, seed=3)
+    want = otp.tp_forward(oracle_spec(tp), x1.numpy(), x2.numpy(), w.numpy() if tp.weight_numel else None)
+    wd = expand(w, x1)
+    assert wd.shape[-1] == dense_tp.weight_numel
+    got = otp.tp_forward(oracle_spec(dense_tp, irrep_normalization="none", path_normalization="none",
+                                     user_path_weights=[t.path_weight**2 for t in tp.instructions]), x1.numpy(), x2.numpy(), wd.numpy())
+    np.testing.assert_allclose(got, want, rtol=1e-10, atol=1e-12)
