@@ -306,6 +306,78 @@ __global__ __launch_bounds__(kWave) void sh_generic_kernel(const float* __restri
   }
 }
 
+// Reverse sweep of the same recurrence for any l list: the forward values of the tile stay in LDS, the adjoint of
+// Y^l_j collects coef * a * adj(Y^{l+1}_i) from the level above (entries are ordered by level, so walking them
+// backwards finds every adjoint complete), the adjoint of the coordinate a collects coef * Y^l_j * adj(Y^{l+1}_i).
+// blockDim.x = 64, or 32 when two tables of 64 columns would not fit in 64 KB of LDS.
+__global__ __launch_bounds__(kWave) void sh_generic_bwd_kernel(const float* __restrict__ xyz,
+                                                               const float* __restrict__ gout,
+                                                               float* __restrict__ gxyz, long long n, int lmax,
+                                                               int n_out, int normalize, const ColMap cmap) {
+  extern __shared__ float s_mem[];
+  const int W = blockDim.x, lane = threadIdx.x;
+  const int n_col = (lmax + 1) * (lmax + 1);
+  float* s_y = s_mem;
+  float* s_g = s_mem + n_col * W;
+  for (long long v = (long long)blockIdx.x * W + lane; v - lane < n; v += (long long)gridDim.x * W) {
+    const bool live = v < n;
+    float x = 0.f, y = 0.f, z = 0.f;
+    if (live) {
+      x = xyz[v * 3 + 0];
+      y = xyz[v * 3 + 1];
+      z = xyz[v * 3 + 2];
+    }
+    const float r = sqrtf(x * x + y * y + z * z);
+    const float inv = 1.0f / fmaxf(r, 1e-12f);
+    if (normalize) {
+      x *= inv;
+      y *= inv;
+      z *= inv;
+    }
+    s_y[lane] = 1.0f;
+    const int n_ent = c_rec_end[lmax];
+    int cur = -1;
+    float acc = 0.f;
+    for (int e = 0; e < n_ent; ++e) {
+      const RecEntry t = c_rec[e];
+      if ((int)t.out_col != cur) {
+        if (cur >= 0) s_y[cur * W + lane] = acc;
+        cur = t.out_col;
+        acc = 0.f;
+      }
+      const float a = t.axis == 0 ? x : (t.axis == 1 ? y : z);
+      acc = fmaf(t.coef * a, s_y[t.in_col * W + lane], acc);
+    }
+    if (cur >= 0) s_y[cur * W + lane] = acc;
+    for (int c = 0; c < n_col; ++c) s_g[c * W + lane] = 0.f;
+    if (live)
+      for (int c = 0; c < n_out; ++c) s_g[cmap.src[c] * W + lane] += cmap.scale[c] * gout[v * n_out + c];
+    float gx = 0.f, gy = 0.f, gz = 0.f;
+    for (int e = n_ent - 1; e >= 0; --e) {
+      const RecEntry t = c_rec[e];
+      const float go = s_g[t.out_col * W + lane];
+      const float a = t.axis == 0 ? x : (t.axis == 1 ? y : z);
+      s_g[t.in_col * W + lane] = fmaf(t.coef * a, go, s_g[t.in_col * W + lane]);
+      const float d = t.coef * s_y[t.in_col * W + lane] * go;
+      gx += t.axis == 0 ? d : 0.f;
+      gy += t.axis == 1 ? d : 0.f;
+      gz += t.axis == 2 ? d : 0.f;
+    }
+    if (normalize) {
+      // x / max(|x|, eps): (g - xhat (xhat . g)) / |x| above the clamp, g / eps below it
+      const float dot = r > 1e-12f ? x * gx + y * gy + z * gz : 0.f;
+      gx = (gx - x * dot) * inv;
+      gy = (gy - y * dot) * inv;
+      gz = (gz - z * dot) * inv;
+    }
+    if (live) {
+      gxyz[v * 3 + 0] = gx;
+      gxyz[v * 3 + 1] = gy;
+      gxyz[v * 3 + 2] = gz;
+    }
+  }
+}
+
 std::mutex g_mu;
 bool g_tables_ready[64] = {false};
 
@@ -434,20 +506,50 @@ extern "C" int e3x_sh_backward(const int32_t* ls, int32_t n_ls, int32_t normaliz
   if (dtype != E3X_F32) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: only fp32 storage is implemented");
   if (normalization < 0 || normalization > 2)
     return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: normalization must be integral, component or norm");
-  for (int i = 0; i < n_ls; ++i)
-    if (ls[i] != i) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: the l list must be 0, 1, ..., lmax");
-  const int lmax = n_ls - 1;
-  if (lmax > 3) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: implemented for lmax <= 3");
+  int lmax = 0, n_out = 0;
+  bool is_range = true;
+  for (int i = 0; i < n_ls; ++i) {
+    if (ls[i] < 0 || ls[i] > kMaxL) return e3x::fail(E3X_ERR_INVALID, "spherical_harmonics maximum l implemented is 12");
+    lmax = ls[i] > lmax ? ls[i] : lmax;
+    is_range = is_range && ls[i] == i;
+    n_out += 2 * ls[i] + 1;
+  }
+  if (n_out > kMaxCols) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: more than 169 output columns");
   if (n == 0) return E3X_OK;
   if (!xyz || !grad_out || !grad_xyz) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: null pointer");
   if (n >= (1LL << 31) * 256) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward: too many vectors for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  if (!is_range || lmax > 3) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return e3x::fail(E3X_ERR_HIP, "hipGetDevice failed");
+    std::lock_guard<std::mutex> lock(g_mu);
+    int rc = upload_tables(dev);
+    if (rc) return rc;
+    ColMap cm;
+    int c = 0;
+    for (int i = 0; i < n_ls; ++i)
+      for (int m = 0; m < 2 * ls[i] + 1; ++m, ++c) {
+        cm.src[c] = (unsigned char)(ls[i] * ls[i] + m);
+        cm.scale[c] = normalization == E3X_NORM_INTEGRAL ? (float)(1.0 / std::sqrt(4.0 * M_PI))
+                      : normalization == E3X_NORM_NORM   ? (float)(1.0 / std::sqrt(2.0 * ls[i] + 1.0))
+                                                         : 1.0f;
+      }
+    const int n_col = (lmax + 1) * (lmax + 1);
+    const int width = 2 * n_col * kWave * (int)sizeof(float) <= 65536 ? kWave : kWave / 2;
+    long long blocks = (n + width - 1) / width;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    const size_t shmem = (size_t)2 * n_col * width * sizeof(float);
+    hipLaunchKernelGGL(sh_generic_bwd_kernel, dim3((unsigned)blocks), dim3(width), shmem, st, (const float*)xyz,
+                       (const float*)grad_out, (float*)grad_xyz, (long long)n, lmax, n_out, (int)normalize, cm);
+    if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_sh_backward: kernel launch failed");
+    return E3X_OK;
+  }
   Scale4 sc;
   for (int l = 0; l < 4; ++l) {
     sc.s[l] = 1.0f;
     if (normalization == E3X_NORM_INTEGRAL) sc.s[l] = (float)(1.0 / std::sqrt(4.0 * M_PI));
     if (normalization == E3X_NORM_NORM) sc.s[l] = (float)(1.0 / std::sqrt(2.0 * l + 1.0));
   }
-  hipStream_t st = (hipStream_t)stream;
   const float *px = (const float*)xyz, *pg = (const float*)grad_out;
   float* po = (float*)grad_xyz;
   switch (lmax) {

@@ -42,8 +42,6 @@ class _SphericalHarmonicsFn(torch.autograd.Function):
     def backward(ctx, g):
         (xyz,) = ctx.saved_tensors
         ls, normalize, normalization, batch = ctx.cfg
-        if list(ls) != list(range(len(ls))) or len(ls) > 4:
-            raise NotImplementedError("the spherical-harmonics backward kernel covers l = 0..lmax with lmax <= 3")
         n = xyz.shape[0]
         g = g.reshape(n, -1).contiguous()
         gx = torch.empty_like(xyz)

@@ -185,9 +185,10 @@ int e3x_tp_backward_w_uvw(e3x_plan* plan, const void* x1, const void* x2, const 
 int e3x_sh_forward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization, const void* xyz,
                    void* out, int64_t n, int32_t dtype, void* stream);
 
-/* grad_xyz[n, 3] from grad_out[n, (lmax+1)^2] for ls = 0..lmax, lmax <= 3: the backward pass of
- * e3x_sh_forward (the reference differentiates the polynomial chain of
- * e3nn/o3/_spherical_harmonics.py:93-112,193-249 by autograd). */
+/* grad_xyz[n, 3] from grad_out[n, sum(2 l + 1)] for the same l list: the backward pass of e3x_sh_forward (the
+ * reference differentiates the polynomial chain of e3nn/o3/_spherical_harmonics.py:93-112,193-249 by autograd).
+ * ls = 0..lmax with lmax <= 3 runs on closed forms, any other list (l <= 12) on the reverse sweep of the
+ * recurrence. */
 int e3x_sh_backward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization, const void* xyz,
                     const void* grad_out, void* grad_xyz, int64_t n, int32_t dtype, void* stream);
 

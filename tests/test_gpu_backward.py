@@ -220,3 +220,34 @@ def test_spherical_harmonics_gradient(lmax, normalize, normalization):
     xp[0, 1] += eps
     fd = ((ref_fn(xp) - ref_fn(x.double()))[0] * cot[0].double()).sum() / eps
     assert abs(fd - rx[0, 1]) < 1e-4 * max(1.0, abs(float(fd)))
+
+
+@pytest.mark.parametrize("ls,normalize,normalization", [
+    ([0, 1, 2, 3, 4, 5], True, "component"), ([6], False, "integral"), ([2, 2, 0, 7], True, "norm"), ([1, 3], False, "component"),
+    (list(range(11)), True, "integral"), (list(range(13)), True, "component"), ([12, 11], False, "norm"),
+])  # fmt: skip
+def test_spherical_harmonics_gradient_any_l_list(ls, normalize, normalization):
+    """l lists beyond 0..3 take the reverse sweep of the recurrence: against central differences of the float64 oracle
+    along random directions, point by point."""
+    from e3nn_amd import o3
+    from oracle import spherical_harmonics as osh
+
+    n = 203
+    x = seeded(n, 3, seed=len(ls))
+    n_out = sum(2 * l + 1 for l in ls)
+    cot = seeded(n, n_out, seed=11)
+    xd = x.to(DEV).requires_grad_(True)
+    out = o3.spherical_harmonics(ls, xd, normalize, normalization)
+    assert out.shape == (n, n_out)
+    out.backward(cot.to(DEV))
+    got = xd.grad.cpu().double().numpy()
+    x64, c64 = x.numpy().astype(np.float64), cot.numpy().astype(np.float64)
+    rng = np.random.default_rng(7)
+    f = lambda p: osh.spherical_harmonics(ls, p, normalize, normalization)  # noqa: E731
+    for _ in range(3):
+        v = rng.normal(size=x64.shape)
+        eps = 1e-6
+        want = ((f(x64 + eps * v) - f(x64 - eps * v)) * c64).sum(axis=1) / (2 * eps)
+        have = (got * v).sum(axis=1)
+        scale = max(1.0, float(np.abs(want).max()))
+        assert np.abs(have - want).max() < 2e-4 * scale, (np.abs(have - want).max(), scale)
