@@ -886,10 +886,14 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   // one thread per (path, v, w) column of the weight blocks
   long long cols = 0;
   for (const auto& q : P->paths) cols += (long long)P->in2[q.in2].mul * P->out[q.out].mul;
-  const long long wblocks = (cols + 255) / 256;
-  // enough batch slices to fill the chip a few times over, at least 16 rows each
-  long long slices = (4096 + wblocks - 1) / wblocks;
-  if (slices > (Z + 15) / 16) slices = (Z + 15) / 16;
+  // with fewer than 256 columns a workgroup is (power of two >= columns) x (interleaved rows of its slice)
+  long long cpb = 1;
+  while (cpb < cols && cpb < 256) cpb *= 2;
+  const long long row_lanes = 256 / cpb;
+  const long long wblocks = (cols + cpb - 1) / cpb;
+  // enough batch slices to fill the chip a few times over, at least 16 rows per row lane
+  long long slices = (2048 + wblocks - 1) / wblocks;
+  if (slices > (Z + 16 * row_lanes - 1) / (16 * row_lanes)) slices = (Z + 16 * row_lanes - 1) / (16 * row_lanes);
   if (slices < 1) slices = 1;
   if (slices > 65535) slices = 65535;
   long long rows_per_slice = (Z + slices - 1) / slices;
