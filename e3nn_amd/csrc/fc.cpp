@@ -36,6 +36,12 @@ struct e3x_fc_plan {
   hipFunction_t fn_pack[kMaxDevices] = {nullptr};
   hipFunction_t fn_fwd[kMaxDevices] = {nullptr};
   int n_cu[kMaxDevices] = {0};
+  // weight gradient of a one-layer plan: a code object of its own, built on first use
+  double scale0 = 1.0;  // factor on x @ W of the first layer
+  int dw_col_groups = 0;
+  std::string dw_key, dw_hsaco;
+  hipModule_t dw_module[kMaxDevices] = {nullptr};
+  hipFunction_t fn_dw[kMaxDevices] = {nullptr};
 };
 
 namespace {
@@ -107,6 +113,7 @@ extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, 
       post = 1.0;
     }
     if (last) out_post = post;
+    if (l == 0) P->scale0 = wscale[0];
     post_prev = post;
     var_in = var_out;
   }
@@ -147,6 +154,60 @@ extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, 
 
 extern "C" int e3x_fc_plan_destroy(e3x_fc_plan* plan) {
   delete plan;  // code objects stay loaded for the life of the process
+  return E3X_OK;
+}
+
+extern "C" int e3x_fc_plan_prepare_backward_w(e3x_fc_plan* P) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_fc_plan_prepare_backward_w: null plan");
+  if (P->n_layers != 1) return fail(E3X_ERR_INVALID, "e3x_fc_backward_w: one-layer plans only");
+  std::lock_guard<std::mutex> lock(P->mu);
+  if (!P->dw_hsaco.empty()) return E3X_OK;
+  const int mt = (P->hs[0] + 31) / 32, nt = (P->hs[1] + 31) / 32;
+  if (mt > 8) return fail(E3X_ERR_INVALID, "e3x_fc_backward_w: input width above 256");
+  int ntw = std::min((nt + 3) / 4, std::max(1, 10 / mt));  // <= 160 accumulator registers per lane
+  P->dw_col_groups = (nt + 4 * ntw - 1) / (4 * ntw);
+  std::ostringstream s;
+  s << "// generated: weight gradient of one dense layer\n#include <stdint.h>\n";
+  if (const char* v = std::getenv("E3X_FCDW_KU")) s << "#define E3X_FCDW_KU " << std::atoi(v) << "\n";
+  if (const char* v = std::getenv("E3X_FCDW_OCC")) s << "#define E3X_FCDW_OCC " << std::atoi(v) << "\n";
+  s << "namespace cfg {\n";
+  s << "constexpr int H_IN = " << P->hs[0] << ", H_OUT = " << P->hs[1] << ", NTW = " << ntw << ";\n";
+  s << "constexpr float SCALE = " << fstr(P->scale0) << ";\n}  // namespace cfg\n";
+  const std::string src = s.str() + e3x::kTplCommon + e3x::kTplFcDw;
+  return e3x::get_code_object("fc_dw", src, &P->dw_key, &P->dw_hsaco);
+}
+
+extern "C" int e3x_fc_backward_w(e3x_fc_plan* P, const void* x, const void* grad_out, void* grad_w, int64_t Z, void* stream) {
+  int rc = e3x_fc_plan_prepare_backward_w(P);
+  if (rc) return rc;
+  if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_fc_backward_w: negative batch");
+  if (!grad_w || (Z > 0 && (!x || !grad_out))) return fail(E3X_ERR_INVALID, "e3x_fc_backward_w: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  if ((rc = e3x::fill_zero_bytes(grad_w, (size_t)P->hs[0] * P->hs[1] * 4, stream))) return rc;
+  if (Z == 0) return E3X_OK;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(E3X_ERR_HIP, "hipGetDevice failed");
+  {
+    std::lock_guard<std::mutex> lock(P->mu);
+    if (!P->dw_module[dev]) {
+      hipModule_t mod = nullptr;
+      hipError_t err = hipModuleLoad(&mod, P->dw_hsaco.c_str());
+      if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + P->dw_hsaco + ") failed: " + hipGetErrorString(err));
+      if (hipModuleGetFunction(&P->fn_dw[dev], mod, "e3x_fc_dw_k") != hipSuccess)
+        return fail(E3X_ERR_HIP, "kernel e3x_fc_dw_k missing from " + P->dw_hsaco);
+      P->dw_module[dev] = mod;
+    }
+  }
+  // two workgroups per compute unit (over all column groups) share the rows in trips of 16
+  int per_cu = 2;
+  if (const char* v = std::getenv("E3X_FCDW_OCC")) per_cu = std::atoi(v);
+  long long slices = std::max(1, 256 * per_cu / P->dw_col_groups);
+  slices = std::min<long long>(slices, (Z + 255) / 256);
+  long long n_rows = Z;
+  void* args[] = {&x, &grad_out, &grad_w, &n_rows};
+  hipError_t err = hipModuleLaunchKernel(P->fn_dw[dev], (unsigned)slices, (unsigned)P->dw_col_groups, 1, 256, 1, 1, 0, st, args,
+                                         nullptr);
+  if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_fc_backward_w: launch failed: ") + hipGetErrorString(err));
   return E3X_OK;
 }
 

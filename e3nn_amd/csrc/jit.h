@@ -12,6 +12,7 @@ extern const char* const kTplUvwMfma;
 extern const char* const kTplUvwMfmaBf16;
 extern const char* const kTplUvwMfmaDw;
 extern const char* const kTplFcMfma;
+extern const char* const kTplFcDw;
 
 std::string cache_dir();
 

@@ -41,9 +41,12 @@ class _DenseFn(torch.autograd.Function):
             wt = (w.t() * (layer._scale * layer.h_out**0.5)).contiguous()
             gx = layer._bwd.forward(g, [wt])
         if ctx.needs_input_grad[1]:
-            ones = x.new_ones(x.shape[0], 1)
-            gw = layer._tp._plan(torch.float32).backward_w_uvw(x, ones, g, True).reshape(layer.h_in, layer.h_out)
-            gw = gw * (layer._scale * layer.h_in**0.5)  # the tensor product's path weight is 1 / sqrt(h_in)
+            if layer._fwd.has_backward_w:
+                gw = layer._fwd.backward_w(x, g)
+            else:  # wider than the dense weight-gradient kernel takes: the uvw weight gradient of the same layer
+                ones = x.new_ones(x.shape[0], 1)
+                gw = layer._tp._plan(torch.float32).backward_w_uvw(x, ones, g, True).reshape(layer.h_in, layer.h_out)
+                gw = gw * (layer._scale * layer.h_in**0.5)  # the tensor product's path weight is 1 / sqrt(h_in)
         return gx, gw, None
 
 
@@ -74,6 +77,7 @@ class _Layer(torch.nn.Module):
             if fwd.handle is None or bwd.handle is None:
                 self._fwd = self._bwd = False
             else:
+                fwd.prepare_backward_w()
                 self._fwd, self._bwd = fwd, bwd
         return self._fwd, self._bwd
 
@@ -136,6 +140,24 @@ class _FusedPlan:
                 _lib.lib().e3x_fc_plan_destroy(self.handle)
             except Exception:
                 pass
+
+    has_backward_w = False
+
+    def prepare_backward_w(self):
+        """Builds the weight-gradient kernel of a one-layer plan; ``has_backward_w`` stays False outside its limits."""
+        rc = _lib.lib().e3x_fc_plan_prepare_backward_w(self.handle)
+        if rc != _lib.ERR_INVALID:
+            _lib.check(rc)
+            self.has_backward_w = True
+
+    def backward_w(self, x, g):
+        hs = self._args[0]
+        gw = torch.empty(hs[0], hs[1], device=x.device, dtype=torch.float32)
+        with torch.cuda.device(x.device):
+            _lib.check(
+                _lib.lib().e3x_fc_backward_w(self.handle, _lib.ptr(x), _lib.ptr(g), _lib.ptr(gw), x.shape[0], _lib.stream_ptr(x.device))
+            )
+        return gw
 
     def forward(self, x, weights):
         L = _lib.lib()

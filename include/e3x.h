@@ -225,6 +225,13 @@ size_t e3x_fc_workspace_bytes(const e3x_fc_plan* plan);
 const char* e3x_fc_plan_key(const e3x_fc_plan* plan);
 int e3x_fc_forward(e3x_fc_plan* plan, const void* x, const void* const* weights, void* out, int64_t Z, void* workspace,
                    size_t workspace_bytes, void* stream);
+/* One-layer plans (n_hs = 2, no activation) only: grad_w[hs[0], hs[1]] = s * x^T grad_out with the layer's factor
+ * s = 1 / sqrt(hs[0] variance_in / variance_out), i.e. the gradient autograd derives for `weight` from
+ * `x @ (weight * s)` (e3nn/nn/_fc.py:38-48).  Batch slices are added with fp32 atomics (last-bit run-to-run
+ * variation); grad_w is fully overwritten.  hs[0] <= 256.  e3x_fc_plan_prepare_backward_w builds the kernel ahead of
+ * the first call (no GPU needed). */
+int e3x_fc_plan_prepare_backward_w(e3x_fc_plan* plan);
+int e3x_fc_backward_w(e3x_fc_plan* plan, const void* x, const void* grad_out, void* grad_w, int64_t Z, void* stream);
 
 /* Plain device copy dst[i] = src[i], n_bytes multiple of 16: the calibration kernel
  * for bandwidth counters (known traffic: n_bytes read + n_bytes written). */

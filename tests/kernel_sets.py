@@ -180,6 +180,7 @@ FUSED_FC_CASES = [
 def fused_fc_nets():
     from e3nn_amd import nn
 
+    torch.manual_seed(20240611)  # the weights are drawn at construction
     return [nn.FullyConnectedNet(hs, act, variance_in=vi, variance_out=vo, out_act=oa) for hs, act, oa, vi, vo in FUSED_FC_CASES]
 
 

@@ -112,6 +112,38 @@ def test_fully_connected_net_one_kernel(case):
     assert_close(out.reshape(-1, hs[-1]), want, what="one-kernel fc, batch dims")
 
 
+@pytest.mark.parametrize("case", range(len(ks.FUSED_FC_CASES)))
+def test_fully_connected_net_gradients(case):
+    """Under autograd the dense layers run on the one-layer kernels (x @ W, g @ W^T, x^T g): every gradient against
+    central differences of the float64 oracle along random directions, on a batch with ragged row tiles."""
+    hs, act, out_act, vi, vo = ks.FUSED_FC_CASES[case]
+    net = ks.fused_fc_nets()[case].to(DEV)
+    n_layers = len(hs) - 1
+    assert all(getattr(net, f"layer{i}").dense_plans()[0] for i in range(n_layers))
+    Z = 1237
+    x = seeded(Z, hs[0], seed=40 + case)
+    ws = [getattr(net, f"layer{i}").weight.detach().cpu().numpy().astype(np.float64) for i in range(n_layers)]
+    f = lambda xx, ww: onn.fc_forward(ww, xx, act, variance_in=vi, variance_out=vo, out_act=out_act)  # noqa: E731
+    xd = x.to(DEV).requires_grad_(True)
+    out = net(xd)
+    assert_close(out, f(x.numpy(), ws), what="layer-by-layer forward")
+    cot = seeded(Z, hs[-1], seed=60 + case)
+    out.backward(cot.to(DEV))
+    rng = np.random.default_rng(case)
+    x64, c64 = x.numpy().astype(np.float64), cot.numpy().astype(np.float64)
+    eps = 1e-6  # small: relu has kinks, and a step across one biases the difference quotient
+    v = rng.normal(size=x64.shape)
+    fd = ((f(x64 + eps * v, ws) - f(x64 - eps * v, ws)) * c64).sum() / (2 * eps)
+    assert float((xd.grad.cpu().double().numpy() * v).sum()) == pytest.approx(fd, rel=3e-4, abs=1e-3)
+    for i in range(n_layers):
+        dw = rng.normal(size=ws[i].shape)
+        wp = [w + eps * dw if k == i else w for k, w in enumerate(ws)]
+        wm = [w - eps * dw if k == i else w for k, w in enumerate(ws)]
+        fd = ((f(x64, wp) - f(x64, wm)) * c64).sum() / (2 * eps)
+        got = getattr(net, f"layer{i}").weight.grad.cpu().double().numpy()
+        assert float((got * dw).sum()) == pytest.approx(fd, rel=3e-4, abs=1e-3), f"layer {i}"
+
+
 def test_fully_connected_net_wide_hidden_layer():
     """Outside the limits of the fused kernel every layer runs on the tensor-product kernels, forward and backward."""
     fc = dict(ks.nn_modules())["fc_wide_hidden"].to(DEV)
