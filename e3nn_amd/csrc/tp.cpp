@@ -41,6 +41,8 @@ struct SubKernel {
   hipFunction_t fn_bwd_edge[kMaxDevices] = {nullptr};
   hipFunction_t fn_dw[kMaxDevices] = {nullptr};
   hipFunction_t fn_pack[kMaxDevices] = {nullptr};
+  // uvu: the edge-parallel backward kernel is a code object of its own (other lane layout), built on first use
+  std::unique_ptr<SubKernel> bwd;
 };
 
 struct e3x_plan {
@@ -172,7 +174,7 @@ std::vector<std::vector<int>> split_uvu_paths(const e3x_plan& P) {
   return parts;
 }
 
-int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src) {
+int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only = false) {
   int max_mul = 1;
   std::vector<char> used1(P.in1.size(), 0), usedo(P.out.size(), 0);
   long long unrolled = 0;
@@ -201,6 +203,14 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src) {
   };
   while (upl > 1 && !fits(upl)) upl /= 2;
   upl = env_int("E3X_UVU_UPL", upl);
+  // the backward kernel also holds the output gradient of its indices: one index per lane keeps it at several waves
+  // per SIMD (measured on the 32-channel l <= 2 set: 1.39 ms against 1.85 ms with four)
+  // -- as long as a wavefront still covers every index of an edge (one chunk: grad_x2 needs no atomics then)
+  if (bwd_only) {
+    int b = 1;
+    while (b < upl && (max_mul + b - 1) / b > 64) b *= 2;
+    upl = env_int("E3X_UVU_BWD_UPL", b);
+  }
   if (upl != 1 && upl != 2 && upl != 4) return fail(E3X_ERR_INVALID, "E3X_UVU_UPL must be 1, 2 or 4");
   for (size_t a = 0; a < P.in1.size(); ++a)
     if (used1[a] && P.in1[a].mul % upl) return fail(E3X_ERR_INVALID, "uvu kernel: multiplicity not divisible by UPL");
@@ -256,6 +266,7 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src) {
   s << "constexpr bool PREFETCH = " << (prefetch ? "true" : "false") << ";\n";
   K.waves_per_block = env_int("E3X_UVU_WAVES_PER_BLOCK", 4);
   s << "#define E3X_WAVES_PER_BLOCK " << K.waves_per_block << "\n";
+  if (bwd_only) s << "#define E3X_UVU_BWD_ONLY 1\n";
   // All loads of an edge ahead of its first product (a scheduling barrier in the edge loop) while the operands of an
   // edge leave room for three waves per SIMD; measured: + 3 % on the 32-channel l <= 2 set, + 13 % in bf16 storage,
   // - 2 % on the 128-channel l <= 3 set in fp32, whose operands alone take ~150 registers.
@@ -521,8 +532,6 @@ int load_functions(e3x_plan* P, int dev) {
     if (P->family == "uvu") {
       if (hipModuleGetFunction(&K->fn_fused[dev], mod, "e3x_uvu_fused") != hipSuccess)
         return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused missing from " + K->hsaco);
-      if (hipModuleGetFunction(&K->fn_bwd_edge[dev], mod, "e3x_uvu_bwd_edge") != hipSuccess)
-        return fail(E3X_ERR_HIP, "kernel e3x_uvu_bwd_edge missing from " + K->hsaco);
     }
     if (P->family == "uvw_mfma" && P->dtype == E3X_BF16) {
       if (hipModuleGetFunction(&K->fn_pack[dev], mod, "e3x_uvw_mfma_pack") != hipSuccess)
@@ -533,6 +542,37 @@ int load_functions(e3x_plan* P, int dev) {
         return fail(E3X_ERR_HIP, "kernel e3x_uvw_small_dw missing from " + K->hsaco);
     }
     K->module[dev] = mod;
+  }
+  return E3X_OK;
+}
+
+// builds (or finds in the cache) the backward code objects of a uvu plan
+int prepare_uvu_bwd(e3x_plan* P) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  for (auto& K : P->subs) {
+    if (K->bwd) continue;
+    std::unique_ptr<SubKernel> B(new SubKernel);
+    B->path_ids = K->path_ids;
+    std::string src;
+    int rc;
+    if ((rc = build_uvu_source(*P, *B, &src, true))) return rc;
+    if ((rc = e3x::get_code_object("uvu_bwd", src, &B->key, &B->hsaco))) return rc;
+    K->bwd = std::move(B);
+  }
+  return E3X_OK;
+}
+
+int load_uvu_bwd_functions(e3x_plan* P, int dev) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  for (auto& K : P->subs) {
+    SubKernel* B = K->bwd.get();
+    if (B->module[dev]) continue;
+    hipModule_t mod = nullptr;
+    hipError_t err = hipModuleLoad(&mod, B->hsaco.c_str());
+    if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + B->hsaco + ") failed: " + hipGetErrorString(err));
+    if (hipModuleGetFunction(&B->fn_bwd_edge[dev], mod, "e3x_uvu_bwd_edge") != hipSuccess)
+      return fail(E3X_ERR_HIP, "kernel e3x_uvu_bwd_edge missing from " + B->hsaco);
+    B->module[dev] = mod;
   }
   return E3X_OK;
 }
@@ -805,10 +845,11 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
     if (grad_x2 && (rc = e3x::fill_zero_bytes(grad_x2, (size_t)E * P->in2_dim * esz, st))) return rc;
     return E3X_OK;
   }
-  if ((rc = load_functions(P, dev))) return rc;
+  if ((rc = prepare_uvu_bwd(P))) return rc;
+  if ((rc = load_uvu_bwd_functions(P, dev))) return rc;
   int x2_atomic = 0;
   for (auto& K : P->subs)
-    if (K->chunks > 1) x2_atomic = 1;
+    if (K->bwd->chunks > 1) x2_atomic = 1;
   if (P->subs.size() > 1) x2_atomic = 1;
   if (grad_x2 && x2_atomic) {
     if (P->dtype != E3X_F32)
@@ -825,7 +866,8 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
   long long n_edges = E, n_src = num_src_nodes;
   void* args[] = {(void*)&x1,  (void*)&x2,     (void*)&w,       (void*)&grad_out,  (void*)&src,     (void*)&dst,
                   (void*)&idx64, (void*)&grad_w, (void*)&grad_x2, (void*)&x2_atomic, (void*)&n_edges, (void*)&n_src};
-  for (auto& K : P->subs) {
+  for (auto& F : P->subs) {
+    SubKernel* K = F->bwd.get();
     const int groups = 64 / K->lanes;
     const long long items = (E + groups - 1) / groups * K->chunks;
     const long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
@@ -844,7 +886,8 @@ extern "C" int e3x_tp_plan_prepare_backward_w(e3x_plan* P) {
     if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: fp32 storage only");
     return prepare_mfma_dw(P);
   }
-  return E3X_OK;  // the other families carry their gradient kernels in the forward code object
+  if (P->family == "uvu") return P->paths.empty() ? E3X_OK : prepare_uvu_bwd(P);
+  return E3X_OK;  // uvw_small carries its gradient kernel in the forward code object
 }
 
 extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2, const void* grad_out, void* grad_w,

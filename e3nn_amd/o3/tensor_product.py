@@ -483,6 +483,8 @@ class TensorProduct(torch.nn.Module):
             self._dense_equivalent()[0].compile_backward(dtype)
             return self
         self._grad_plan("x1", dtype)
+        if self._live_mode() == "uvu":
+            _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(self._plan(dtype).handle))
         if self._live_mode() == "uvw":
             self._grad_plan("x2", dtype)
             if dtype == torch.float32 and self.weight_numel:
