@@ -51,6 +51,11 @@ _SIGNATURES = {
     "e3x_index_check": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p]),
     "e3x_tp_gather_scatter": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_int64, c_int64, c_int64, c_void_p]),
+    "e3x_row_order_workspace_bytes": (c_size_t, [c_int64]),
+    "e3x_row_order_build": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p,
+                                    ctypes.POINTER(c_int32), c_void_p, c_size_t, c_void_p]),
+    "e3x_tp_gather_scatter_ordered": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                              c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     "e3x_tp_backward_w_x2": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     "e3x_tp_plan_prepare_backward_w": (c_int, [c_void_p]),

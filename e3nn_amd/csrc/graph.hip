@@ -57,6 +57,45 @@ __global__ __launch_bounds__(kBlock) void rowptr_kernel(const unsigned* __restri
   }
 }
 
+// key[n] = smallest source row among the in-edges of output row n (all ones for a row without edges), second[n] the
+// smallest one above it, ids[n] = n
+template <typename IdxT>
+__global__ __launch_bounds__(kBlock) void rowkey_kernel(const IdxT* __restrict__ src, const int* __restrict__ rowptr,
+                                                        const int* __restrict__ perm, long long N, long long n_src,
+                                                        unsigned* __restrict__ keys, unsigned* __restrict__ second,
+                                                        int* __restrict__ ids) {
+  for (long long n = (long long)blockIdx.x * kBlock + threadIdx.x; n < N; n += (long long)gridDim.x * kBlock) {
+    unsigned k1 = 0xffffffffu, k2 = 0xffffffffu;
+    for (int k = rowptr[n]; k < rowptr[n + 1]; ++k) {
+      long long s = (long long)src[perm ? perm[k] : k];
+      if (s < 0) s += n_src;  // gather semantics: negative indices wrap
+      const unsigned v = (unsigned)s;
+      if (v < k1) {
+        k2 = k1;
+        k1 = v;
+      } else if (v > k1 && v < k2) {
+        k2 = v;
+      }
+    }
+    keys[n] = k1;
+    second[n] = k2;
+    ids[n] = (int)n;
+  }
+}
+
+// counts the neighbours in the order that agree in BOTH smallest sources: chance alone makes rows share one
+// (a small id is the minimum of many rows), two in common mean overlapping source sets
+__global__ __launch_bounds__(kBlock) void order_score_kernel(const int* __restrict__ order, const unsigned* __restrict__ keys,
+                                                             const unsigned* __restrict__ second, long long N,
+                                                             int* __restrict__ score) {
+  int hits = 0;
+  for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i + 1 < N; i += (long long)gridDim.x * kBlock) {
+    const int a = order[i], b = order[i + 1];
+    if (keys[a] != 0xffffffffu && keys[a] == keys[b] && second[a] != 0xffffffffu && second[a] == second[b]) ++hits;
+  }
+  if (hits) atomicAdd(score, hits);
+}
+
 __global__ __launch_bounds__(kBlock) void fill_zero_kernel(int* p, int n) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -162,6 +201,57 @@ extern "C" int e3x_csr_build(const void* dst, int idx_bits, int64_t E, int64_t n
       hipStreamSynchronize(st) != hipSuccess)
     return e3x::fail(E3X_ERR_HIP, "e3x_csr_build: reading back the range flags failed");
   if (h_flags[0]) return e3x::fail(E3X_ERR_INDEX, "index out of range in scatter destination");
+  return E3X_OK;
+}
+
+extern "C" size_t e3x_row_order_workspace_bytes(int64_t num_nodes) {
+  if (num_nodes < 0) return 0;
+  const size_t n4 = align_up((size_t)(num_nodes > 0 ? num_nodes : 1) * 4, 256);
+  size_t temp = 0;
+  (void)rocprim::radix_sort_pairs(nullptr, temp, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr, (int*)nullptr,
+                                  (size_t)(num_nodes > 0 ? num_nodes : 1), 0, 32, (hipStream_t)0);
+  return 256 + 4 * n4 + align_up(temp, 256);  // score | keys_in | keys_out | ids_in | second | rocPRIM temp
+}
+
+extern "C" int e3x_row_order_build(const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm, int64_t E,
+                                   int64_t num_nodes, int64_t num_src_nodes, int32_t* row_order, int32_t* shared_pairs,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+  if (E < 0 || num_nodes < 0 || num_src_nodes < 0 || num_nodes >= (1LL << 31) || num_src_nodes >= (1LL << 31))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_row_order_build: sizes must fit in int32");
+  if (idx_bits != 32 && idx_bits != 64) return e3x::fail(E3X_ERR_INVALID, "e3x_row_order_build: idx_bits must be 32 or 64");
+  if (shared_pairs) *shared_pairs = 0;
+  if (num_nodes == 0) return E3X_OK;
+  if (!rowptr || !row_order || !workspace || (E > 0 && !src)) return e3x::fail(E3X_ERR_INVALID, "e3x_row_order_build: null pointer");
+  if (workspace_bytes < e3x_row_order_workspace_bytes(num_nodes))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_row_order_build: workspace smaller than e3x_row_order_workspace_bytes()");
+  hipStream_t st = (hipStream_t)stream;
+  const size_t n4 = align_up((size_t)num_nodes * 4, 256);
+  char* ws = (char*)workspace;
+  int* score = (int*)ws;
+  unsigned* keys_in = (unsigned*)(ws + 256);
+  unsigned* keys_out = (unsigned*)(ws + 256 + n4);
+  int* ids_in = (int*)(ws + 256 + 2 * n4);
+  unsigned* second = (unsigned*)(ws + 256 + 3 * n4);
+  void* temp = ws + 256 + 4 * n4;
+  size_t temp_bytes = workspace_bytes - 256 - 4 * n4;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(kBlock), 0, st, score, 1);
+  if (idx_bits == 64)
+    hipLaunchKernelGGL((rowkey_kernel<long long>), dim3(grid_for(num_nodes, kBlock)), dim3(kBlock), 0, st, (const long long*)src,
+                       rowptr, perm, (long long)num_nodes, (long long)num_src_nodes, keys_in, second, ids_in);
+  else
+    hipLaunchKernelGGL((rowkey_kernel<int>), dim3(grid_for(num_nodes, kBlock)), dim3(kBlock), 0, st, (const int*)src, rowptr,
+                       perm, (long long)num_nodes, (long long)num_src_nodes, keys_in, second, ids_in);
+  if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_row_order_build: launch failed");
+  // stable: rows with the same key keep their numbering
+  hipError_t err = rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, ids_in, row_order, (size_t)num_nodes, 0, 32, st);
+  if (err != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_row_order_build: radix sort failed");
+  if (shared_pairs) {
+    hipLaunchKernelGGL(order_score_kernel, dim3(grid_for(num_nodes, kBlock)), dim3(kBlock), 0, st, row_order, keys_in, second,
+                       (long long)num_nodes, score);
+    if (hipMemcpyAsync(shared_pairs, score, sizeof(int), hipMemcpyDeviceToHost, st) != hipSuccess ||
+        hipStreamSynchronize(st) != hipSuccess)
+      return e3x::fail(E3X_ERR_HIP, "e3x_row_order_build: reading back the score failed");
+  }
   return E3X_OK;
 }
 

@@ -788,6 +788,14 @@ extern "C" int e3x_tp_gather_scatter(e3x_plan* P, const void* node_x, const void
                                      const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
                                      void* out, int64_t E, int64_t num_src_nodes, int64_t num_out_nodes,
                                      void* stream) {
+  return e3x_tp_gather_scatter_ordered(P, node_x, edge_attr, w, src, idx_bits, rowptr, perm, nullptr, out, E,
+                                       num_src_nodes, num_out_nodes, stream);
+}
+
+extern "C" int e3x_tp_gather_scatter_ordered(e3x_plan* P, const void* node_x, const void* edge_attr, const void* w,
+                                             const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
+                                             const int32_t* row_order, void* out, int64_t E, int64_t num_src_nodes,
+                                             int64_t num_out_nodes, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: null plan");
   if (P->family != "uvu") return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: the plan must be all-uvu");
   if (P->shared_weights && P->weight_numel)
@@ -807,8 +815,8 @@ extern "C" int e3x_tp_gather_scatter(e3x_plan* P, const void* node_x, const void
   if ((rc = load_functions(P, dev))) return rc;
   int idx64 = idx_bits == 64;
   long long n_rows = num_out_nodes, n_src = num_src_nodes;
-  void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&w,    (void*)&out,    (void*)&src,
-                  (void*)&idx64,  (void*)&rowptr,    (void*)&perm, (void*)&n_rows, (void*)&n_src};
+  void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&w,         (void*)&out,    (void*)&src,  (void*)&idx64,
+                  (void*)&rowptr, (void*)&perm,      (void*)&row_order, (void*)&n_rows, (void*)&n_src};
   for (auto& K : P->subs) {
     const long long items = n_rows * K->chunks;
     long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;

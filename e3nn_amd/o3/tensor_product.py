@@ -113,10 +113,10 @@ class _Plan:
         out = torch.empty(edges.num_nodes, self.out_dim, dtype=table.dtype, device=table.device)
         with torch.cuda.device(table.device):
             _lib.check(
-                _lib.lib().e3x_tp_gather_scatter(
+                _lib.lib().e3x_tp_gather_scatter_ordered(
                     self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(gather_idx),
-                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(out),
-                    edges.num_edges, num_table_rows, edges.num_nodes, _lib.stream_ptr(table.device),
+                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(edges.row_order),
+                    _lib.ptr(out), edges.num_edges, num_table_rows, edges.num_nodes, _lib.stream_ptr(table.device),
                 )  # fmt: skip
             )
         return out

@@ -154,6 +154,26 @@ int e3x_tp_gather_scatter(e3x_plan* plan, const void* node_x, const void* edge_a
                           const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm, void* out,
                           int64_t E, int64_t num_src_nodes, int64_t num_out_nodes, void* stream);
 
+/* Processing order of the output rows for e3x_tp_gather_scatter_ordered: row_order[num_nodes] (int32 device array owned
+ * by the caller) is the permutation of the rows sorted, stably, by the smallest source row among their in-edges.  Rows
+ * that share their smallest source share most of their sources (a one-permutation min-hash of the neighbour sets), so
+ * rows processed next to each other gather the same rows of the node table and find them in L2, whatever the
+ * caller's node numbering; the results are bit-identical to the unordered call.  No counterpart in the reference
+ * (torch scatter_add_ has no processing order to choose).  rowptr / perm as built by e3x_csr_build; `workspace` is
+ * device scratch of at least e3x_row_order_workspace_bytes(num_nodes).  With a non-NULL `shared_pairs` (a HOST int)
+ * the call also counts the rows that agree with their successor in the order in their TWO smallest sources and
+ * synchronises the stream to return it: on a graph without neighbourhood structure (uniformly random edges) the
+ * count is a vanishing fraction of the rows, the order is a random permutation of them and is better not used. */
+size_t e3x_row_order_workspace_bytes(int64_t num_nodes);
+int e3x_row_order_build(const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm, int64_t E,
+                        int64_t num_nodes, int64_t num_src_nodes, int32_t* row_order, int32_t* shared_pairs,
+                        void* workspace, size_t workspace_bytes, void* stream);
+/* e3x_tp_gather_scatter with the output rows walked in `row_order` (NULL: in row order). */
+int e3x_tp_gather_scatter_ordered(e3x_plan* plan, const void* node_x, const void* edge_attr, const void* w,
+                                  const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
+                                  const int32_t* row_order, void* out, int64_t E, int64_t num_src_nodes,
+                                  int64_t num_out_nodes, void* stream);
+
 /* Gradients of the `uvu` product (plain: src = dst = NULL, row e of every table; fused: the edge lists
  * of e3x_tp_gather_scatter, unsorted) with respect to the per-sample weights and the second input:
  *   grad_w[E, weight_numel] (shared weights: one [weight_numel] vector summed over the edges with fp32 atomics),

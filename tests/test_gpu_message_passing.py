@@ -104,6 +104,45 @@ def test_run_to_run_bit_reproducible_and_prebuilt_edges():
     assert torch.equal(a, tp.forward_gather_scatter(node_x, attr, w, edges=edges))
 
 
+@pytest.mark.parametrize("idx", [torch.int32, torch.int64])
+def test_row_processing_order(idx):
+    """The rows are walked in the order of their smallest source row (stable), rows without edges last; the order
+    changes which row a wavefront takes, not what it computes: outputs are bit-identical with and without it."""
+    tp = ks.cfg3(True)
+    N, E = 900, 15_000
+    src, dst = random_graph(N, E, seed=5, dtype=idx)
+    dst = torch.where(dst % 7 == 3, (dst + 1) % N, dst)  # some rows keep no in-edge
+    src[::11] -= N  # negative gather indices wrap
+    node_x, attr, w = seeded(N, 288, seed=1).to(DEV), seeded(E, 9, seed=2).to(DEV), seeded(E, 352, seed=3).to(DEV)
+    edges = DstSortedEdges(src.to(DEV), dst.to(DEV), N, locality_order=True)
+    order = edges.row_order.cpu().long().numpy()
+    assert sorted(order.tolist()) == list(range(N))
+    key = np.full(N, 2**32 - 1, dtype=np.int64)
+    np.minimum.at(key, dst.long().numpy(), (src.long().numpy() % N))
+    assert np.array_equal(order, np.argsort(key, kind="stable"))
+    assert (key[order[-5:]] == 2**32 - 1).all()  # the test graph has more than five empty rows
+    plain = DstSortedEdges(src.to(DEV), dst.to(DEV), N, locality_order=False)
+    assert plain.row_order is None
+    a = tp.forward_gather_scatter(node_x, attr, w, edges=edges)
+    b = tp.forward_gather_scatter(node_x, attr, w, edges=plain)
+    assert torch.equal(a, b)
+    assert not a[torch.from_numpy(key == 2**32 - 1).to(DEV)].any()
+    # the transposed edge list (for the gradient with respect to the node features) inherits the choice
+    src0 = src % N
+    assert DstSortedEdges(src0.to(DEV), dst.to(DEV), N, locality_order=True).transposed().row_order is not None
+    assert DstSortedEdges(src0.to(DEV), dst.to(DEV), N, locality_order=False).transposed().row_order is None
+    # default ("auto"): uniformly random edges have no neighbourhoods to exploit and keep the plain row order ...
+    auto = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    assert auto.row_order is None and auto.locality_score < 0.02
+    # ... a radius graph (random node numbering) has them
+    g = torch.Generator().manual_seed(1)
+    pos = torch.rand(1500, 3, generator=g) * 10.0
+    near = (torch.cdist(pos, pos) < 1.6) & ~torch.eye(1500, dtype=torch.bool)
+    rs, rd = near.nonzero(as_tuple=True)
+    geo = DstSortedEdges(rs.to(idx).to(DEV), rd.to(idx).to(DEV), 1500)
+    assert geo.row_order is not None and geo.locality_score > 0.1, geo.locality_score
+
+
 @pytest.mark.parametrize("maker,N,E,idx", [
     (lambda: ks.cfg3(True), 700, 26_000, torch.int64),
     (lambda: ks.cfg3(False), 300, 9_000, torch.int64),
