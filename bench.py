@@ -25,8 +25,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # L2-miss traffic of one e3x_uvu_fused launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt): 3376908 KiB fetched + 56251 KiB written
-NEQUIP_TRAFFIC_BYTES = (3376908 + 56251) * 1024
+# scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt): 3374122 KiB fetched + 56251 KiB written
+NEQUIP_TRAFFIC_BYTES = (3374122 + 56251) * 1024
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 
