@@ -267,6 +267,10 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only 
   K.waves_per_block = env_int("E3X_UVU_WAVES_PER_BLOCK", 4);
   s << "#define E3X_WAVES_PER_BLOCK " << K.waves_per_block << "\n";
   if (bwd_only) s << "#define E3X_UVU_BWD_ONLY 1\n";
+  // coefficient folded into the edge attribute (see accumulate_edge); measured on one GPU, old -> new: 32 channels
+  // l <= 2 at four indices per lane 0.637 -> 0.635 ms (degree 354: 4.91 -> 4.84), 128 channels l <= 3 in bf16 storage
+  // 1.60 -> 1.48 ms, in fp32 at two indices per lane 1.68 -> 1.77 ms
+  if (env_int("E3X_UVU_FOLD", (upl == 4 || P.dtype == E3X_BF16) ? 1 : 0)) s << "#define E3X_UVU_FOLD 1\n";
   // All loads of an edge ahead of its first product (a scheduling barrier in the edge loop) while the operands of an
   // edge leave room for three waves per SIMD; measured: + 3 % on the 32-channel l <= 2 set, + 13 % in bf16 storage,
   // - 2 % on the 128-channel l <= 3 set in fp32, whose operands alone take ~150 registers.
