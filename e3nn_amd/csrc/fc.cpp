@@ -143,7 +143,6 @@ extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, 
   s << "};\nconstexpr float WSCALE[NL] = {";
   for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << fstr(wscale[l]);
   s << "};\nconstexpr float OUT_POST = " << fstr(out_post) << ";\n";
-  if (const char* v = std::getenv("E3X_FC_EXP")) s << "#define E3X_FC_EXP " << std::atoi(v) << "\n";
   s << "constexpr int RS = " << rs << ", WAVES = " << waves << ";\n}  // namespace cfg\n";
   const std::string src = s.str() + e3x::kTplCommon + e3x::kTplFcMfma;
   int rc = e3x::get_code_object("fc_mfma", src, &P->key, &P->hsaco);
