@@ -176,3 +176,51 @@ def test_dense_uvw_equivalent_of_general_modes(name):
     got = otp.tp_forward(oracle_spec(dense_tp, irrep_normalization="none", path_normalization="none",
                                      user_path_weights=[t.path_weight**2 for t in tp.instructions]), x1.numpy(), x2.numpy(), wd.numpy())
     np.testing.assert_allclose(got, want, rtol=1e-10, atol=1e-12)
+
+
+def test_fully_connected_plans_need_no_gpu_and_reject_what_the_kernel_cannot_hold():
+    """Plans of the fused network kernel are built (or found in the cache) without a GPU; widths beyond the register
+    and LDS budgets, unknown activations and empty layer lists are E3X_ERR_INVALID, which the module answers by
+    running layer by layer."""
+    import ctypes
+
+    from e3nn_amd import nn
+    from e3nn_amd.nn.fc import _FusedPlan
+
+    L = _lib.lib()
+    plan = _FusedPlan([8, 64, 352], "silu", False, 1, 1)
+    assert plan.handle is not None and plan.key.startswith("fc_mfma_")
+    assert plan.workspace_bytes == (8 * 64 + 64 * 352) * 4  # packed weights: widths already multiples of 8 / 32
+    assert _FusedPlan([5, 100, 50], "tanh", False, 1, 1).workspace_bytes == (8 * 128 + 128 * 64) * 4  # zero padded
+    for hs in ([8, 512, 16], [128, 256, 8], [600, 8]):
+        bad = _FusedPlan(hs, "silu", False, 1, 1)
+        assert bad.handle is None and "e3x_fc_plan_create" in bad.reason
+    h = ctypes.c_void_p()
+    arr = (ctypes.c_int32 * 2)(4, 4)
+    assert L.e3x_fc_plan_create(arr, 2, 99, 1.0, 0, 1.0, 1.0, 0, ctypes.byref(h)) == _lib.ERR_INVALID  # activation
+    assert L.e3x_fc_plan_create(arr, 1, 1, 1.0, 0, 1.0, 1.0, 0, ctypes.byref(h)) == _lib.ERR_INVALID  # no layer
+    assert L.e3x_fc_plan_create(arr, 2, 1, 1.0, 0, -1.0, 1.0, 0, ctypes.byref(h)) == _lib.ERR_INVALID  # variance
+    assert L.e3x_fc_plan_create(arr, 2, 1, 1.0, 0, 1.0, 1.0, 1, ctypes.byref(h)) == _lib.ERR_INVALID  # bf16 storage
+    # the weight gradient exists for one-layer plans only
+    assert L.e3x_fc_plan_prepare_backward_w(plan.handle) == _lib.ERR_INVALID
+    one = _FusedPlan([64, 352], "identity", False, 1, 1)
+    one.prepare_backward_w()
+    assert one.has_backward_w
+    net = nn.FullyConnectedNet([8, 512, 16], torch.nn.functional.silu)
+    assert net.fused_plan().handle is None and not net.layer0.dense_plans()[0]
+    assert [tuple(p.shape) for p in net.parameters()] == [(8, 512), (512, 16)]  # the reference's parameters
+    assert list(dict(net.named_parameters())) == ["layer0.weight", "layer1.weight"]
+
+
+def test_row_order_entry_point_validates_its_arguments():
+    import ctypes
+
+    L = _lib.lib()
+    assert L.e3x_row_order_workspace_bytes(-1) == 0
+    small, large = L.e3x_row_order_workspace_bytes(10), L.e3x_row_order_workspace_bytes(1_000_000)
+    assert 0 < small < large and large >= 4 * 4 * 1_000_000
+    pairs = ctypes.c_int32(7)
+    null = ctypes.c_void_p(0)
+    assert L.e3x_row_order_build(null, 16, null, null, 0, 4, 4, null, ctypes.byref(pairs), null, 0, null) == _lib.ERR_INVALID
+    assert L.e3x_row_order_build(null, 32, null, null, 0, 0, 0, null, ctypes.byref(pairs), null, 0, null) == 0 and pairs.value == 0
+    assert L.e3x_row_order_build(null, 32, null, null, 0, 4, 4, null, None, null, 0, null) == _lib.ERR_INVALID  # null pointers
