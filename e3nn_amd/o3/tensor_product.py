@@ -190,16 +190,21 @@ class _TensorProductFn(torch.autograd.Function):
                 g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, w)
             if need2 or (needw and tp.weight_numel):
                 if tp.shared_weights and needw and tp.weight_numel and x1.dtype != torch.float32:
-                    raise NotImplementedError("the gradient of shared uvu weights has an fp32 kernel only")
-                gw, g2 = tp._plan(x1.dtype).backward_w_x2(x1, x2, w, g, None, None, needw and tp.weight_numel > 0, need2, x1.shape[0])
+                    # the sum over the batch is taken by fp32 atomics: the fp32 kernel on widened copies
+                    gw, g2 = tp._plan(torch.float32).backward_w_x2(
+                        x1.float(), x2.float(), w.float(), g.float(), None, None, True, need2, x1.shape[0]
+                    )
+                    gw = gw.to(x1.dtype)
+                    g2 = None if g2 is None else g2.to(x1.dtype)
+                else:
+                    gw, g2 = tp._plan(x1.dtype).backward_w_x2(x1, x2, w, g, None, None, needw and tp.weight_numel > 0, need2, x1.shape[0])
         elif mode == "uvw":
             if needw and tp.weight_numel:
                 if x1.dtype != torch.float32:
-                    raise NotImplementedError(
-                        "the weight gradient of uvw tensor products has an fp32 kernel only; call "
-                        "weight.requires_grad_(False) to differentiate with respect to the inputs only"
-                    )
-                gw = tp._plan(x1.dtype).backward_w_uvw(x1, x2, g, tp.shared_weights)
+                    # the weight-gradient kernels read fp32 rows: widened copies of the operands, result in storage type
+                    gw = tp._plan(torch.float32).backward_w_uvw(x1.float(), x2.float(), g.float(), tp.shared_weights).to(x1.dtype)
+                else:
+                    gw = tp._plan(x1.dtype).backward_w_uvw(x1, x2, g, tp.shared_weights)
             if need1:
                 g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, _permuted_weights(tp, w, (2, 1, 0)))
             if need2:
@@ -485,10 +490,12 @@ class TensorProduct(torch.nn.Module):
         self._grad_plan("x1", dtype)
         if self._live_mode() == "uvu":
             _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(self._plan(dtype).handle))
+            if dtype != torch.float32 and self.shared_weights and self.weight_numel:  # summed over the batch in fp32
+                _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(self._plan(torch.float32).handle))
         if self._live_mode() == "uvw":
             self._grad_plan("x2", dtype)
-            if dtype == torch.float32 and self.weight_numel:
-                _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(self._plan(dtype).handle))
+            if self.weight_numel:  # the weight gradient always runs on the fp32 plan
+                _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(self._plan(torch.float32).handle))
         return self
 
     def __getstate__(self):

@@ -29,6 +29,10 @@ def golden_meta():
         return json.load(f)
 
 
+# backward pass in bf16 storage: a matrix-core uvw set, shared uvu weights, per-edge uvu weights
+BACKWARD_BF16_CASES = ["mfma_small", "uvu_shared_v2", "cfg3_merged"]
+
+
 def tp_from_meta(m, **extra):
     upw = m.get("user_path_weights", [1.0] * len(m["instructions"]))
     ins = [tuple(t[:5]) + (pw,) for t, pw in zip(m["instructions"], upw)]
@@ -221,6 +225,8 @@ def prebuild(verbose=True, workers=6):
         keys = [tp._plan(dt).key for dt in dtypes]
         if backward:
             tp.compile_backward(torch.float32)
+        if name.replace("kernel ", "") in BACKWARD_BF16_CASES:
+            tp.compile_backward(torch.bfloat16)
         return name, keys
 
     with ThreadPoolExecutor(max_workers=workers) as pool:

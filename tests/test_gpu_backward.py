@@ -251,3 +251,23 @@ def test_spherical_harmonics_gradient_any_l_list(ls, normalize, normalization):
         have = (got * v).sum(axis=1)
         scale = max(1.0, float(np.abs(want).max()))
         assert np.abs(have - want).max() < 2e-4 * scale, (np.abs(have - want).max(), scale)
+
+
+@pytest.mark.parametrize("maker,Z,shared", [(ks.mfma_small, 300, True), (lambda: ks.golden_tp("uvu_shared_v2"), 200, True),
+                                            (lambda: ks.cfg3(True), 130, False)])  # fmt: skip
+def test_gradients_in_bf16_storage(maker, Z, shared):
+    """bf16 storage, fp32 accumulation: every gradient against float64 autograd of the oracle on the same (bf16-rounded)
+    inputs, to the bf16 tolerance rel 1e-2 of the largest entry (inputs, outputs and gradients are rounded to bf16)."""
+    tp = maker().to(DEV)
+    spec = oracle_spec(tp)
+    bf = torch.bfloat16
+    wshape = (tp.weight_numel,) if shared else (Z, tp.weight_numel)
+    x1, x2 = seeded(Z, tp.irreps_in1.dim, seed=1).to(bf), seeded(Z, tp.irreps_in2.dim, seed=2).to(bf)
+    w, cot = seeded(*wshape, seed=3).to(bf), seeded(Z, tp.irreps_out.dim, seed=4).to(bf)
+    _, (r1, r2, rw) = _oracle_grads(lambda a, b, c: tp_forward_torch(spec, a, b, c), (x1.float(), x2.float(), w.float()), cot.float())
+    a, b, c = (t.to(DEV).requires_grad_(True) for t in (x1, x2, w))
+    tp(a, b, c).backward(cot.to(DEV))
+    for got, ref, what in ((a.grad, r1, "d/dx1"), (b.grad, r2, "d/dx2"), (c.grad, rw, "d/dw")):
+        assert got.dtype == bf
+        err = (got.float().cpu().double() - ref).abs().max().item()
+        assert err <= 2e-2 * max(1.0, ref.abs().max().item()), f"{what}: {err} vs {ref.abs().max().item()}"
