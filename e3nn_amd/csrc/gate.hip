@@ -141,6 +141,50 @@ __global__ __launch_bounds__(kCols* kRows) void gate_bwd_kernel(Tables t, const 
   }
 }
 
+// One activation over whole contiguous rows (an Activation on n x0e, the hidden layer of a radial network): the
+// tensor is one flat array, 16 bytes per thread and access.
+__global__ __launch_bounds__(256) void act_flat_fwd_kernel(int kind, float cst, const float4* __restrict__ x,
+                                                           float4* __restrict__ out, long long n4) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n4; i += (long long)gridDim.x * 256) {
+    const float4 v = x[i];
+    float f[4], df;
+    activation(kind, v.x, f[0], df);
+    activation(kind, v.y, f[1], df);
+    activation(kind, v.z, f[2], df);
+    activation(kind, v.w, f[3], df);
+    out[i] = make_float4(cst * f[0], cst * f[1], cst * f[2], cst * f[3]);
+  }
+}
+
+__global__ __launch_bounds__(256) void act_flat_bwd_kernel(int kind, float cst, const float4* __restrict__ x,
+                                                           const float4* __restrict__ gout, float4* __restrict__ gx,
+                                                           long long n4) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n4; i += (long long)gridDim.x * 256) {
+    const float4 v = x[i], g = gout[i];
+    float f, d[4];
+    activation(kind, v.x, f, d[0]);
+    activation(kind, v.y, f, d[1]);
+    activation(kind, v.z, f, d[2]);
+    activation(kind, v.w, f, d[3]);
+    gx[i] = make_float4(cst * d[0] * g.x, cst * d[1] * g.y, cst * d[2] * g.z, cst * d[3] * g.w);
+  }
+}
+
+// true when the tables describe one activation applied to every column of contiguous, 16-byte aligned rows
+bool is_flat(const Tables& t, int64_t Z, int64_t in_dim, int64_t out_dim, const void* a, const void* b, const void* c) {
+  if (t.n_gate != 0 || t.n_act != 1 || in_dim != out_dim) return false;
+  const e3x_act_block& k = t.act[0];
+  if (k.offset_in != 0 || k.offset_out != 0 || k.count != in_dim) return false;
+  if ((Z * in_dim) % 4) return false;
+  return ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) && (!c || (uintptr_t)c % 16 == 0);
+}
+
+unsigned flat_grid(long long n4) {
+  long long b = (n4 + 255) / 256;
+  if (b > 256 * 32) b = 256 * 32;
+  return (unsigned)(b < 1 ? 1 : b);
+}
+
 // grid of the column-walk kernels: all column blocks, enough row blocks for a few workgroups per CU
 dim3 walk_grid(int64_t Z, int64_t dim) {
   const long long cb = (dim + kCols - 1) / kCols;
@@ -191,6 +235,13 @@ extern "C" int e3x_gate_forward(const e3x_act_block* acts, int32_t n_acts, const
   if (Z < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: negative batch");
   if (Z == 0 || out_dim == 0) return E3X_OK;
   if (!x || !out) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: null pointer");
+  if (is_flat(t, Z, in_dim, out_dim, x, out, nullptr)) {
+    const long long n4 = Z * in_dim / 4;
+    hipLaunchKernelGGL(act_flat_fwd_kernel, dim3(flat_grid(n4)), dim3(256), 0, (hipStream_t)stream, t.act[0].act, t.act[0].cst,
+                       (const float4*)x, (float4*)out, n4);
+    if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_forward: kernel launch failed");
+    return E3X_OK;
+  }
   hipLaunchKernelGGL(gate_fwd_kernel, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
                      (float*)out, (long long)Z, (int)in_dim, (int)out_dim);
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_forward: kernel launch failed");
@@ -207,6 +258,13 @@ extern "C" int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, cons
   if (Z < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: negative batch");
   if (Z == 0 || in_dim == 0) return E3X_OK;
   if (!x || !grad_out || !grad_x) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: null pointer");
+  if (is_flat(t, Z, in_dim, out_dim, x, grad_out, grad_x)) {
+    const long long n4 = Z * in_dim / 4;
+    hipLaunchKernelGGL(act_flat_bwd_kernel, dim3(flat_grid(n4)), dim3(256), 0, (hipStream_t)stream, t.act[0].act, t.act[0].cst,
+                       (const float4*)x, (const float4*)grad_out, (float4*)grad_x, n4);
+    if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward: kernel launch failed");
+    return E3X_OK;
+  }
   hipLaunchKernelGGL(gate_bwd_kernel, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
                      (const float*)grad_out, (float*)grad_x, (long long)Z, (int)in_dim, (int)out_dim);
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward: kernel launch failed");
