@@ -184,6 +184,11 @@ class Gate(_BlockModule):
         # (_gate.py:10-24,103-116)
         names_s, names_g = [activation_name(a) for a in act_scalars], [activation_name(a) for a in act_gates]
         groups = [irreps_scalars, irreps_gates, irreps_gated]
+        # the reference multiplies gates and gated irreps with an ElementwiseTensorProduct submodule `mul`, whose
+        # (empty) weight and output mask are in its state_dict
+        self.mul = torch.nn.Module()
+        self.mul.register_buffer("weight", torch.Tensor())
+        self.mul.register_buffer("output_mask", torch.ones(Irreps(irreps_gated).dim))
         simplified = [g.simplify() for g in groups]
         if any(len(s) != len(g) for s, g in zip(simplified[:2], groups[:2])):
             raise NotImplementedError("Gate: give irreps_scalars and irreps_gates in simplified form (one entry per irrep run)")

@@ -57,9 +57,10 @@ class _Layer(torch.nn.Module):
         self.h_in, self.h_out, self.var_in, self.var_out = h_in, h_out, var_in, var_out
         self._act_name = None if act is None else activation_name(act)
         # path weight of the tensor product: 1 / sqrt(h_in); the variance factors of _fc.py:41-48 ride on top
-        self._tp = TensorProduct(
+        # (kept out of the module tree: the reference's layer has `weight` only in its state_dict)
+        object.__setattr__(self, "_tp", TensorProduct(
             f"{h_in}x0e", "0e", f"{h_out}x0e", [(0, 0, 0, "uvw", True)], internal_weights=False, shared_weights=True
-        )
+        ))  # fmt: skip
         self.act = None if act is None else Activation(f"{h_out}x0e", [self._act_name])
         # _fc.py:41-48: x @ W / sqrt(h_in var_in) before an activation, x @ W / sqrt(h_in var_in / var_out) without
         self._scale = (h_in * var_in) ** -0.5 if act is not None else (h_in * var_in / var_out) ** -0.5

@@ -91,10 +91,11 @@ class Linear(torch.nn.Module):
 
         # the same map as a tensor product with "0e": the reference's own normalisation formula for TensorProduct
         # (component / element or path) reproduces alpha^(-1/2) once the delta / sqrt(2l+1) of the 3j tensor is counted
-        self._tp = TensorProduct(
+        # (kept out of the module tree: the reference's Linear has no such submodule in its state_dict)
+        object.__setattr__(self, "_tp", TensorProduct(
             irreps_in, "0e", irreps_out, [(i, 0, o, "uvw", True) for i, o in instructions],
             path_normalization=path_normalization, internal_weights=False, shared_weights=shared_weights,
-        )  # fmt: skip
+        ))  # fmt: skip
         self.weight_numel = self._tp.weight_numel
         self.bias_numel = sum(sl.stop - sl.start for sl in self._bias_slices)
         if internal_weights and self.weight_numel > 0:

@@ -244,6 +244,15 @@ class _GatherScatterFn(torch.autograd.Function):
         return g1, g2, gw, None, None
 
 
+class _Constants(torch.nn.Module):
+    """Holder of constant buffers under the names the reference's generated modules give them."""
+
+    def __init__(self, tensors) -> None:
+        super().__init__()
+        for name, value in tensors.items():
+            self.register_buffer(name, value)
+
+
 class TensorProduct(torch.nn.Module):
     r"""Tensor product with parametrised paths (see the reference docstring, ``_tensor_product.py:25-194``).
 
@@ -366,6 +375,44 @@ class TensorProduct(torch.nn.Module):
             output_mask = torch.ones(0)
         self.register_buffer("output_mask", output_mask)
         self._plans = {}
+        # The reference keeps the Wigner tensors (and the index pairs of the triangular modes) as buffers of its
+        # generated modules, so they are part of its state_dict.  The kernels here carry those constants as
+        # immediates; the buffers exist so that checkpoints load in both directions with strict=True.
+        self._compiled_main_left_right = _Constants(self._reference_constants(right=False))
+        if compile_right:
+            self._compiled_main_right = _Constants(self._reference_constants(right=True))
+
+    def _reference_constants(self, right: bool):
+        """Names and values of the buffers of the reference's generated module (``_codegen.py:143-144,289-325`` for
+        ``forward``, ``:514-515,560-641`` for ``right``): a tensor ``_w3j_l1_l2_l3`` for every instruction whose
+        contraction is not one of the specialised einsums, ``_triu_indices_n`` for the modes over pairs u < v."""
+        from .wigner import wigner_3j
+
+        spec = self._specialized_code
+        out = {}
+        for t in self.instructions:
+            m1, m2, mo = self.irreps_in1[t.i_in1], self.irreps_in2[t.i_in2], self.irreps_out[t.i_out]
+            if m1.dim == 0 or m2.dim == 0 or mo.dim == 0:
+                continue
+            l = (m1.ir.l, m2.ir.l, mo.ir.l)
+            mode, special = t.connection_mode, spec and 0 in l
+            if mode in ("uvu<v", "u<vw"):
+                if right:
+                    raise NotImplementedError  # as the reference (_codegen.py:620-623)
+                uses = True
+            elif mode == "uvuv" or (mode == "uuw" and (right or not t.has_weight)):
+                uses = True
+            elif mode in ("uvu", "uvv") and not t.has_weight and (right or mode == "uvu"):
+                uses = True
+            elif mode == "uuu":
+                uses = not (special or (spec and l == (1, 1, 1) and not right))
+            else:
+                uses = not special
+            if uses:
+                out.setdefault(f"_w3j_{l[0]}_{l[1]}_{l[2]}", wigner_3j(*l))
+            if mode in ("uvu<v", "u<vw"):
+                out.setdefault(f"_triu_indices_{m1.mul}", torch.triu_indices(m1.mul, m1.mul, 1))
+        return out
 
     # ------------------------------------------------------------------ plans
     def _kernel_instructions(self):

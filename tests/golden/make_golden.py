@@ -18,6 +18,9 @@ expected outputs only:
                    gather -> TensorProduct -> scatter
 * nn_cases.npz/json  (``python tests/golden/make_golden.py nn``) o3.Linear, nn.Activation, nn.Gate,
                    nn.FullyConnectedNet and the v2106 Convolution: parameters, inputs, outputs, irreps strings
+* state_dict_keys.json  (``python tests/golden/make_golden.py state``) names and shapes of the entries of
+                   ``TensorProduct.state_dict()`` (weights, output mask and the constant buffers of the generated
+                   modules) for a list of constructor arguments
 """
 import json
 import os
@@ -85,6 +88,57 @@ def describe(tp):
         # one flag per output irrep block (the mask is constant inside a block)
         "output_mask_blocks": [int(tp.output_mask[s.start]) if s.stop > s.start else -1 for s in tp.irreps_out.slices()],
     }
+
+
+STATE_CASES = [
+    # (name, irreps_in1, irreps_in2, irreps_out, instructions, kwargs)
+    ("fctp_l2", "2x0e+2x1o+2x2e", "0e+1o+2e", "2x0e+2x1o+2x2e", None, {}),
+    ("fctp_l2_unspecialized", "2x0e+2x1o+2x2e", "0e+1o+2e", "2x0e+2x1o+2x2e", None, {"_specialized_code": False}),
+    ("fctp_right", "2x0e+2x1o", "0e+1o", "2x0e+2x1o+1x2e", None, {"compile_right": True}),
+    ("uvu_mixed", "3x0e+3x1o", "2x0e+2x1o", "3x0e+3x1o",
+     [(0, 0, 0, "uvu", True), (0, 1, 1, "uvu", True), (1, 0, 1, "uvu", False), (1, 1, 0, "uvu", True), (1, 1, 0, "uvu", False)], {}),
+    ("modes", "3x1o+3x2e+3x0e", "3x1o+3x0e", "3x1e+3x2e+9x1o+2x2o+3x1o+3x0e+1x0e",
+     [(0, 0, 0, "uuu", True), (1, 1, 1, "uuu", False), (0, 1, 2, "uvuv", True), (1, 0, 3, "uuw", True), (0, 1, 4, "uvv", True),
+      (2, 1, 5, "uuu", False), (0, 0, 6, "uuw", False), (1, 1, 1, "uvv", False)], {}),
+    ("modes_right", "3x1o+3x2e", "3x1o+3x0e", "3x1e+3x2e+9x1o+2x2o+3x1o",
+     [(0, 0, 0, "uuu", True), (1, 1, 1, "uuu", False), (0, 1, 2, "uvuv", True), (1, 0, 3, "uuw", True), (0, 1, 4, "uvv", True)],
+     {"compile_right": True}),
+    ("triangular", "4x1o+4x0e", "4x1o+4x0e", "6x1e+3x2e+6x0e", [(0, 0, 0, "uvu<v", True), (0, 0, 1, "u<vw", True), (1, 1, 2, "uvu<v", False)], {}),
+    ("empty_paths", "2x0e+0x1o", "1o", "2x1o+3x2e", [(0, 0, 0, "uvu", True), (1, 0, 1, "uvw", True)], {}),
+    ("external_weights", "2x0e+2x1o", "0e+1o", "2x0e+2x1o", None, {"internal_weights": False, "shared_weights": False}),
+]
+
+
+def main_state():
+    ref = sys.argv[2] if len(sys.argv) > 2 else "/root/reference"
+    o3 = import_reference(ref)
+    out = {}
+    for name, i1, i2, io, ins, kw in STATE_CASES:
+        tp = o3.FullyConnectedTensorProduct(i1, i2, io, **kw) if ins is None else o3.TensorProduct(i1, i2, io, ins, **kw)
+        out[name] = {
+            "args": [i1, i2, io, ins, kw],
+            "state_dict": {k: list(v.shape) for k, v in tp.state_dict().items()},
+        }
+    # node-wise blocks: module constructors by name, positional arguments as JSON
+    from e3nn import nn
+    from e3nn.nn.models.v2106.points_convolution import Convolution
+
+    silu, sigmoid, tanh = torch.nn.functional.silu, torch.sigmoid, torch.tanh
+    modules = {
+        "linear": (o3.Linear, ["2x0e+2x1o", "3x0e+1x1o"], {"biases": True}),
+        "linear_l2": (o3.Linear, ["2x0e+2x1o+2x2e", "3x0e+1x1o+2x2e"], {}),
+        "fc": (nn.FullyConnectedNet, [[4, 8, 2], silu], {}),
+        "gate": (nn.Gate, ["4x0e+2x0o", [silu, tanh], "3x0e", [sigmoid], "2x1o+1x2e"], {}),
+        "activation": (nn.Activation, ["4x0e+2x0o", [silu, tanh]], {}),
+        "convolution_l1": (Convolution, ["4x0e+4x1o", "2x0e", "0e+1o", "4x0e+4x1o", [3, 8], 3.0], {}),
+        "convolution_l2": (Convolution, ["4x0e+4x1o+4x2e", "2x0e", "0e+1o+2e", "4x0e+4x1o+4x2e", [3, 8], 3.0], {}),
+    }
+    for name, (ctor, args, kw) in modules.items():
+        m = ctor(*args, **kw)
+        out["module_" + name] = {"state_dict": {k: list(v.shape) for k, v in m.state_dict().items()}}
+    with open(os.path.join(HERE, "state_dict_keys.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    print("wrote state_dict_keys.json:", {k: len(v["state_dict"]) for k, v in out.items()})
 
 
 def main():
@@ -285,7 +339,9 @@ def main_nn(ref="/root/reference"):
 
 
 if __name__ == "__main__":
-    if len(sys.argv) > 1 and sys.argv[1] == "nn":
+    if len(sys.argv) > 1 and sys.argv[1] == "state":
+        main_state()
+    elif len(sys.argv) > 1 and sys.argv[1] == "nn":
         main_nn(*sys.argv[2:])
     else:
         main()

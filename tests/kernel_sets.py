@@ -206,8 +206,10 @@ def prebuild(verbose=True, workers=6):
     jobs = []
     for name, mod in nn_modules() + [(f"fused_fc{i}", net) for i, net in enumerate(fused_fc_nets())]:
         for sub in mod.modules():
-            if isinstance(sub, o3.TensorProduct):
-                jobs.append((f"module {name}", sub, (torch.float32,), True))
+            inner = sub.__dict__.get("_tp")  # Linear and the dense layers keep theirs out of the module tree
+            for tp in (sub, inner):
+                if isinstance(tp, o3.TensorProduct):
+                    jobs.append((f"module {name}", tp, (torch.float32,), True))
             if isinstance(sub, nn.FullyConnectedNet):
                 jobs.append((f"module {name} (one kernel)", sub, None, False))
     for name, tp, dtypes in all_tensor_products():

@@ -113,7 +113,8 @@ def test_builders_match_reference_golden(golden_tp):
 
 def test_module_state_and_api_details():
     tp = ks.cfg1()
-    assert set(tp.state_dict()) == {"weight", "output_mask"}
+    # weight, mask and the Wigner buffers of the reference's generated module (see the state_dict test below)
+    assert set(tp.state_dict()) == {"weight", "output_mask", "_compiled_main_left_right._w3j_1_1_2", "_compiled_main_left_right._w3j_1_2_1"}
     assert repr(tp).startswith("FullyConnectedTensorProduct(16x0e+16x1o x 1x0e+1x1o+1x2e -> 16x0e+16x1o+16x2e | 1792 paths | 1792 weights")
     views = list(tp.weight_views())
     assert [tuple(v.shape) for v in views] == [(16, 1, 16)] * 7
@@ -224,3 +225,41 @@ def test_row_order_entry_point_validates_its_arguments():
     assert L.e3x_row_order_build(null, 16, null, null, 0, 4, 4, null, ctypes.byref(pairs), null, 0, null) == _lib.ERR_INVALID
     assert L.e3x_row_order_build(null, 32, null, null, 0, 0, 0, null, ctypes.byref(pairs), null, 0, null) == 0 and pairs.value == 0
     assert L.e3x_row_order_build(null, 32, null, null, 0, 4, 4, null, None, null, 0, null) == _lib.ERR_INVALID  # null pointers
+
+
+def test_state_dict_keys_match_the_reference():
+    """Names and shapes of every state_dict entry as the reference has them (fixture written from the reference's
+    modules): weights, output masks, the Wigner / index buffers of its generated modules, the `mul` submodule of the
+    gate -- so that checkpoints load with strict=True in both directions."""
+    import json
+
+    from e3nn_amd import nn
+
+    with open(os.path.join(ROOT, "tests", "golden", "state_dict_keys.json")) as f:
+        ref = json.load(f)
+    silu, sigmoid, tanh = torch.nn.functional.silu, torch.sigmoid, torch.tanh
+    modules = {
+        "module_linear": lambda: o3.Linear("2x0e+2x1o", "3x0e+1x1o", biases=True),
+        "module_linear_l2": lambda: o3.Linear("2x0e+2x1o+2x2e", "3x0e+1x1o+2x2e"),
+        "module_fc": lambda: nn.FullyConnectedNet([4, 8, 2], silu),
+        "module_gate": lambda: nn.Gate("4x0e+2x0o", [silu, tanh], "3x0e", [sigmoid], "2x1o+1x2e"),
+        "module_activation": lambda: nn.Activation("4x0e+2x0o", [silu, tanh]),
+        "module_convolution_l1": lambda: nn.Convolution("4x0e+4x1o", "2x0e", "0e+1o", "4x0e+4x1o", [3, 8], 3.0),
+        "module_convolution_l2": lambda: nn.Convolution("4x0e+4x1o+4x2e", "2x0e", "0e+1o+2e", "4x0e+4x1o+4x2e", [3, 8], 3.0),
+    }
+    assert set(modules) == {k for k in ref if k.startswith("module_")}
+    for name, entry in ref.items():
+        if name in modules:
+            m = modules[name]()
+        else:
+            i1, i2, io, ins, kw = entry["args"]
+            m = o3.FullyConnectedTensorProduct(i1, i2, io, **kw) if ins is None else o3.TensorProduct(i1, i2, io, [tuple(t) for t in ins], **kw)
+        mine = {k: list(v.shape) for k, v in m.state_dict().items()}
+        assert mine == entry["state_dict"], name
+        # a state_dict with the reference's keys loads strictly, and the constants are the Wigner tensors
+        fake = {k: torch.zeros(shape, dtype=m.state_dict()[k].dtype) for k, shape in entry["state_dict"].items()}
+        m.load_state_dict(fake, strict=True)
+    tp = o3.FullyConnectedTensorProduct("2x0e+2x1o+2x2e", "0e+1o+2e", "2x0e+2x1o+2x2e")
+    assert torch.equal(tp._compiled_main_left_right._w3j_1_2_1, o3.wigner_3j(1, 2, 1))
+    with pytest.raises(NotImplementedError):  # the reference's right() has no triangular modes
+        o3.TensorProduct("4x1o", "4x1o", "6x1e", [(0, 0, 0, "uvu<v", True)], compile_right=True)
