@@ -11,6 +11,7 @@ extern const char* const kTplUvwSmall;
 extern const char* const kTplUvwMfma;
 extern const char* const kTplUvwMfmaBf16;
 extern const char* const kTplUvwMfmaDw;
+extern const char* const kTplUvwNode;
 extern const char* const kTplFcMfma;
 extern const char* const kTplFcDw;
 

@@ -54,6 +54,7 @@ struct e3x_plan {
   std::string family, key;
   bool zero_fill = false;  // some output irrep is reached by no instruction
   int n_targets = 0;       // uvw_mfma: grid.y
+  std::vector<int> node_tile_rows;  // uvw_node: rows per workgroup of each target, in grid order
   std::mutex mu;
   std::vector<std::unique_ptr<SubKernel>> subs;
   // uvw_mfma: the weight-gradient kernel is a code object of its own, built on first use
@@ -436,6 +437,83 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   return E3X_OK;
 }
 
+// ---- uvw with a scalar second input (node-wise linear layers) on the matrix cores ------------------
+// A target (one output irrep x 32 channels) keeps the weights of all its paths in LDS: at most kNodeMaxBlocks
+// blocks of 8 x 32 floats (64 KB, two workgroups per CU).
+constexpr int kNodeMaxBlocks = 64;
+
+bool uvw_node_eligible(const e3x_plan& P) {
+  if (P.dtype != E3X_F32 || !uvw_mfma_eligible(P) || env_int("E3X_UVW_NODE", 1) == 0) return false;
+  if (P.in2_dim < 1 || P.in2_dim > 16 || (P.in1_dim | P.out_dim) % 4) return false;
+  for (const auto& r : P.in2) if (r.l != 0) return false;
+  std::vector<int> blocks(P.out.size(), 0);
+  for (const auto& p : P.paths) {
+    const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2], &c = P.out[p.out];
+    if (a.l != c.l || a.l > 3 || a.mul % 32 || c.mul % 32 || (P.off1[p.in1] | P.offo[p.out]) % 4) return false;
+    // the coupling with a scalar is a multiple of the identity
+    const auto& C = e3x::wigner_3j(a.l, 0, c.l);
+    const int d = 2 * a.l + 1;
+    for (int i = 0; i < d; ++i)
+      for (int k = 0; k < d; ++k)
+        if (std::fabs(C[i * d + k] - (i == k ? C[0] : 0.0)) > 1e-12) return false;
+    blocks[p.out] += a.mul / 8 * b.mul;
+  }
+  for (int n : blocks) if (n > kNodeMaxBlocks) return false;
+  return true;
+}
+
+int build_uvw_node_source(e3x_plan& P, std::string* src) {
+  struct T { int out, w0; long long work; };
+  std::vector<T> targets;
+  for (size_t c = 0; c < P.out.size(); ++c) {
+    long long blocks = 0;
+    for (const auto& p : P.paths) if (p.out == (int)c) blocks += P.in1[p.in1].mul / 8 * P.in2[p.in2].mul;
+    if (!blocks) continue;
+    for (int w0 = 0; w0 < P.out[c].mul; w0 += 32) targets.push_back({(int)c, w0, blocks * (2 * P.out[c].l + 1)});
+  }
+  // heaviest first: the grid is walked in this order and the light targets fill its tail
+  std::stable_sort(targets.begin(), targets.end(), [](const T& a, const T& b) { return a.work > b.work; });
+  std::ostringstream s, ps, ts;
+  emit_header(s, P);
+  int n_path = 0, max_blocks = 1, max_d = 1;
+  P.node_tile_rows.clear();
+  for (const T& t : targets) {
+    const int d = 2 * P.out[t.out].l + 1;
+    // rows per wave: 32; 64 for scalars, where one row set would leave a single chain of dependent matrix instructions
+    const int rs = env_int("E3X_NODE_RS", d == 1 ? 2 : 1);
+    if (rs != 1 && rs != 2) return fail(E3X_ERR_INVALID, "E3X_NODE_RS must be 1 or 2");
+    // register sets of the load ring: about twelve 16-byte loads per lane in flight
+    const int nbuf = std::max(2, std::min(8, env_int("E3X_NODE_INFLIGHT", 12) / (d * rs)));
+    max_d = std::max(max_d, d);
+    const int beg = n_path;
+    int blocks = 0;
+    for (const auto& p : P.paths) {
+      if (p.out != t.out) continue;
+      const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2];
+      const double c = e3x::wigner_3j(a.l, 0, a.l)[0] * p.pw;
+      ps << "  {" << P.off1[p.in1] << ", " << a.mul << ", " << P.off2[p.in2] << ", " << b.mul << ", " << p.woff << ", "
+         << blocks << ", " << fstr(c) << "},\n";
+      blocks += a.mul / 8 * b.mul;
+      ++n_path;
+    }
+    max_blocks = std::max(max_blocks, blocks);
+    ts << "  {" << P.offo[t.out] << ", " << d << ", " << t.w0 << ", " << P.out[t.out].mul << ", " << rs << ", " << nbuf << ", "
+       << beg << ", " << n_path << "},\n";
+    P.node_tile_rows.push_back(128 * rs);
+  }
+  // W_p[u, v, w] at wbase + (u * O + v) * W + w; lds_block: first LDS block of the path inside its target
+  s << "struct NPath { int x_off, U, o_off, O; long long wbase; int lds_block; float c; };\n";
+  s << "constexpr int N_NPATH = " << n_path << ";\nconstexpr NPath npaths[N_NPATH] = {\n" << ps.str() << "};\n";
+  s << "struct NTarget { int out_off, d, w0, W, rs, nbuf, path_beg, path_end; };\n";
+  s << "constexpr int N_NTARGET = " << targets.size() << ";\nconstexpr NTarget ntargets[N_NTARGET] = {\n" << ts.str() << "};\n";
+  s << "constexpr int MAX_BLOCKS = " << max_blocks << ";\n";
+  // workgroups per CU the register budget is set for: three when their weights fit (160 KB of LDS per CU)
+  s << "constexpr int MIN_WGS = " << env_int("E3X_NODE_WGS", max_blocks <= 48 && max_d <= 5 ? 3 : 2) << ";\n";
+  s << "}  // namespace cfg\n";
+  *src = s.str() + e3x::kTplCommon + e3x::kTplUvwNode;
+  return E3X_OK;
+}
+
 // Tables of the matrix-core weight-gradient kernel: per path the M operand is the input with the smaller l.
 
 int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
@@ -667,6 +745,7 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
   std::vector<std::vector<int>> parts;
   if (n_uvw || general) {
     P->family = (!general && uvw_mfma_eligible(*P) && !(force_small && force_small[0] == '1')) ? "uvw_mfma" : "uvw_small";
+    if (P->family == "uvw_mfma" && uvw_node_eligible(*P)) P->family = "uvw_node";
     std::vector<int> all(P->paths.size());
     for (size_t i = 0; i < all.size(); ++i) all[i] = (int)i;
     parts.push_back(all);
@@ -682,6 +761,7 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
       rc = build_uvw_mfma_source(*P, &src);
       K->waves_per_block = P->dtype == E3X_BF16 ? 8 : 4;
     }
+    else if (P->family == "uvw_node") rc = build_uvw_node_source(*P, &src);
     else if (P->family == "uvw_small") rc = build_uvw_small_source(*P, *K, &src);
     else rc = build_uvu_source(*P, *K, &src);
     if (rc) return rc;
@@ -773,6 +853,11 @@ extern "C" int e3x_tp_forward_ws(e3x_plan* P, const void* x1, const void* x2, co
         blocks = (blocks + 7) / 8 * 8 * P->n_targets;  // row tiles padded to the 8 XCDs
         grid_y = 1;
       }
+    } else if (P->family == "uvw_node") {
+      if (((uintptr_t)x1 | (uintptr_t)w | (uintptr_t)out) & 15)
+        return fail(E3X_ERR_INVALID, "e3x_tp_forward: x1, the weights and out must be 16-byte aligned");
+      blocks = 0;
+      for (int rows : P->node_tile_rows) blocks += (Z + rows - 1) / rows;
     } else {
       const int groups = 64 / K->lanes;
       const long long items = (Z + groups - 1) / groups * K->chunks;
@@ -894,7 +979,7 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
 
 extern "C" int e3x_tp_plan_prepare_backward_w(e3x_plan* P) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: null plan");
-  if (P->family == "uvw_mfma") {
+  if (P->family == "uvw_mfma" || P->family == "uvw_node") {
     if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: fp32 storage only");
     return prepare_mfma_dw(P);
   }
@@ -905,7 +990,7 @@ extern "C" int e3x_tp_plan_prepare_backward_w(e3x_plan* P) {
 extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2, const void* grad_out, void* grad_w,
                                      int64_t Z, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null plan");
-  if (P->family != "uvw_small" && P->family != "uvw_mfma")
+  if (P->family != "uvw_small" && P->family != "uvw_mfma" && P->family != "uvw_node")
     return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: the plan must be all-uvw");
   if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: fp32 storage only");
   if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: negative batch");
@@ -914,7 +999,7 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   hipStream_t st = (hipStream_t)stream;
   int dev, rc;
   if ((rc = current_device(&dev))) return rc;
-  const bool mfma = P->family == "uvw_mfma";
+  const bool mfma = P->family == "uvw_mfma" || P->family == "uvw_node";  // both take the matrix-core gradient kernel
   if (Z == 0) return P->shared_weights ? e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st) : E3X_OK;
   if (!grad_out || (P->in1_dim && !x1) || (P->in2_dim && !x2)) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null pointer");
   long long n_rows = Z;

@@ -99,6 +99,9 @@ class _Plan:
             # scratch for the weights repacked for the matrix cores; the kernel reads rows with 16-byte loads
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x1.device)
             x1, x2 = (t if t.data_ptr() % 16 == 0 else t.clone() for t in (x1, x2))
+        if self.family == "uvw_node":
+            # rows and weights are read with 16-byte loads
+            x1, w = (t if t.data_ptr() % 16 == 0 else t.clone() for t in (x1, w))
         with torch.cuda.device(x1.device):
             _lib.check(
                 _lib.lib().e3x_tp_forward_ws(

@@ -84,6 +84,18 @@ def node_fctp():
     return o3.FullyConnectedTensorProduct("128x0e+64x1o+32x2e", "4x0e", "128x0e+64x1o+96x2e")
 
 
+def node_wide_out():
+    # scalar second input with several 32-channel output tiles per irrep, l = 3 and a pseudoscalar attribute: the
+    # shape of an input gradient of a node-wise layer (few channels in, many out)
+    return o3.FullyConnectedTensorProduct("32x0e+32x1o+32x3o", "3x0e+2x0o", "96x0e+64x1o+64x1e+32x3o+32x3e")
+
+
+def outer_split():
+    # 32-channel output tiles with several outer indices and a second input that is not scalar: the matrix-core
+    # kernel gives its second wave column every other outer index
+    return o3.FullyConnectedTensorProduct("64x0e+32x1o", "4x0e+2x1o", "32x1o+32x1e+32x2e")
+
+
 def wide_k():
     # GEMM K extents above 128 (256 and 160): the K operand is resident in LDS in blocks of 128, restaged per outer index
     return o3.FullyConnectedTensorProduct("256x0e+160x1o", "32x0e+32x1o", "64x0e+64x1o")
@@ -127,6 +139,8 @@ def all_tensor_products():
         ("node_fctp", node_fctp(), (torch.float32,)),
         ("radial_layer", radial_layer(), (torch.float32,)),
         ("wide_k", wide_k(), (torch.float32,)),
+        ("outer_split", outer_split(), (torch.float32,)),
+        ("node_wide_out", node_wide_out(), (torch.float32,)),
         ("mixed_modes", mixed_modes(), (torch.float32,)),
         ("scalar_exact", scalar_exact(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),
@@ -136,7 +150,7 @@ def all_tensor_products():
 
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
-                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "radial_layer", "odd_mul",
+                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "node_wide_out", "radial_layer", "odd_mul",
                   "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
 
 

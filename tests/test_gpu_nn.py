@@ -33,7 +33,7 @@ def test_linear_against_reference_fixture(name):
 
 def test_linear_on_the_matrix_cores():
     lin = dict(ks.nn_modules())["linear_wide"].to(DEV)
-    assert lin._tp._plan(torch.float32).family == "uvw_mfma"
+    assert lin._tp._plan(torch.float32).family == "uvw_node"
     x = seeded(300, lin.irreps_in.dim, seed=5)
     ref = onn.linear_forward(str(lin.irreps_in), str(lin.irreps_out), x.numpy(), lin.weight.detach().cpu().numpy())
     xd = x.to(DEV).requires_grad_(True)
@@ -176,7 +176,7 @@ def test_fully_connected_net():
     assert_close(fc(_t(arr["fc/x"])), arr["fc/out"], what="fc fixture")
     # radial-network shape: 8 -> 64 -> 352, the second layer on the matrix cores
     fc = dict(ks.nn_modules())["fc_radial"].to(DEV)
-    assert fc.layer1._tp._plan(torch.float32).family == "uvw_mfma"
+    assert fc.layer1._tp._plan(torch.float32).family == "uvw_node"
     x = seeded(1000, 8, seed=8)
     ws = [fc.layer0.weight.detach().cpu().numpy(), fc.layer1.weight.detach().cpu().numpy()]
     xd = x.to(DEV).requires_grad_(True)

@@ -165,10 +165,17 @@ def _fan_in_weights(tp, seed=0):
     return w
 
 
-@pytest.mark.parametrize("maker,Z", [(ks.mfma_small, 150), (ks.cfg5, 70), (ks.node_fctp, 333), (ks.radial_layer, 1000), (ks.wide_k, 130)])
-def test_uvw_matrix_core_kernel_against_oracle(maker, Z):
+@pytest.mark.parametrize(
+    "maker,Z,family",
+    [(ks.mfma_small, 150, "uvw_mfma"), (ks.cfg5, 70, "uvw_mfma"), (ks.wide_k, 130, "uvw_mfma"), (ks.outer_split, 200, "uvw_mfma"),
+     # scalar second input: the node-wise kernel; batches that end inside a wave's 64 rows, inside a workgroup's 256
+     # rows, and below one wave
+     (ks.node_fctp, 333, "uvw_node"), (ks.node_fctp, 17, "uvw_node"), (ks.node_fctp, 1280, "uvw_node"),
+     (ks.radial_layer, 1000, "uvw_node"), (ks.node_wide_out, 77, "uvw_node")],
+)  # fmt: skip
+def test_uvw_matrix_core_kernel_against_oracle(maker, Z, family):
     tp = maker().to(DEV)
-    assert tp._plan(torch.float32).family == "uvw_mfma"
+    assert tp._plan(torch.float32).family == family
     w = _fan_in_weights(tp)
     with torch.no_grad():
         tp.weight.copy_(w)
