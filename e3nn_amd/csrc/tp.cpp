@@ -443,13 +443,15 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
 constexpr int kNodeMaxBlocks = 64;
 
 bool uvw_node_eligible(const e3x_plan& P) {
-  if (P.dtype != E3X_F32 || !uvw_mfma_eligible(P) || env_int("E3X_UVW_NODE", 1) == 0) return false;
-  if (P.in2_dim < 1 || P.in2_dim > 16 || (P.in1_dim | P.out_dim) % 4) return false;
+  if (P.dtype != E3X_F32 || !P.shared_weights || P.paths.empty() || env_int("E3X_UVW_NODE", 1) == 0) return false;
+  if (P.in2_dim < 1 || P.in2_dim > 16 || P.in1_dim % 4) return false;
   for (const auto& r : P.in2) if (r.l != 0) return false;
   std::vector<int> blocks(P.out.size(), 0);
+  long long pairs = 0;
   for (const auto& p : P.paths) {
     const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2], &c = P.out[p.out];
-    if (a.l != c.l || a.l > 3 || a.mul % 32 || c.mul % 32 || (P.off1[p.in1] | P.offo[p.out]) % 4) return false;
+    // rows are read in 16-byte pieces of 4 multiplicity indices, 8 indices per matrix-core block
+    if (p.mode != E3X_MODE_UVW || a.l != c.l || a.l > 3 || a.mul % 8 || P.off1[p.in1] % 4) return false;
     // the coupling with a scalar is a multiple of the identity
     const auto& C = e3x::wigner_3j(a.l, 0, c.l);
     const int d = 2 * a.l + 1;
@@ -457,9 +459,12 @@ bool uvw_node_eligible(const e3x_plan& P) {
       for (int k = 0; k < d; ++k)
         if (std::fabs(C[i * d + k] - (i == k ? C[0] : 0.0)) > 1e-12) return false;
     blocks[p.out] += a.mul / 8 * b.mul;
+    pairs += (long long)a.mul * b.mul;
   }
   for (int n : blocks) if (n > kNodeMaxBlocks) return false;
-  return true;
+  // a handful of (u, v) pairs in shapes the other matrix-core kernel does not take: the vector-ALU kernel keeps the
+  // weights in registers and needs no padding to 32 channels
+  return pairs > 64 || uvw_mfma_eligible(P);
 }
 
 int build_uvw_node_source(e3x_plan& P, std::string* src) {
@@ -506,6 +511,9 @@ int build_uvw_node_source(e3x_plan& P, std::string* src) {
   s << "constexpr int N_NPATH = " << n_path << ";\nconstexpr NPath npaths[N_NPATH] = {\n" << ps.str() << "};\n";
   s << "struct NTarget { int out_off, d, w0, W, rs, nbuf, path_beg, path_end; };\n";
   s << "constexpr int N_NTARGET = " << targets.size() << ";\nconstexpr NTarget ntargets[N_NTARGET] = {\n" << ts.str() << "};\n";
+  bool w_aligned = true;  // weight rows of every path are whole 16-byte pieces
+  for (const auto& p : P.paths) w_aligned = w_aligned && P.out[p.out].mul % 4 == 0 && p.woff % 4 == 0;
+  s << "constexpr bool W_ALIGNED = " << (w_aligned ? "true" : "false") << ";\n";
   s << "constexpr int MAX_BLOCKS = " << max_blocks << ";\n";
   // workgroups per CU the register budget is set for: three when their weights fit (160 KB of LDS per CU)
   s << "constexpr int MIN_WGS = " << env_int("E3X_NODE_WGS", max_blocks <= 48 && max_d <= 5 ? 3 : 2) << ";\n";
@@ -596,6 +604,36 @@ int load_dw_function(e3x_plan* P, int dev) {
   if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + K->hsaco + ") failed: " + hipGetErrorString(err));
   if (hipModuleGetFunction(&K->fn_dw[dev], mod, "e3x_uvw_mfma_dw") != hipSuccess)
     return fail(E3X_ERR_HIP, "kernel e3x_uvw_mfma_dw missing from " + K->hsaco);
+  K->module[dev] = mod;
+  return E3X_OK;
+}
+
+// A uvw_node plan that the matrix-core gradient kernel does not take (multiplicities that are not multiples of 32)
+// gets its weight gradient from the vector-ALU family: that code object is built on first use.
+bool node_dw_on_valu(const e3x_plan* P) { return P->family == "uvw_node" && !uvw_mfma_eligible(*P); }
+
+int prepare_valu_dw(e3x_plan* P) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  if (P->dw) return E3X_OK;
+  std::unique_ptr<SubKernel> K(new SubKernel);
+  for (size_t i = 0; i < P->paths.size(); ++i) K->path_ids.push_back((int)i);
+  std::string src;
+  int rc;
+  if ((rc = build_uvw_small_source(*P, *K, &src))) return rc;
+  if ((rc = e3x::get_code_object("uvw_small", src, &K->key, &K->hsaco))) return rc;
+  P->dw = std::move(K);
+  return E3X_OK;
+}
+
+int load_valu_dw_function(e3x_plan* P, int dev) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  SubKernel* K = P->dw.get();
+  if (K->module[dev]) return E3X_OK;
+  hipModule_t mod = nullptr;
+  hipError_t err = hipModuleLoad(&mod, K->hsaco.c_str());
+  if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + K->hsaco + ") failed: " + hipGetErrorString(err));
+  if (hipModuleGetFunction(&K->fn_dw[dev], mod, "e3x_uvw_small_dw") != hipSuccess)
+    return fail(E3X_ERR_HIP, "kernel e3x_uvw_small_dw missing from " + K->hsaco);
   K->module[dev] = mod;
   return E3X_OK;
 }
@@ -745,7 +783,7 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
   std::vector<std::vector<int>> parts;
   if (n_uvw || general) {
     P->family = (!general && uvw_mfma_eligible(*P) && !(force_small && force_small[0] == '1')) ? "uvw_mfma" : "uvw_small";
-    if (P->family == "uvw_mfma" && uvw_node_eligible(*P)) P->family = "uvw_node";
+    if (!general && uvw_node_eligible(*P) && !(force_small && force_small[0] == '1')) P->family = "uvw_node";
     std::vector<int> all(P->paths.size());
     for (size_t i = 0; i < all.size(); ++i) all[i] = (int)i;
     parts.push_back(all);
@@ -854,8 +892,8 @@ extern "C" int e3x_tp_forward_ws(e3x_plan* P, const void* x1, const void* x2, co
         grid_y = 1;
       }
     } else if (P->family == "uvw_node") {
-      if (((uintptr_t)x1 | (uintptr_t)w | (uintptr_t)out) & 15)
-        return fail(E3X_ERR_INVALID, "e3x_tp_forward: x1, the weights and out must be 16-byte aligned");
+      if (((uintptr_t)x1 | (uintptr_t)w) & 15)
+        return fail(E3X_ERR_INVALID, "e3x_tp_forward: x1 and the weights must be 16-byte aligned");
       blocks = 0;
       for (int rows : P->node_tile_rows) blocks += (Z + rows - 1) / rows;
     } else {
@@ -979,6 +1017,7 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
 
 extern "C" int e3x_tp_plan_prepare_backward_w(e3x_plan* P) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: null plan");
+  if (node_dw_on_valu(P)) return prepare_valu_dw(P);
   if (P->family == "uvw_mfma" || P->family == "uvw_node") {
     if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: fp32 storage only");
     return prepare_mfma_dw(P);
@@ -999,7 +1038,8 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   hipStream_t st = (hipStream_t)stream;
   int dev, rc;
   if ((rc = current_device(&dev))) return rc;
-  const bool mfma = P->family == "uvw_mfma" || P->family == "uvw_node";  // both take the matrix-core gradient kernel
+  // the node-wise family has no gradient kernel of its own: the matrix-core one where its tiling fits, else the vector-ALU one
+  const bool mfma = P->family == "uvw_mfma" || (P->family == "uvw_node" && !node_dw_on_valu(P));
   if (Z == 0) return P->shared_weights ? e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st) : E3X_OK;
   if (!grad_out || (P->in1_dim && !x1) || (P->in2_dim && !x2)) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null pointer");
   long long n_rows = Z;
@@ -1027,7 +1067,15 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
     return E3X_OK;
   }
   if (P->shared_weights && (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st))) return rc;
-  if ((rc = load_functions(P, dev))) return rc;
+  hipFunction_t fn_dw = nullptr;
+  if (node_dw_on_valu(P)) {
+    if ((rc = prepare_valu_dw(P))) return rc;
+    if ((rc = load_valu_dw_function(P, dev))) return rc;
+    fn_dw = P->dw->fn_dw[dev];
+  } else {
+    if ((rc = load_functions(P, dev))) return rc;
+    fn_dw = P->subs[0]->fn_dw[dev];
+  }
   // one thread per (path, v, w) column of the weight blocks
   long long cols = 0;
   for (const auto& q : P->paths) cols += (long long)P->in2[q.in2].mul * P->out[q.out].mul;
@@ -1044,8 +1092,7 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   long long rows_per_slice = (Z + slices - 1) / slices;
   slices = (Z + rows_per_slice - 1) / rows_per_slice;
   void* args[] = {(void*)&x1, (void*)&x2, (void*)&grad_out, (void*)&grad_w, (void*)&n_rows, (void*)&rows_per_slice};
-  hipError_t err = hipModuleLaunchKernel(P->subs[0]->fn_dw[dev], (unsigned)wblocks, (unsigned)slices, 1, 256, 1, 1, 0, st,
-                                         args, nullptr);
+  hipError_t err = hipModuleLaunchKernel(fn_dw, (unsigned)wblocks, (unsigned)slices, 1, 256, 1, 1, 0, st, args, nullptr);
   if (err != hipSuccess)
     return fail(E3X_ERR_HIP, std::string("e3x_tp_backward_w_uvw: launch failed: ") + hipGetErrorString(err));
   return E3X_OK;

@@ -90,6 +90,18 @@ def node_wide_out():
     return o3.FullyConnectedTensorProduct("32x0e+32x1o+32x3o", "3x0e+2x0o", "96x0e+64x1o+64x1e+32x3o+32x3e")
 
 
+def node_narrow():
+    # scalar second input, channel counts that are not multiples of 4 (weight rows read float by float, a partly
+    # filled 32-channel tile) and multiplicities 8 / 24 / 40: the shape of the per-node mixing coefficient of a
+    # convolution (reference e3nn/nn/models/v2106/points_convolution.py:92-97) with two more irreps
+    return o3.FullyConnectedTensorProduct("96x0e+40x1o+8x2e", "4x0e", "1x0e+23x1o+9x2e")
+
+
+def node_partial_tile():
+    # channel counts that are multiples of 4 but not of 32: 16-byte weight pieces inside and outside the last tile
+    return o3.FullyConnectedTensorProduct("64x0e+16x1o", "3x0e", "48x0e+20x1o")
+
+
 def outer_split():
     # 32-channel output tiles with several outer indices and a second input that is not scalar: the matrix-core
     # kernel gives its second wave column every other outer index
@@ -141,6 +153,8 @@ def all_tensor_products():
         ("wide_k", wide_k(), (torch.float32,)),
         ("outer_split", outer_split(), (torch.float32,)),
         ("node_wide_out", node_wide_out(), (torch.float32,)),
+        ("node_narrow", node_narrow(), (torch.float32,)),
+        ("node_partial_tile", node_partial_tile(), (torch.float32,)),
         ("mixed_modes", mixed_modes(), (torch.float32,)),
         ("scalar_exact", scalar_exact(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),
@@ -150,7 +164,7 @@ def all_tensor_products():
 
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
-                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "node_wide_out", "radial_layer", "odd_mul",
+                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
                   "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
 
 

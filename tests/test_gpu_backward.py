@@ -72,7 +72,7 @@ def test_fused_message_gradients(maker, N, E, idx):
 
 
 @pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.mfma_small, 70),
-                                     (lambda: ks.golden_tp("fctp_per_sample_weights"), 5), (ks.node_fctp, 90), (ks.radial_layer, 77), (ks.node_wide_out, 45)])  # fmt: skip
+                                     (lambda: ks.golden_tp("fctp_per_sample_weights"), 5), (ks.node_fctp, 90), (ks.radial_layer, 77), (ks.node_wide_out, 45), (ks.node_narrow, 40)])  # fmt: skip
 def test_uvw_input_gradients(maker, Z):
     tp = maker().to(DEV)
     spec = oracle_spec(tp)
@@ -91,7 +91,8 @@ def test_uvw_input_gradients(maker, Z):
 
 @pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.cfg1, 4099),
                                      (lambda: ks.golden_tp("fctp_per_sample_weights"), 5), (ks.mfma_small, 70),
-                                     (ks.mfma_small, 1500), (ks.node_fctp, 700), (ks.radial_layer, 513), (ks.node_wide_out, 300)])  # fmt: skip
+                                     (ks.mfma_small, 1500), (ks.node_fctp, 700), (ks.radial_layer, 513), (ks.node_wide_out, 300), (ks.node_narrow, 260),
+                                     (ks.node_partial_tile, 100)])  # fmt: skip
 def test_uvw_weight_gradients(maker, Z):
     tp = maker().to(DEV)
     spec = oracle_spec(tp)
