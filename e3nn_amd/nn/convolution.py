@@ -67,9 +67,12 @@ class Convolution(torch.nn.Module):
         if edges is None:
             edges = DstSortedEdges(edge_src, edge_dst, node_input.shape[0])
         node_features = self.tp.forward_gather_scatter(node_features, edge_attr, weight, edges=edges)
-        node_features = node_features.div(self.num_neighbors**0.5)
+        # lin2 and alpha are linear in the features, so the division by sqrt(num_neighbors) that the reference applies
+        # to the summed messages (points_convolution.py:108) is applied to their outputs instead, which are four to a
+        # thousand times narrower than the messages
+        inv = 1.0 / self.num_neighbors**0.5
         node_conv_out = self.lin2(node_features, node_attr)
         alpha = self.alpha(node_features, node_attr)
         m = self.sc.output_mask
-        alpha = (1 - m) + alpha * m
-        return node_self_connection + alpha * node_conv_out
+        alpha = (1 - m) + alpha * (m * inv)
+        return torch.addcmul(node_self_connection, alpha, node_conv_out, value=inv)
