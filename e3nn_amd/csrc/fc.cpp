@@ -29,6 +29,7 @@ constexpr int kMaxLiveRegs = 192;
 struct e3x_fc_plan {
   std::vector<int> hs, hp;
   int n_layers = 0, rows_per_wg = 0, waves = 8;
+  bool epilogue = false;  // outputs are multiplied by an activation derivative of a caller-supplied tensor
   int64_t packed_numel = 0;
   std::string key, hsaco;
   std::mutex mu;
@@ -76,7 +77,16 @@ int load_functions(e3x_fc_plan* P, int dev) {
 
 extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act,
                                   double variance_in, double variance_out, int32_t dtype, e3x_fc_plan** out) {
+  return e3x_fc_plan_create_epilogue(hs, n_hs, act, act_cst, out_act, variance_in, variance_out, dtype, E3X_ACT_IDENTITY,
+                                     1.0, out);
+}
+
+extern "C" int e3x_fc_plan_create_epilogue(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act,
+                                           double variance_in, double variance_out, int32_t dtype, int32_t epilogue_act,
+                                           double epilogue_cst, e3x_fc_plan** out) {
   if (!hs || !out) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: null argument");
+  if (epilogue_act < E3X_ACT_IDENTITY || epilogue_act > E3X_ACT_RELU)
+    return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: unknown epilogue activation");
   if (dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: only fp32 storage is implemented");
   if (n_hs < 2 || n_hs - 1 > kMaxLayers) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: 1 to 8 layers");
   if (act < E3X_ACT_IDENTITY || act > E3X_ACT_RELU) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: unknown activation");
@@ -143,6 +153,8 @@ extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, 
   s << "};\nconstexpr float WSCALE[NL] = {";
   for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << fstr(wscale[l]);
   s << "};\nconstexpr float OUT_POST = " << fstr(out_post) << ";\n";
+  s << "constexpr int EPI_ACT = " << epilogue_act << ";\nconstexpr float EPI_CST = " << fstr(epilogue_cst) << ";\n";
+  P->epilogue = epilogue_act != E3X_ACT_IDENTITY;
   s << "constexpr int RS = " << rs << ", WAVES = " << waves << ";\n}  // namespace cfg\n";
   const std::string src = s.str() + e3x::kTplCommon + e3x::kTplFcMfma;
   int rc = e3x::get_code_object("fc_mfma", src, &P->key, &P->hsaco);
@@ -216,7 +228,16 @@ extern "C" const char* e3x_fc_plan_key(const e3x_fc_plan* P) { return P ? P->key
 
 extern "C" int e3x_fc_forward(e3x_fc_plan* P, const void* x, const void* const* weights, void* out, int64_t Z,
                               void* workspace, size_t workspace_bytes, void* stream) {
+  return e3x_fc_forward_epilogue(P, x, weights, nullptr, out, Z, workspace, workspace_bytes, stream);
+}
+
+extern "C" int e3x_fc_forward_epilogue(e3x_fc_plan* P, const void* x, const void* const* weights, const void* z, void* out,
+                                       int64_t Z, void* workspace, size_t workspace_bytes, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_fc_forward: null plan");
+  if (P->epilogue && !z && Z > 0)
+    return fail(E3X_ERR_INVALID, "e3x_fc_forward: this plan multiplies by an activation derivative and needs z "
+                                 "(e3x_fc_forward_epilogue)");
+  if (!P->epilogue) z = nullptr;
   if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_fc_forward: negative batch");
   if (Z == 0) return E3X_OK;
   if (!x || !out || !weights || !workspace) return fail(E3X_ERR_INVALID, "e3x_fc_forward: null pointer");
@@ -244,7 +265,7 @@ extern "C" int e3x_fc_forward(e3x_fc_plan* P, const void* x, const void* const* 
   long long n_rows = Z;
   long long tiles = (Z + P->rows_per_wg - 1) / P->rows_per_wg;
   long long blocks = tiles < P->n_cu[dev] ? tiles : P->n_cu[dev];  // one persistent workgroup per compute unit
-  void* args[] = {&x, &workspace, &out, &n_rows};
+  void* args[] = {&x, &workspace, &out, &n_rows, &z};
   hipError_t err = hipModuleLaunchKernel(P->fn_fwd[dev], (unsigned)blocks, 1, 1, 64 * P->waves, 1, 1, 0, st, args, nullptr);
   if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_fc_forward: launch failed: ") + hipGetErrorString(err));
   return E3X_OK;

@@ -50,6 +50,36 @@ class _DenseFn(torch.autograd.Function):
         return gx, gw, None
 
 
+class _ActDenseFn(torch.autograd.Function):
+    """``dense(act(z))`` of two consecutive layers: the forward pass is the activation kernel followed by the dense
+    kernel; the backward pass takes the input gradient through the activation inside the dense kernel's epilogue,
+    ``(g @ W^T * s) * cst * act'(z)``, so the gradient of the hidden activations is never written."""
+
+    @staticmethod
+    def forward(ctx, z, w, layer, prev):
+        with torch.no_grad():
+            h = prev.act(z)
+        ctx.layer = layer
+        ctx.plan = layer.act_dense_plan(prev)
+        ctx.save_for_backward(z, h, w)
+        return layer._fwd.forward(h, [w.contiguous()])
+
+    @staticmethod
+    def backward(ctx, g):
+        z, h, w = ctx.saved_tensors
+        layer = ctx.layer
+        g = g.contiguous()
+        if g.data_ptr() % 16:
+            g = g.clone()
+        gz = gw = None
+        if ctx.needs_input_grad[0]:
+            wt = (w.t() * (layer._scale * layer.h_out**0.5)).contiguous()
+            gz = ctx.plan.forward(g, [wt], z)
+        if ctx.needs_input_grad[1]:
+            gw = layer._fwd.backward_w(h, g)
+        return gz, gw, None, None
+
+
 class _Layer(torch.nn.Module):
     def __init__(self, h_in, h_out, act, var_in, var_out) -> None:
         super().__init__()
@@ -65,6 +95,17 @@ class _Layer(torch.nn.Module):
         # _fc.py:41-48: x @ W / sqrt(h_in var_in) before an activation, x @ W / sqrt(h_in var_in / var_out) without
         self._scale = (h_in * var_in) ** -0.5 if act is not None else (h_in * var_in / var_out) ** -0.5
         self._fwd = self._bwd = None
+        self._bwd_act = {}
+
+    def act_dense_plan(self, prev):
+        """Plan of ``g @ W^T`` of this layer times the derivative of the activation of ``prev`` (the layer in front);
+        None when one of the kernels involved is outside its limits."""
+        name = prev._act_name
+        if name not in self._bwd_act:
+            ok = self.dense_plans()[0] and self._fwd.has_backward_w and prev.var_out == 1
+            plan = _FusedPlan([self.h_out, self.h_in], "identity", False, 1, 1, epilogue=name) if ok else None
+            self._bwd_act[name] = plan if plan is not None and plan.handle is not None else None
+        return self._bwd_act[name]
 
     def __repr__(self) -> str:
         return f"Layer({self.h_in}->{self.h_out}, act={self._act_name})"
@@ -112,17 +153,20 @@ class _Layer(torch.nn.Module):
 class _FusedPlan:
     """Handle of a fused-network plan of the library; ``None`` handle when the network is outside its limits."""
 
-    def __init__(self, hs, act_name, out_act, variance_in, variance_out) -> None:
+    def __init__(self, hs, act_name, out_act, variance_in, variance_out, epilogue=None) -> None:
+        """``epilogue``: name of an activation; the outputs are then multiplied by ``cst * act'(z)`` of a tensor ``z``
+        given to ``forward`` (the input gradient of a layer taken through the activation in front of it)."""
         self.handle = None
         self.key = None
         self.reason = None
-        self._args = (list(hs), act_name, out_act, variance_in, variance_out)
+        self._args = (list(hs), act_name, out_act, variance_in, variance_out, epilogue)
         L = _lib.lib()
         arr = (ctypes.c_int32 * len(hs))(*hs)
         h = ctypes.c_void_p()
-        rc = L.e3x_fc_plan_create(
+        rc = L.e3x_fc_plan_create_epilogue(
             arr, len(hs), _KINDS[act_name], second_moment_constant(act_name), int(bool(out_act)), float(variance_in),
-            float(variance_out), 0, ctypes.byref(h),
+            float(variance_out), 0, _KINDS[epilogue or "identity"], second_moment_constant(epilogue) if epilogue else 1.0,
+            ctypes.byref(h),
         )  # fmt: skip
         if rc == _lib.ERR_INVALID:
             self.reason = L.e3x_last_error().decode()  # outside the fused kernel's limits: layer by layer instead
@@ -160,16 +204,17 @@ class _FusedPlan:
             )
         return gw
 
-    def forward(self, x, weights):
+    def forward(self, x, weights, z=None):
         L = _lib.lib()
         Z = x.shape[0]
         out = torch.empty((Z, weights[-1].shape[1]), device=x.device, dtype=torch.float32)
         ws = torch.empty(self.workspace_bytes, device=x.device, dtype=torch.uint8)
         ptrs = (ctypes.c_void_p * len(weights))(*[w.data_ptr() for w in weights])
+        assert z is None or (z.shape == out.shape and z.is_contiguous() and z.dtype == torch.float32)
         with torch.cuda.device(x.device):
             _lib.check(
-                L.e3x_fc_forward(self.handle, _lib.ptr(x), ptrs, _lib.ptr(out), Z, _lib.ptr(ws), self.workspace_bytes,
-                                 _lib.stream_ptr(x.device))
+                L.e3x_fc_forward_epilogue(self.handle, _lib.ptr(x), ptrs, _lib.ptr(z) if z is not None else None, _lib.ptr(out),
+                                          Z, _lib.ptr(ws), self.workspace_bytes, _lib.stream_ptr(x.device))
             )  # fmt: skip
         return out
 
@@ -215,6 +260,32 @@ class FullyConnectedNet(torch.nn.Sequential):
                 ws = [l.weight.detach().contiguous() for l in layers]
                 if all(w.is_cuda and w.dtype == torch.float32 for w in ws):
                     return plan.forward(x2, ws).reshape(lead + (self.hs[-1],))
+        if wants_grad and len(layers) > 1 and x.is_cuda and x.dtype == torch.float32 and x.shape[-1] == self.hs[0]:
+            out = self._forward_chained(x, layers)
+            if out is not None:
+                return out
         for layer in layers:
             x = layer(x)
         return x
+
+    def _forward_chained(self, x, layers):
+        """Layer by layer with every hidden activation attached to the dense layer behind it (``_ActDenseFn``); None
+        when a layer is outside the limits of the kernels involved."""
+        for prev, layer in zip(layers, layers[1:]):
+            if prev.act is None or prev.weight.dtype != torch.float32 or layer.act_dense_plan(prev) is None:
+                return None
+        if not layers[0].dense_plans()[0] or layers[-1].weight.dtype != torch.float32:
+            return None
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.hs[0]).contiguous()
+        if x2.data_ptr() % 16:
+            x2 = x2.clone()
+        z = _DenseFn.apply(x2, layers[0].weight, layers[0])
+        for prev, layer in zip(layers, layers[1:]):
+            z = _ActDenseFn.apply(z, layer.weight, layer, prev)
+        last = layers[-1]
+        if last.act is not None:
+            z = last.act(z)
+            if last.var_out != 1:
+                z = z * last.var_out**0.5
+        return z.reshape(lead + (self.hs[-1],))

@@ -127,6 +127,15 @@ def test_fully_connected_net_gradients(case):
     xd = x.to(DEV).requires_grad_(True)
     out = net(xd)
     assert_close(out, f(x.numpy(), ws), what="layer-by-layer forward")
+    if n_layers > 1 and act is not None:
+        # hidden activations are differentiated inside the epilogue of the next layer's input-gradient kernel
+        seen, todo = set(), [out.grad_fn]
+        while todo:
+            fn = todo.pop()
+            if fn is not None and fn not in seen:
+                seen.add(fn)
+                todo += [g for g, _ in fn.next_functions]
+        assert sum("_ActDenseFn" in type(fn).__name__ for fn in seen) == n_layers - 1
     cot = seeded(Z, hs[-1], seed=60 + case)
     out.backward(cot.to(DEV))
     rng = np.random.default_rng(case)
