@@ -68,8 +68,9 @@ _SIGNATURES = {
                                 c_int32, c_void_p]),
     "e3x_fc_plan_create": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, ctypes.c_double, c_int32, ctypes.c_double,
                                    ctypes.c_double, c_int32, ctypes.POINTER(c_void_p)]),
-    "e3x_fc_plan_create_epilogue": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, ctypes.c_double, c_int32, ctypes.c_double,
-                                            ctypes.c_double, c_int32, c_int32, ctypes.c_double, ctypes.POINTER(c_void_p)]),
+    "e3x_fc_plan_create_fused": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, ctypes.c_double, c_int32, ctypes.c_double,
+                                         ctypes.c_double, c_int32, c_int32, ctypes.c_double, c_int32, ctypes.c_double,
+                                         ctypes.POINTER(c_void_p)]),
     "e3x_fc_forward_epilogue": (c_int, [c_void_p, c_void_p, ctypes.POINTER(c_void_p), c_void_p, c_void_p, c_int64, c_void_p,
                                         c_size_t, c_void_p]),
     "e3x_fc_plan_destroy": (c_int, [c_void_p]),

@@ -30,6 +30,8 @@ struct e3x_fc_plan {
   std::vector<int> hs, hp;
   int n_layers = 0, rows_per_wg = 0, waves = 8;
   bool epilogue = false;  // outputs are multiplied by an activation derivative of a caller-supplied tensor
+  int input_act = 0;      // the rows given are pre-activations: the network starts from input_cst * act(x)
+  double input_cst = 1.0;
   int64_t packed_numel = 0;
   std::string key, hsaco;
   std::mutex mu;
@@ -77,16 +79,16 @@ int load_functions(e3x_fc_plan* P, int dev) {
 
 extern "C" int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act,
                                   double variance_in, double variance_out, int32_t dtype, e3x_fc_plan** out) {
-  return e3x_fc_plan_create_epilogue(hs, n_hs, act, act_cst, out_act, variance_in, variance_out, dtype, E3X_ACT_IDENTITY,
-                                     1.0, out);
+  return e3x_fc_plan_create_fused(hs, n_hs, act, act_cst, out_act, variance_in, variance_out, dtype, E3X_ACT_IDENTITY, 1.0,
+                                  E3X_ACT_IDENTITY, 1.0, out);
 }
 
-extern "C" int e3x_fc_plan_create_epilogue(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act,
-                                           double variance_in, double variance_out, int32_t dtype, int32_t epilogue_act,
-                                           double epilogue_cst, e3x_fc_plan** out) {
+extern "C" int e3x_fc_plan_create_fused(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act,
+                                        double variance_in, double variance_out, int32_t dtype, int32_t input_act,
+                                        double input_cst, int32_t epilogue_act, double epilogue_cst, e3x_fc_plan** out) {
   if (!hs || !out) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: null argument");
-  if (epilogue_act < E3X_ACT_IDENTITY || epilogue_act > E3X_ACT_RELU)
-    return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: unknown epilogue activation");
+  if (epilogue_act < E3X_ACT_IDENTITY || epilogue_act > E3X_ACT_RELU || input_act < E3X_ACT_IDENTITY || input_act > E3X_ACT_RELU)
+    return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: unknown input or epilogue activation");
   if (dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: only fp32 storage is implemented");
   if (n_hs < 2 || n_hs - 1 > kMaxLayers) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: 1 to 8 layers");
   if (act < E3X_ACT_IDENTITY || act > E3X_ACT_RELU) return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: unknown activation");
@@ -154,7 +156,10 @@ extern "C" int e3x_fc_plan_create_epilogue(const int32_t* hs, int32_t n_hs, int3
   for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << fstr(wscale[l]);
   s << "};\nconstexpr float OUT_POST = " << fstr(out_post) << ";\n";
   s << "constexpr int EPI_ACT = " << epilogue_act << ";\nconstexpr float EPI_CST = " << fstr(epilogue_cst) << ";\n";
+  s << "constexpr int IN_ACT = " << input_act << ";\nconstexpr float IN_CST = " << fstr(input_cst) << ";\n";
   P->epilogue = epilogue_act != E3X_ACT_IDENTITY;
+  P->input_act = input_act;
+  P->input_cst = input_cst;
   s << "constexpr int RS = " << rs << ", WAVES = " << waves << ";\n}  // namespace cfg\n";
   const std::string src = s.str() + e3x::kTplCommon + e3x::kTplFcMfma;
   int rc = e3x::get_code_object("fc_mfma", src, &P->key, &P->hsaco);
@@ -183,7 +188,8 @@ extern "C" int e3x_fc_plan_prepare_backward_w(e3x_fc_plan* P) {
   if (const char* v = std::getenv("E3X_FCDW_OCC")) s << "#define E3X_FCDW_OCC " << std::atoi(v) << "\n";
   s << "namespace cfg {\n";
   s << "constexpr int H_IN = " << P->hs[0] << ", H_OUT = " << P->hs[1] << ", NTW = " << ntw << ";\n";
-  s << "constexpr float SCALE = " << fstr(P->scale0) << ";\n}  // namespace cfg\n";
+  s << "constexpr float SCALE = " << fstr(P->scale0) << ";\n";
+  s << "constexpr int IN_ACT = " << P->input_act << ";\nconstexpr float IN_CST = " << fstr(P->input_cst) << ";\n}  // namespace cfg\n";
   const std::string src = s.str() + e3x::kTplCommon + e3x::kTplFcDw;
   return e3x::get_code_object("fc_dw", src, &P->dw_key, &P->dw_hsaco);
 }

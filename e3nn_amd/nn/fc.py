@@ -51,32 +51,29 @@ class _DenseFn(torch.autograd.Function):
 
 
 class _ActDenseFn(torch.autograd.Function):
-    """``dense(act(z))`` of two consecutive layers: the forward pass is the activation kernel followed by the dense
-    kernel; the backward pass takes the input gradient through the activation inside the dense kernel's epilogue,
-    ``(g @ W^T * s) * cst * act'(z)``, so the gradient of the hidden activations is never written."""
+    """``dense(act(z))`` of two consecutive layers without the activated tensor: the dense kernel applies the
+    activation to its input rows as it loads them (forward and weight gradient), and the backward pass takes the input
+    gradient through the activation in the epilogue of the input-gradient kernel, ``(g @ W^T * s) * cst * act'(z)``."""
 
     @staticmethod
     def forward(ctx, z, w, layer, prev):
-        with torch.no_grad():
-            h = prev.act(z)
-        ctx.layer = layer
-        ctx.plan = layer.act_dense_plan(prev)
-        ctx.save_for_backward(z, h, w)
-        return layer._fwd.forward(h, [w.contiguous()])
+        ctx.plans = layer.act_dense_plans(prev)
+        ctx.scale = layer._scale * layer.h_out**0.5
+        ctx.save_for_backward(z, w)
+        return ctx.plans[0].forward(z, [w.contiguous()])
 
     @staticmethod
     def backward(ctx, g):
-        z, h, w = ctx.saved_tensors
-        layer = ctx.layer
+        z, w = ctx.saved_tensors
+        fwd, bwd = ctx.plans
         g = g.contiguous()
         if g.data_ptr() % 16:
             g = g.clone()
         gz = gw = None
         if ctx.needs_input_grad[0]:
-            wt = (w.t() * (layer._scale * layer.h_out**0.5)).contiguous()
-            gz = ctx.plan.forward(g, [wt], z)
+            gz = bwd.forward(g, [(w.t() * ctx.scale).contiguous()], z)
         if ctx.needs_input_grad[1]:
-            gw = layer._fwd.backward_w(h, g)
+            gw = fwd.backward_w(z, g)
         return gz, gw, None, None
 
 
@@ -97,14 +94,21 @@ class _Layer(torch.nn.Module):
         self._fwd = self._bwd = None
         self._bwd_act = {}
 
-    def act_dense_plan(self, prev):
-        """Plan of ``g @ W^T`` of this layer times the derivative of the activation of ``prev`` (the layer in front);
-        None when one of the kernels involved is outside its limits."""
+    def act_dense_plans(self, prev):
+        """Plans of this layer fused with the activation of ``prev`` (the layer in front): ``act(z) @ W`` with its weight
+        gradient, and ``g @ W^T`` times the derivative of the activation; None when a kernel involved is outside its
+        limits."""
         name = prev._act_name
         if name not in self._bwd_act:
-            ok = self.dense_plans()[0] and self._fwd.has_backward_w and prev.var_out == 1
-            plan = _FusedPlan([self.h_out, self.h_in], "identity", False, 1, 1, epilogue=name) if ok else None
-            self._bwd_act[name] = plan if plan is not None and plan.handle is not None else None
+            pair = None
+            if self.dense_plans()[0] and self._fwd.has_backward_w and prev.var_out == 1:
+                var_ratio = self.var_in if self.act is not None else self.var_in / self.var_out
+                fwd = _FusedPlan([self.h_in, self.h_out], "identity", False, var_ratio, 1, input_act=name)
+                bwd = _FusedPlan([self.h_out, self.h_in], "identity", False, 1, 1, epilogue=name)
+                if fwd.handle is not None and bwd.handle is not None:
+                    fwd.prepare_backward_w()
+                    pair = (fwd, bwd) if fwd.has_backward_w else None
+            self._bwd_act[name] = pair
         return self._bwd_act[name]
 
     def __repr__(self) -> str:
@@ -153,20 +157,21 @@ class _Layer(torch.nn.Module):
 class _FusedPlan:
     """Handle of a fused-network plan of the library; ``None`` handle when the network is outside its limits."""
 
-    def __init__(self, hs, act_name, out_act, variance_in, variance_out, epilogue=None) -> None:
+    def __init__(self, hs, act_name, out_act, variance_in, variance_out, epilogue=None, input_act=None) -> None:
         """``epilogue``: name of an activation; the outputs are then multiplied by ``cst * act'(z)`` of a tensor ``z``
-        given to ``forward`` (the input gradient of a layer taken through the activation in front of it)."""
+        given to ``forward`` (the input gradient of a layer taken through the activation in front of it).
+        ``input_act``: the rows given are pre-activations, the network starts from ``cst * act(x)``."""
         self.handle = None
         self.key = None
         self.reason = None
-        self._args = (list(hs), act_name, out_act, variance_in, variance_out, epilogue)
+        self._args = (list(hs), act_name, out_act, variance_in, variance_out, epilogue, input_act)
         L = _lib.lib()
         arr = (ctypes.c_int32 * len(hs))(*hs)
         h = ctypes.c_void_p()
-        rc = L.e3x_fc_plan_create_epilogue(
+        rc = L.e3x_fc_plan_create_fused(
             arr, len(hs), _KINDS[act_name], second_moment_constant(act_name), int(bool(out_act)), float(variance_in),
-            float(variance_out), 0, _KINDS[epilogue or "identity"], second_moment_constant(epilogue) if epilogue else 1.0,
-            ctypes.byref(h),
+            float(variance_out), 0, _KINDS[input_act or "identity"], second_moment_constant(input_act) if input_act else 1.0,
+            _KINDS[epilogue or "identity"], second_moment_constant(epilogue) if epilogue else 1.0, ctypes.byref(h),
         )  # fmt: skip
         if rc == _lib.ERR_INVALID:
             self.reason = L.e3x_last_error().decode()  # outside the fused kernel's limits: layer by layer instead
@@ -272,7 +277,7 @@ class FullyConnectedNet(torch.nn.Sequential):
         """Layer by layer with every hidden activation attached to the dense layer behind it (``_ActDenseFn``); None
         when a layer is outside the limits of the kernels involved."""
         for prev, layer in zip(layers, layers[1:]):
-            if prev.act is None or prev.weight.dtype != torch.float32 or layer.act_dense_plan(prev) is None:
+            if prev.act is None or prev.weight.dtype != torch.float32 or layer.act_dense_plans(prev) is None:
                 return None
         if not layers[0].dense_plans()[0] or layers[-1].weight.dtype != torch.float32:
             return None

@@ -239,13 +239,16 @@ int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_
 typedef struct e3x_fc_plan e3x_fc_plan;
 int e3x_fc_plan_create(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act, double variance_in,
                        double variance_out, int32_t dtype, e3x_fc_plan** out);
-/* The same network whose outputs are multiplied by epilogue_cst * act'(z), z[Z, hs[n_hs-1]] given at launch: with
- * hs = {h_out, h_in}, no activation and the transposed weights this is the input gradient of a dense layer taken
- * through the normalised activation in front of it (autograd of e3nn/nn/_fc.py:38-48 over two layers) in one kernel.
- * e3x_fc_forward on such a plan is an error; e3x_fc_forward_epilogue on a plan without epilogue ignores z. */
-int e3x_fc_plan_create_epilogue(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act,
-                                double variance_in, double variance_out, int32_t dtype, int32_t epilogue_act,
-                                double epilogue_cst, e3x_fc_plan** out);
+/* The same network with an activation fused at either end, for the layer-by-layer path under autograd (one-layer
+ * plans): input_act != E3X_ACT_IDENTITY: the rows given are pre-activations and the network starts from
+ * input_cst * act(x) -- also in e3x_fc_backward_w -- so the activated tensor is never stored; epilogue_act: the
+ * outputs are multiplied by epilogue_cst * act'(z), z[Z, hs[n_hs-1]] given at launch: with hs = {h_out, h_in} and the
+ * transposed weights this is the input gradient of a dense layer taken through the normalised activation in front of
+ * it (autograd of e3nn/nn/_fc.py:38-48 over two layers) in one kernel.  e3x_fc_forward on a plan with an epilogue
+ * is an error; e3x_fc_forward_epilogue on a plan without one ignores z. */
+int e3x_fc_plan_create_fused(const int32_t* hs, int32_t n_hs, int32_t act, double act_cst, int32_t out_act,
+                             double variance_in, double variance_out, int32_t dtype, int32_t input_act, double input_cst,
+                             int32_t epilogue_act, double epilogue_cst, e3x_fc_plan** out);
 int e3x_fc_forward_epilogue(e3x_fc_plan* plan, const void* x, const void* const* weights, const void* z, void* out,
                             int64_t Z, void* workspace, size_t workspace_bytes, void* stream);
 int e3x_fc_plan_destroy(e3x_fc_plan* plan);

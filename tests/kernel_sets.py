@@ -253,8 +253,8 @@ def prebuild(verbose=True, workers=6):
                 keys += [fwd.key, bwd.key] if fwd else ["(tensor-product kernels)"]
             layers = list(tp)
             for prev, layer in zip(layers, layers[1:]):  # input gradient through the activation in one kernel
-                plan = layer.act_dense_plan(prev) if prev.act is not None else None
-                keys += [plan.key] if plan is not None else []
+                pair = layer.act_dense_plans(prev) if prev.act is not None else None
+                keys += [pair[0].key, pair[1].key] if pair is not None else []
             return name, keys
         keys = [tp._plan(dt).key for dt in dtypes]
         if backward:
