@@ -7,6 +7,7 @@ namespace e3x {
 // Device template sources, embedded at library build time from templates/*.inc.
 extern const char* const kTplCommon;
 extern const char* const kTplUvu;
+extern const char* const kTplUvuFc;
 extern const char* const kTplUvwSmall;
 extern const char* const kTplUvwMfma;
 extern const char* const kTplUvwMfmaBf16;

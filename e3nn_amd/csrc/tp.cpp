@@ -55,6 +55,9 @@ struct e3x_plan {
   bool zero_fill = false;  // some output irrep is reached by no instruction
   int n_targets = 0;       // uvw_mfma: grid.y
   std::vector<int> node_tile_rows;  // uvw_node: rows per workgroup of each target, in grid order
+  // uvu: the message kernel with the radial network inside, one per network description, built on first use
+  std::unique_ptr<SubKernel> radial;
+  std::string radial_desc;
   std::mutex mu;
   std::vector<std::unique_ptr<SubKernel>> subs;
   // uvw_mfma: the weight-gradient kernel is a code object of its own, built on first use
@@ -175,7 +178,9 @@ std::vector<std::vector<int>> split_uvu_paths(const e3x_plan& P) {
   return parts;
 }
 
-int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only = false) {
+// extra_cfg: more constants for the generated namespace; tpl: the device template to specialise (default: uvu.inc)
+int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only = false, const std::string* extra_cfg = nullptr,
+                     const char* tpl = nullptr) {
   int max_mul = 1;
   std::vector<char> used1(P.in1.size(), 0), usedo(P.out.size(), 0);
   long long unrolled = 0;
@@ -277,8 +282,9 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only 
   // - 2 % on the 128-channel l <= 3 set in fp32, whose operands alone take ~150 registers.
   const bool loads_first = P.dtype == E3X_BF16 || upl * (accregs + x1regs + wregs) + (int)P.in2_dim <= 140;
   if (env_int("E3X_UVU_SCHED", loads_first ? 1 : 0) == 0) s << "#define E3X_UVU_SCHED 0\n";
+  if (extra_cfg) s << *extra_cfg;
   s << "}  // namespace cfg\n";
-  *src = s.str() + e3x::kTplCommon + e3x::kTplUvu;
+  *src = s.str() + e3x::kTplCommon + (tpl ? tpl : e3x::kTplUvu);
   return E3X_OK;
 }
 
@@ -954,6 +960,121 @@ extern "C" int e3x_tp_gather_scatter_ordered(e3x_plan* P, const void* node_x, co
     if (err != hipSuccess)
       return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
   }
+  return E3X_OK;
+}
+
+// ---- message step with the radial network inside ---------------------------------------------------------
+namespace {
+
+// what the fused kernel assumes about the instruction set
+const char* radial_unsupported(const e3x_plan* P) {
+  if (P->family != "uvu") return "the plan must be all-uvu";
+  if (P->dtype != E3X_F32) return "fp32 storage only";
+  if (P->shared_weights || P->paths.empty()) return "per-edge weights are required";
+  if (P->in2_dim > 64) return "irreps_in2.dim > 64";
+  for (size_t i = 0; i < P->paths.size(); ++i) {
+    const PathInfo& p = P->paths[i];
+    if (!p.has_w || P->in2[p.in2].mul != 1 || P->in1[p.in1].mul != 32 || P->out[p.out].mul != 32 || p.woff != 32 * (int)i)
+      return "every instruction needs a weight, multiplicity 32 on the first input and the output, 1 on the second";
+  }
+  return nullptr;
+}
+
+int prepare_radial(e3x_plan* P, int n_in, int n_hidden, int act, double c1, double c2) {
+  std::ostringstream d;
+  d << n_in << "/" << n_hidden << "/" << act << "/" << fstr(c1) << "/" << fstr(c2);
+  std::lock_guard<std::mutex> lock(P->mu);
+  if (P->radial && P->radial_desc == d.str()) return E3X_OK;
+  std::unique_ptr<SubKernel> K(new SubKernel);
+  for (size_t i = 0; i < P->paths.size(); ++i) K->path_ids.push_back((int)i);
+  std::ostringstream x;
+  x << "constexpr int FC_H0 = " << n_in << ", FC_H1 = " << n_hidden << ", FC_ACT = " << act << ";\n";
+  x << "constexpr float FC_C1 = " << fstr(c1) << ", FC_C2 = " << fstr(c2) << ";\n";
+  if (std::getenv("E3X_UVUFC_STAGGER")) x << "#define E3X_UVUFC_STAGGER " << env_int("E3X_UVUFC_STAGGER", 1) << "\n";
+  const std::string extra = x.str();
+  std::string src;
+  int rc;
+  if ((rc = build_uvu_source(*P, *K, &src, false, &extra, e3x::kTplUvuFc))) return rc;
+  if ((rc = e3x::get_code_object("uvu_fc", src, &K->key, &K->hsaco))) return rc;
+  P->radial = std::move(K);
+  P->radial_desc = d.str();
+  return E3X_OK;
+}
+
+int load_radial_function(e3x_plan* P, int dev) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  SubKernel* K = P->radial.get();
+  if (K->module[dev]) return E3X_OK;
+  hipModule_t mod = nullptr;
+  hipError_t err = hipModuleLoad(&mod, K->hsaco.c_str());
+  if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + K->hsaco + ") failed: " + hipGetErrorString(err));
+  if (hipModuleGetFunction(&K->fn_fused[dev], mod, "e3x_uvu_fc_fused") != hipSuccess)
+    return fail(E3X_ERR_HIP, "kernel e3x_uvu_fc_fused missing from " + K->hsaco);
+  K->module[dev] = mod;
+  return E3X_OK;
+}
+
+}  // namespace
+
+// validation of the network description and construction of the kernel (shared by the two entry points below)
+static int radial_kernel(e3x_plan* P, int32_t n_in, int32_t n_hidden, int32_t act, double act_cst, double variance_in,
+                         double variance_out) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: null plan");
+  if (const char* why = radial_unsupported(P))
+    return fail(E3X_ERR_INVALID, std::string("e3x_tp_gather_scatter_radial: ") + why);
+  if (n_in < 1 || n_in > 64 || n_hidden < 16 || n_hidden > 128 || n_hidden % 16)
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: 1..64 inputs and 16..128 hidden units in multiples of 16");
+  const int64_t packed = (int64_t)((n_in + 3) / 4) * 64 * (n_hidden / 16) + (int64_t)n_hidden * P->weight_numel;
+  if (packed * 4 > 160 * 1024)
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: the network does not fit the LDS of a compute unit");
+  if (act < E3X_ACT_IDENTITY || act > E3X_ACT_RELU) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: unknown activation");
+  if (!(variance_in > 0) || !(variance_out > 0)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: variances must be positive");
+  // e3nn/nn/_fc.py:38-48,70-88 for two layers: act(x @ W1 / sqrt(h0 var_in)) * cst @ W2 / sqrt(h1 / var_out)
+  const bool has_act = act != E3X_ACT_IDENTITY;
+  const double c1 = 1.0 / std::sqrt((double)n_in * variance_in);
+  const double c2 = (has_act ? act_cst : 1.0) * std::sqrt(variance_out / (double)n_hidden);
+  return prepare_radial(P, n_in, n_hidden, act, c1, c2);
+}
+
+extern "C" int e3x_tp_plan_prepare_radial(e3x_plan* P, int32_t n_in, int32_t n_hidden, int32_t act, double act_cst,
+                                          double variance_in, double variance_out) {
+  return radial_kernel(P, n_in, n_hidden, act, act_cst, variance_in, variance_out);
+}
+
+extern "C" int e3x_tp_gather_scatter_radial(e3x_plan* P, const void* node_x, const void* edge_attr,
+                                            const void* edge_scalars, const void* w1, const void* w2, int32_t n_in,
+                                            int32_t n_hidden, int32_t act, double act_cst, double variance_in,
+                                            double variance_out, const void* src, int idx_bits, const int32_t* rowptr,
+                                            const int32_t* perm, void* out, int64_t E, int64_t num_src_nodes,
+                                            int64_t num_out_nodes, void* stream) {
+  int rc;
+  if ((rc = radial_kernel(P, n_in, n_hidden, act, act_cst, variance_in, variance_out))) return rc;
+  if (idx_bits != 32 && idx_bits != 64) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: idx_bits must be 32 or 64");
+  if (E < 0 || num_src_nodes < 0 || num_out_nodes < 0) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: negative size");
+  if (E >= (1LL << 31) || num_src_nodes >= (1LL << 31))
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: edge and node counts must fit in int32");
+  if (num_out_nodes == 0 || P->out_dim == 0) return E3X_OK;
+  if (!out || !rowptr || (E > 0 && (!src || !node_x || (P->in2_dim && !edge_attr) || !edge_scalars || !w1 || !w2)))
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  int dev;
+  if ((rc = current_device(&dev))) return rc;
+  // rows are written by stores or by atomic additions, rows without edges by nobody: everything starts at zero
+  if ((rc = zero_output(P, out, num_out_nodes, st))) return rc;
+  if (E == 0) return E3X_OK;
+  if ((rc = load_radial_function(P, dev))) return rc;
+  int n_cu = 0;
+  if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0) n_cu = 256;
+  // one persistent workgroup of 8 waves per compute unit, 32 workers (quads) each; no more workers than groups of 4 edges
+  long long blocks = std::min<long long>(n_cu, (E + 127) / 128);
+  int idx64 = idx_bits == 64;
+  long long n_rows = num_out_nodes, n_src = num_src_nodes, n_edges = E;
+  void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&edge_scalars, (void*)&w1,     (void*)&w2,
+                  (void*)&out,    (void*)&src,       (void*)&idx64,        (void*)&rowptr, (void*)&perm,
+                  (void*)&n_rows, (void*)&n_src,     (void*)&n_edges};
+  hipError_t err = hipModuleLaunchKernel(P->radial->fn_fused[dev], (unsigned)blocks, 1, 1, 512, 1, 1, 0, st, args, nullptr);
+  if (err != hipSuccess)
+    return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter_radial: launch failed: ") + hipGetErrorString(err));
   return E3X_OK;
 }
 

@@ -61,12 +61,21 @@ class Convolution(torch.nn.Module):
         ), f"irreps_mid={irreps_mid} and irreps_node_attr={self.irreps_node_attr} are not able to generate scalars"
 
     def forward(self, node_input, node_attr, edge_src, edge_dst, edge_attr, edge_scalars, edges=None) -> torch.Tensor:
-        weight = self.fc(edge_scalars)
         node_self_connection = self.sc(node_input, node_attr)
         node_features = self.lin1(node_input, node_attr)
         if edges is None:
             edges = DstSortedEdges(edge_src, edge_dst, node_input.shape[0])
-        node_features = self.tp.forward_gather_scatter(node_features, edge_attr, weight, edges=edges)
+        messages = None
+        wants_grad = torch.is_grad_enabled() and (
+            any(t.requires_grad for t in (node_features, edge_attr, edge_scalars)) or any(p.requires_grad for p in self.fc.parameters())
+        )
+        if not wants_grad:
+            # the radial network inside the message kernel: the [E, weight_numel] weights are never stored
+            messages = self.tp.forward_gather_scatter_radial(node_features, edge_attr, edge_scalars, self.fc, edges)
+        if messages is None:
+            weight = self.fc(edge_scalars)
+            messages = self.tp.forward_gather_scatter(node_features, edge_attr, weight, edges=edges)
+        node_features = messages
         # lin2 and alpha are linear in the features, so the division by sqrt(num_neighbors) that the reference applies
         # to the summed messages (points_convolution.py:108) is applied to their outputs instead, which are four to a
         # thousand times narrower than the messages

@@ -124,6 +124,23 @@ class _Plan:
             )
         return out
 
+    def gather_scatter_radial(self, table, edge_attr, edge_scalars, w1, w2, act_kind, act_cst, variance_in, variance_out,
+                              gather_idx, edges, num_table_rows):
+        """``gather_scatter`` with the per-edge weights computed in the kernel by the two-layer network
+        ``(edge_scalars, w1, w2)``; returns None when the library does not take this instruction set or network."""
+        out = torch.empty(edges.num_nodes, self.out_dim, dtype=table.dtype, device=table.device)
+        with torch.cuda.device(table.device):
+            rc = _lib.lib().e3x_tp_gather_scatter_radial(
+                self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(edge_scalars), _lib.ptr(w1), _lib.ptr(w2),
+                w1.shape[0], w1.shape[1], act_kind, act_cst, float(variance_in), float(variance_out), _lib.ptr(gather_idx),
+                gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(out), edges.num_edges,
+                num_table_rows, edges.num_nodes, _lib.stream_ptr(table.device),
+            )  # fmt: skip
+        if rc == _lib.ERR_INVALID:
+            return None
+        _lib.check(rc)
+        return out
+
     def backward_w_uvw(self, x1, x2, grad_out, shared_weights):
         shape = (self.weight_numel,) if shared_weights else (x1.shape[0], self.weight_numel)
         gw = torch.empty(shape, dtype=x1.dtype, device=x1.device)
@@ -706,6 +723,56 @@ class TensorProduct(torch.nn.Module):
         else:
             w = node_x.new_empty(0)
         return _GatherScatterFn.apply(node_x.contiguous(), edge_attr.to(node_x.dtype).contiguous(), w, self, edges)
+
+
+    def _radial_description(self, net):
+        """Arguments of the library's fused radial-network kernel for ``net``; None when ``net`` is not a two-layer
+        ``nn.FullyConnectedNet`` ending in this product's per-edge weights."""
+        from ..nn.activation import _KINDS, second_moment_constant
+
+        layers = list(net)
+        if len(layers) != 2 or layers[1].act is not None or net.hs[-1] != self.weight_numel or self.shared_weights:
+            return None
+        if not self.instructions or any(t.connection_mode != "uvu" for t in self.instructions):
+            return None
+        name = layers[0]._act_name or "identity"
+        cst = second_moment_constant(name) if layers[0].act is not None else 1.0
+        return net.hs[0], net.hs[1], _KINDS[name], cst, float(layers[0].var_in), float(layers[1].var_out)
+
+    def prepare_gather_scatter_radial(self, net) -> bool:
+        """Builds the kernel of ``forward_gather_scatter_radial`` for ``net`` ahead of the first call (no GPU needed);
+        False when the instruction set or the network is outside what the kernel takes."""
+        desc = self._radial_description(net)
+        if desc is None:
+            return False
+        rc = _lib.lib().e3x_tp_plan_prepare_radial(self._plan(torch.float32).handle, *desc)
+        if rc == _lib.ERR_INVALID:
+            return False
+        _lib.check(rc)
+        return True
+
+    def forward_gather_scatter_radial(self, node_x, edge_attr, edge_scalars, net, edges):
+        """``forward_gather_scatter(node_x, edge_attr, net(edge_scalars), edges=edges)`` in one kernel, without the
+        ``[E, weight_numel]`` weights ever being stored: ``net`` is a two-layer ``nn.FullyConnectedNet``
+        ``[n_in, n_hidden, weight_numel]``.  Inference only (no autograd graph is recorded); returns None when the
+        instruction set, the network or the tensors are outside what the kernel takes, so that the caller can run the
+        two steps separately."""
+        desc = self._radial_description(net)
+        if desc is None:
+            return None
+        layers = list(net)
+        tensors = (node_x, edge_attr, edge_scalars, layers[0].weight, layers[1].weight)
+        if not all(t.is_cuda and t.dtype == torch.float32 for t in tensors):
+            return None
+        if node_x.ndim != 2 or node_x.shape[-1] != self._in1_dim or edge_attr.shape != (edges.num_edges, self._in2_dim):
+            return None
+        if edge_scalars.shape != (edges.num_edges, net.hs[0]) or edges.num_src_nodes != node_x.shape[0]:
+            return None
+        with torch.no_grad():
+            return self._plan(torch.float32).gather_scatter_radial(
+                node_x.contiguous(), edge_attr.contiguous(), edge_scalars.contiguous(), layers[0].weight.detach().contiguous(),
+                layers[1].weight.detach().contiguous(), desc[2], desc[3], desc[4], desc[5], edges.edge_src, edges, node_x.shape[0],
+            )  # fmt: skip
 
 
 class FullyConnectedTensorProduct(TensorProduct):

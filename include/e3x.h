@@ -154,6 +154,28 @@ int e3x_tp_gather_scatter(e3x_plan* plan, const void* node_x, const void* edge_a
                           const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm, void* out,
                           int64_t E, int64_t num_src_nodes, int64_t num_out_nodes, void* stream);
 
+/* e3x_tp_gather_scatter with the per-edge weights computed inside the kernel by a two-layer radial network,
+ *   w[e, :] = act(edge_scalars[e, :] @ W1 / sqrt(n_in variance_in)) * act_cst @ W2 / sqrt(n_hidden / variance_out),
+ * i.e. weight = fc(edge_length_embedded) followed by the scatter of the tensor product
+ * (e3nn/nn/models/v2106/points_convolution.py:99-106, network e3nn/nn/_fc.py:38-88 with hs = {n_in, n_hidden,
+ * weight_numel}, out_act = False); the [E, weight_numel] weights are never stored.  w1 [n_in, n_hidden] and
+ * w2 [n_hidden, weight_numel] are the reference's layer0.weight / layer1.weight, edge_scalars [E, n_in].
+ * For fp32 all-uvu plans with per-edge weights on every instruction, multiplicity 32 on the first input and the
+ * output and 1 on the second, n_hidden a multiple of 16 (E3X_ERR_INVALID otherwise: run the network and
+ * e3x_tp_gather_scatter instead).  `out` is fully overwritten.  Rows whose edges straddle the ranges of two of the
+ * kernel's workers are summed with fp32 atomics: their last bits may differ between runs, all others are
+ * reproducible.  The kernel is built on first use (one per network shape). */
+int e3x_tp_gather_scatter_radial(e3x_plan* plan, const void* node_x, const void* edge_attr, const void* edge_scalars,
+                                 const void* w1, const void* w2, int32_t n_in, int32_t n_hidden, int32_t act,
+                                 double act_cst, double variance_in, double variance_out, const void* src, int idx_bits,
+                                 const int32_t* rowptr, const int32_t* perm, void* out, int64_t E,
+                                 int64_t num_src_nodes, int64_t num_out_nodes, void* stream);
+
+/* Builds the kernel of e3x_tp_gather_scatter_radial for one network description ahead of the first call (no GPU
+ * needed); E3X_ERR_INVALID when the plan or the network is outside what the kernel takes. */
+int e3x_tp_plan_prepare_radial(e3x_plan* plan, int32_t n_in, int32_t n_hidden, int32_t act, double act_cst,
+                               double variance_in, double variance_out);
+
 /* Processing order of the output rows for e3x_tp_gather_scatter_ordered: row_order[num_nodes] (int32 device array owned
  * by the caller) is the permutation of the rows sorted, stably, by the smallest source row among their in-edges.  Rows
  * that share their smallest source share most of their sources (a one-permutation min-hash of the neighbour sets), so

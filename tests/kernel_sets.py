@@ -216,6 +216,21 @@ def fused_fc_nets():
     return [nn.FullyConnectedNet(hs, act, variance_in=vi, variance_out=vo, out_act=oa) for hs, act, oa, vi, vo in FUSED_FC_CASES]
 
 
+def radial_message_cases():
+    """(name, all-uvu TensorProduct, two-layer radial network) for the message kernel with the network inside."""
+    from e3nn_amd import nn
+
+    torch.manual_seed(20240612)  # the weights are drawn at construction
+    tp = cfg3(merged=True)
+    small = o3.TensorProduct("32x0e+32x1o", "0e+1o", "32x0e+32x1o+32x1e", [(0, 0, 0, "uvu", True), (0, 1, 1, "uvu", True), (1, 0, 1, "uvu", True),
+                             (1, 1, 0, "uvu", True), (1, 1, 2, "uvu", True)], shared_weights=False, internal_weights=False)  # fmt: skip
+    return [
+        ("nequip_silu", tp, nn.FullyConnectedNet([8, 64, tp.weight_numel], torch.nn.functional.silu)),
+        ("small_tanh", small, nn.FullyConnectedNet([5, 32, small.weight_numel], torch.tanh, variance_in=2, variance_out=3)),
+        ("small_linear", small, nn.FullyConnectedNet([12, 16, small.weight_numel], None)),
+    ]
+
+
 def conv_wide():
     # one interaction block at NequIP-like width: 32 channels per irrep, 4 species, 8 radial basis functions
     from e3nn_amd import nn
@@ -242,9 +257,17 @@ def prebuild(verbose=True, workers=6):
                 jobs.append((f"module {name} (one kernel)", sub, None, False))
     for name, tp, dtypes in all_tensor_products():
         jobs.append((f"kernel {name}", tp, dtypes, name in BACKWARD_CASES))
+    for name, tp, net in radial_message_cases():
+        jobs.append((f"radial {name}", tp, net, False))
+    for name, mod in nn_modules():
+        if isinstance(mod, nn.Convolution):  # the block runs its radial network inside the message kernel when it can
+            jobs.append((f"radial {name}", mod.tp, mod.fc, False))
 
     def build(job):
         name, tp, dtypes, backward = job
+        if name.startswith("radial "):
+            plan = dtypes.fused_plan()  # the network on its own, which the tests run beside the fused kernel
+            return name, ["built" if tp.prepare_gather_scatter_radial(dtypes) else "(separate kernels)", plan.key or ""]
         if dtypes is None:
             plan = tp.fused_plan()
             keys = [plan.key or "(layer by layer: " + plan.reason + ")"]

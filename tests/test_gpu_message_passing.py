@@ -181,3 +181,55 @@ def test_fused_bf16_storage():
     )
     scale = float(np.abs(ref).max())
     assert_close(out, ref, atol=1e-2 * scale, rtol=1e-2, what="bf16 fused")
+
+
+@pytest.mark.parametrize("case,N,E,idx", [
+    ("nequip_silu", 400, 9_000, torch.int64), ("nequip_silu", 30, 3, torch.int32), ("nequip_silu", 5, 4_000, torch.int64),
+    ("small_tanh", 200, 5_001, torch.int32), ("small_linear", 64, 777, torch.int64),
+])  # fmt: skip
+def test_message_with_the_radial_network_inside(case, N, E, idx):
+    """weight = fc(edge_scalars); scatter(tp(x[src], attr, weight), dst) as ONE kernel, against the float64 oracle of
+    the network followed by the oracle of the message step, and against the two separate kernels.  Graphs with
+    more workers than groups of four edges, with rows longer than a worker's range, and with rows without edges."""
+    from oracle import nn as onn
+
+    name, tp, net = next(c for c in ks.radial_message_cases() if c[0] == case)
+    net = net.to(DEV)
+    src, dst = random_graph(N, E, seed=11, dtype=idx)
+    dst[dst == 2] = 3  # node 2 receives nothing
+    node_x = seeded(N, tp.irreps_in1.dim, seed=12)
+    lmax = tp.irreps_in2.lmax
+    attr = o3.spherical_harmonics(list(range(lmax + 1)), seeded(E, 3, seed=13).to(DEV), True, "component")
+    scalars = seeded(E, net.hs[0], seed=14)
+    edges = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    out = tp.forward_gather_scatter_radial(node_x.to(DEV), attr, scalars.to(DEV), net, edges)
+    assert out is not None, "the instruction set and the network are inside the kernel's limits"
+    ws = [net.layer0.weight.detach().cpu().numpy(), net.layer1.weight.detach().cpu().numpy()]
+    act = net.layer0._act_name
+    w = onn.fc_forward(ws, scalars.numpy(), act, variance_in=net.layer0.var_in, variance_out=net.layer1.var_out)
+    ref = tp_gather_scatter(oracle_spec(tp), node_x.numpy(), attr.cpu().numpy(), w, src.numpy(), dst.numpy(), N)
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert_close(out, ref, atol=1e-4 * scale, rtol=1e-5, what=f"{case} against the oracle")
+    assert not out[2].any()  # exact zeros where no edge arrives
+    with torch.no_grad():
+        two = tp.forward_gather_scatter(node_x.to(DEV), attr, net(scalars.to(DEV)), edges=edges)
+    assert (out - two).abs().max().item() < 1e-4 * scale
+    # rows that lie inside one worker's range are summed in a fixed order: a second run differs at most in the rows
+    # that straddle two ranges (fp32 atomics), and there only in the last bits
+    again = tp.forward_gather_scatter_radial(node_x.to(DEV), attr, scalars.to(DEV), net, edges)
+    assert (out - again).abs().max().item() <= 1e-5 * scale
+
+
+def test_message_with_the_radial_network_declines_what_it_does_not_take():
+    from e3nn_amd import nn
+
+    tp = ks.cfg3(merged=True)
+    edges = DstSortedEdges(torch.zeros(4, dtype=torch.int64, device=DEV), torch.zeros(4, dtype=torch.int64, device=DEV), 3)
+    x, attr = torch.zeros(3, tp.irreps_in1.dim, device=DEV), torch.zeros(4, tp.irreps_in2.dim, device=DEV)
+    three_layers = nn.FullyConnectedNet([8, 16, 16, tp.weight_numel], torch.tanh).to(DEV)
+    assert tp.forward_gather_scatter_radial(x, attr, torch.zeros(4, 8, device=DEV), three_layers, edges) is None
+    odd_hidden = nn.FullyConnectedNet([8, 24, tp.weight_numel], torch.tanh).to(DEV)  # hidden width not a multiple of 16
+    assert tp.forward_gather_scatter_radial(x, attr, torch.zeros(4, 8, device=DEV), odd_hidden, edges) is None
+    other_mul = ks.cfg4("A")  # multiplicities other than 32
+    net = nn.FullyConnectedNet([8, 16, other_mul.weight_numel], torch.tanh).to(DEV)
+    assert not other_mul.prepare_gather_scatter_radial(net)

@@ -247,6 +247,11 @@ def test_convolution_block_forward_and_backward():
     out = conv(xd, node_attr.to(DEV), src.to(DEV), dst.to(DEV), edge_attr.to(DEV), edge_scalars.to(DEV))
     ref = run(node_input.numpy())
     assert_close(out, ref, atol=1e-4 * max(1.0, float(np.abs(ref).max())), what="convolution block")
+    # without gradients the radial network runs inside the message kernel
+    with torch.no_grad():
+        assert conv.tp.prepare_gather_scatter_radial(conv.fc)
+        out2 = conv(node_input.to(DEV), node_attr.to(DEV), src.to(DEV), dst.to(DEV), edge_attr.to(DEV), edge_scalars.to(DEV))
+    assert_close(out2, ref, atol=1e-4 * max(1.0, float(np.abs(ref).max())), what="convolution block, inference path")
     cot = seeded(N, 288, seed=5)
     out.backward(cot.to(DEV))
     rng = np.random.default_rng(3)
