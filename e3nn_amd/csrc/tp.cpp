@@ -56,7 +56,7 @@ struct e3x_plan {
   int n_targets = 0;       // uvw_mfma: grid.y
   std::vector<int> node_tile_rows;  // uvw_node: rows per workgroup of each target, in grid order
   // uvu: the message kernel with the radial network inside, one per network description, built on first use
-  std::unique_ptr<SubKernel> radial;
+  std::vector<std::unique_ptr<SubKernel>> radial;
   std::string radial_desc;
   std::mutex mu;
   std::vector<std::unique_ptr<SubKernel>> subs;
@@ -142,7 +142,7 @@ void emit_nz_table(std::ostringstream& s, const NzList& L) {
 // Splits the paths into kernels over disjoint output irreps when one kernel would need too many
 // accumulator registers: paths sharing an output stay together, groups are formed per input-1 irrep
 // (so each kernel gathers only its own slice of the source row).
-std::vector<std::vector<int>> split_uvu_paths(const e3x_plan& P) {
+std::vector<std::vector<int>> split_uvu_paths(const e3x_plan& P, int acc_limit = 0) {
   std::vector<int> all(P.paths.size());
   for (size_t i = 0; i < all.size(); ++i) all[i] = (int)i;
   int acc = 0;
@@ -151,13 +151,13 @@ std::vector<std::vector<int>> split_uvu_paths(const e3x_plan& P) {
     if (!usedo[p.out]) { usedo[p.out] = 1; acc += 2 * P.out[p.out].l + 1; }
   // fp32: one kernel up to 128 accumulators per multiplicity index (measured faster on the 99-accumulator
   // MACE set than four kernels); bf16 storage is ALU-bound and prefers the smaller kernels
-  const int limit = P.dtype == E3X_BF16 ? 48 : 128;
+  const int limit = acc_limit > 0 ? acc_limit : (P.dtype == E3X_BF16 ? 48 : 128);
   int x1regs = 0;
   std::vector<char> used1(P.in1.size(), 0);
   for (const auto& p : P.paths)
     if (!used1[p.in1]) { used1[p.in1] = 1; x1regs += 2 * P.in1[p.in1].l + 1; }
   // (transposed plans of the backward pass have many input irreps instead of many outputs)
-  const int want = env_int("E3X_UVU_SPLIT", (acc > limit || x1regs > 64) ? 1 : 0);
+  const int want = acc_limit > 0 ? (acc > limit) : env_int("E3X_UVU_SPLIT", (acc > limit || x1regs > 64) ? 1 : 0);
   if (!want || P.paths.empty()) return {all};
   // an output irrep fed from several input-1 irreps ties those inputs together
   std::vector<int> group_of_in1(P.in1.size());
@@ -984,33 +984,63 @@ int prepare_radial(e3x_plan* P, int n_in, int n_hidden, int act, double c1, doub
   std::ostringstream d;
   d << n_in << "/" << n_hidden << "/" << act << "/" << fstr(c1) << "/" << fstr(c2);
   std::lock_guard<std::mutex> lock(P->mu);
-  if (P->radial && P->radial_desc == d.str()) return E3X_OK;
-  std::unique_ptr<SubKernel> K(new SubKernel);
-  for (size_t i = 0; i < P->paths.size(); ++i) K->path_ids.push_back((int)i);
+  if (!P->radial.empty() && P->radial_desc == d.str()) return E3X_OK;
   std::ostringstream x;
   x << "constexpr int FC_H0 = " << n_in << ", FC_H1 = " << n_hidden << ", FC_ACT = " << act << ";\n";
   x << "constexpr float FC_C1 = " << fstr(c1) << ", FC_C2 = " << fstr(c2) << ";\n";
   if (std::getenv("E3X_UVUFC_STAGGER")) x << "#define E3X_UVUFC_STAGGER " << env_int("E3X_UVUFC_STAGGER", 1) << "\n";
+  if (std::getenv("E3X_UVUFC_SPLIT")) x << "#define E3X_UVUFC_SPLIT " << env_int("E3X_UVUFC_SPLIT", 1) << "\n";
   const std::string extra = x.str();
-  std::string src;
-  int rc;
-  if ((rc = build_uvu_source(*P, *K, &src, false, &extra, e3x::kTplUvuFc))) return rc;
-  if ((rc = e3x::get_code_object("uvu_fc", src, &K->key, &K->hsaco))) return rc;
-  P->radial = std::move(K);
+  // A lane keeps the accumulators of two multiplicity indices next to 8 registers of weights per instruction: above
+  // 18 output components per index the instructions are dealt to several kernels over disjoint output irreps (one
+  // per group of first-input irreps, so each kernel gathers only its own slice of the source row).
+  std::vector<std::unique_ptr<SubKernel>> parts;
+  const int acc_limit = env_int("E3X_UVUFC_ACC_LIMIT", 24);
+  std::vector<std::vector<int>> groups = split_uvu_paths(*P, acc_limit);
+  // neighbouring groups are put together again while their output components stay within the limit
+  auto acc_of = [&](const std::vector<int>& ids) {
+    std::vector<char> seen(P->out.size(), 0);
+    int n = 0;
+    for (int id : ids)
+      if (!seen[P->paths[id].out]) { seen[P->paths[id].out] = 1; n += 2 * P->out[P->paths[id].out].l + 1; }
+    return n;
+  };
+  for (size_t g = 0; g + 1 < groups.size();) {
+    std::vector<int> both = groups[g];
+    both.insert(both.end(), groups[g + 1].begin(), groups[g + 1].end());
+    if (acc_of(both) <= acc_limit) {
+      std::sort(both.begin(), both.end());
+      groups[g] = both;
+      groups.erase(groups.begin() + g + 1);
+    } else {
+      ++g;
+    }
+  }
+  for (auto& ids : groups) {
+    std::unique_ptr<SubKernel> K(new SubKernel);
+    K->path_ids = ids;
+    std::string src;
+    int rc;
+    if ((rc = build_uvu_source(*P, *K, &src, false, &extra, e3x::kTplUvuFc))) return rc;
+    if ((rc = e3x::get_code_object("uvu_fc", src, &K->key, &K->hsaco))) return rc;
+    parts.push_back(std::move(K));
+  }
+  P->radial = std::move(parts);
   P->radial_desc = d.str();
   return E3X_OK;
 }
 
 int load_radial_function(e3x_plan* P, int dev) {
   std::lock_guard<std::mutex> lock(P->mu);
-  SubKernel* K = P->radial.get();
-  if (K->module[dev]) return E3X_OK;
-  hipModule_t mod = nullptr;
-  hipError_t err = hipModuleLoad(&mod, K->hsaco.c_str());
-  if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + K->hsaco + ") failed: " + hipGetErrorString(err));
-  if (hipModuleGetFunction(&K->fn_fused[dev], mod, "e3x_uvu_fc_fused") != hipSuccess)
-    return fail(E3X_ERR_HIP, "kernel e3x_uvu_fc_fused missing from " + K->hsaco);
-  K->module[dev] = mod;
+  for (auto& K : P->radial) {
+    if (K->module[dev]) continue;
+    hipModule_t mod = nullptr;
+    hipError_t err = hipModuleLoad(&mod, K->hsaco.c_str());
+    if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + K->hsaco + ") failed: " + hipGetErrorString(err));
+    if (hipModuleGetFunction(&K->fn_fused[dev], mod, "e3x_uvu_fc_fused") != hipSuccess)
+      return fail(E3X_ERR_HIP, "kernel e3x_uvu_fc_fused missing from " + K->hsaco);
+    K->module[dev] = mod;
+  }
   return E3X_OK;
 }
 
@@ -1024,8 +1054,10 @@ static int radial_kernel(e3x_plan* P, int32_t n_in, int32_t n_hidden, int32_t ac
     return fail(E3X_ERR_INVALID, std::string("e3x_tp_gather_scatter_radial: ") + why);
   if (n_in < 1 || n_in > 64 || n_hidden < 16 || n_hidden > 128 || n_hidden % 16)
     return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: 1..64 inputs and 16..128 hidden units in multiples of 16");
-  const int64_t packed = (int64_t)((n_in + 3) / 4) * 64 * (n_hidden / 16) + (int64_t)n_hidden * P->weight_numel;
-  if (packed * 4 > 160 * 1024)
+  // the second layer is held as three bf16 planes (6 bytes per weight) when the hidden width is a multiple of 32
+  const int64_t packed = (int64_t)((n_in + 3) / 4) * 64 * (n_hidden / 16) * 4 +
+                         (int64_t)n_hidden * P->weight_numel * (n_hidden % 32 == 0 ? 6 : 4);
+  if (packed > 160 * 1024)
     return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: the network does not fit the LDS of a compute unit");
   if (act < E3X_ACT_IDENTITY || act > E3X_ACT_RELU) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: unknown activation");
   if (!(variance_in > 0) || !(variance_out > 0)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_radial: variances must be positive");
@@ -1072,9 +1104,11 @@ extern "C" int e3x_tp_gather_scatter_radial(e3x_plan* P, const void* node_x, con
   void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&edge_scalars, (void*)&w1,     (void*)&w2,
                   (void*)&out,    (void*)&src,       (void*)&idx64,        (void*)&rowptr, (void*)&perm,
                   (void*)&n_rows, (void*)&n_src,     (void*)&n_edges};
-  hipError_t err = hipModuleLaunchKernel(P->radial->fn_fused[dev], (unsigned)blocks, 1, 1, 512, 1, 1, 0, st, args, nullptr);
-  if (err != hipSuccess)
-    return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter_radial: launch failed: ") + hipGetErrorString(err));
+  for (auto& K : P->radial) {
+    hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 512, 1, 1, 0, st, args, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter_radial: launch failed: ") + hipGetErrorString(err));
+  }
   return E3X_OK;
 }
 
