@@ -326,6 +326,30 @@ def bench_radial_network(args, dev, ctx):
             "frac_hbm_peak": out_bytes / (ms1 * 1e-3) / 1e9 / HBM_PEAK_GBS}  # fmt: skip
 
 
+def bench_radial_message(args, dev, ctx):
+    """weight = fc(edge_scalars); scatter(tp(x[src], attr, weight), dst) on the headline graph and instruction set
+    (reference e3nn/nn/models/v2106/points_convolution.py:99-106): the radial network 8 -> 64 -> 352 inside the message
+    kernel, against the two kernels run one after the other."""
+    from e3nn_amd.nn import DstSortedEdges, FullyConnectedNet
+
+    tp, E = ctx["tp"], ctx["src"].shape[0]
+    torch.manual_seed(0)
+    net = FullyConnectedNet([8, 64, tp.weight_numel], torch.nn.functional.silu).to(dev)
+    s = torch.randn(E, 8, generator=torch.Generator().manual_seed(1)).to(dev)
+    edges = DstSortedEdges(ctx["src"], ctx["dst"], ctx["N"])
+    with torch.no_grad():
+        fused = tp.forward_gather_scatter_radial(ctx["node_x"], ctx["attr"], s, net, edges)
+        assert fused is not None
+        ref = tp.forward_gather_scatter(ctx["node_x"], ctx["attr"], net(s), edges=edges)
+        err = float((fused - ref).abs().max()) / max(1.0, float(ref.abs().max()))
+        assert err < 1e-4, err
+        ms_f = event_time_ms(lambda: tp.forward_gather_scatter_radial(ctx["node_x"], ctx["attr"], s, net, edges), max(5, args.steps // 2), 3)
+        ms_s = event_time_ms(lambda: tp.forward_gather_scatter(ctx["node_x"], ctx["attr"], net(s), edges=edges), max(5, args.steps // 2), 3)
+    flop = 2.0 * E * (8 * 64 + 64 * tp.weight_numel)
+    return {"edges": E, "ms_one_kernel": ms_f, "ms_network_then_message": ms_s, "edges_per_s_one_kernel": E / (ms_f * 1e-3),
+            "network_tflops_one_kernel": flop / (ms_f * 1e-3) / 1e12, "max_rel_difference": err}  # fmt: skip
+
+
 def bench_library_gemm(args, dev):
     """Context for the matrix-core rooflines: what the vendor GEMM (torch.matmul -> rocBLAS / hipBLASLt) reaches
     on this GPU with N(0,1) data, 8192^3."""
@@ -427,6 +451,8 @@ def main():
         other["convolution_block"] = bench_convolution(args, dev, ctx)
     if "radial" in want:
         other["radial_network_8_64_352"] = bench_radial_network(args, dev, ctx)
+    if "radial" in want:
+        other["nequip_message_with_radial_network"] = bench_radial_message(args, dev, ctx)
     if "nequip_bwd" in want:
         other["nequip_uvu_forward_backward"] = bench_nequip_backward(args, dev, ctx)
     if "uvw_bwd" in want:
