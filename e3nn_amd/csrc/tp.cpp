@@ -57,6 +57,7 @@ struct e3x_plan {
   std::vector<int> node_tile_rows;  // uvw_node: rows per workgroup of each target, in grid order
   // uvu: the message kernel with the radial network inside, one per network description, built on first use
   std::vector<std::unique_ptr<SubKernel>> radial;
+  std::vector<std::unique_ptr<SubKernel>> radial_retired;  // kernels of earlier network descriptions: a launch may still hold them
   std::string radial_desc;
   std::mutex mu;
   std::vector<std::unique_ptr<SubKernel>> subs;
@@ -1025,6 +1026,7 @@ int prepare_radial(e3x_plan* P, int n_in, int n_hidden, int act, double c1, doub
     if ((rc = e3x::get_code_object("uvu_fc", src, &K->key, &K->hsaco))) return rc;
     parts.push_back(std::move(K));
   }
+  for (auto& old : P->radial) P->radial_retired.push_back(std::move(old));
   P->radial = std::move(parts);
   P->radial_desc = d.str();
   return E3X_OK;
@@ -1104,7 +1106,12 @@ extern "C" int e3x_tp_gather_scatter_radial(e3x_plan* P, const void* node_x, con
   void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&edge_scalars, (void*)&w1,     (void*)&w2,
                   (void*)&out,    (void*)&src,       (void*)&idx64,        (void*)&rowptr, (void*)&perm,
                   (void*)&n_rows, (void*)&n_src,     (void*)&n_edges};
-  for (auto& K : P->radial) {
+  std::vector<SubKernel*> parts;
+  {
+    std::lock_guard<std::mutex> lock(P->mu);
+    for (auto& K : P->radial) parts.push_back(K.get());
+  }
+  for (SubKernel* K : parts) {
     hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 512, 1, 1, 0, st, args, nullptr);
     if (err != hipSuccess)
       return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter_radial: launch failed: ") + hipGetErrorString(err));
