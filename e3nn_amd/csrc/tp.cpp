@@ -989,7 +989,6 @@ int prepare_radial(e3x_plan* P, int n_in, int n_hidden, int act, double c1, doub
   std::ostringstream x;
   x << "constexpr int FC_H0 = " << n_in << ", FC_H1 = " << n_hidden << ", FC_ACT = " << act << ";\n";
   x << "constexpr float FC_C1 = " << fstr(c1) << ", FC_C2 = " << fstr(c2) << ";\n";
-  if (std::getenv("E3X_UVUFC_STAGGER")) x << "#define E3X_UVUFC_STAGGER " << env_int("E3X_UVUFC_STAGGER", 1) << "\n";
   if (std::getenv("E3X_UVUFC_SPLIT")) x << "#define E3X_UVUFC_SPLIT " << env_int("E3X_UVUFC_SPLIT", 1) << "\n";
   const std::string extra = x.str();
   // A lane keeps the accumulators of two multiplicity indices next to 8 registers of weights per instruction: above
