@@ -263,3 +263,36 @@ def test_state_dict_keys_match_the_reference():
     assert torch.equal(tp._compiled_main_left_right._w3j_1_2_1, o3.wigner_3j(1, 2, 1))
     with pytest.raises(NotImplementedError):  # the reference's right() has no triangular modes
         o3.TensorProduct("4x1o", "4x1o", "6x1e", [(0, 0, 0, "uvu<v", True)], compile_right=True)
+
+
+def test_kernel_family_selection_for_scalar_second_inputs():
+    """Shared-weight uvw products whose second input holds scalars only take the node-wise matrix-core kernel when the
+    input multiplicities are multiples of 8; a handful of (u, v) pairs stays on the vector-ALU kernel with its weights
+    in registers; anything with a non-scalar second input, per-sample weights or bf16 storage takes the other kernels."""
+    fam = lambda tp, dt=torch.float32: tp._plan(dt).family  # noqa: E731
+    assert fam(ks.node_fctp()) == fam(ks.node_narrow()) == fam(ks.node_partial_tile()) == fam(ks.node_wide_out()) == "uvw_node"
+    assert fam(ks.outer_split()) == fam(ks.mfma_small()) == "uvw_mfma"  # second input with l > 0
+    assert fam(o3.FullyConnectedTensorProduct("8x0e+8x1o", "2x0e", "8x0e+8x1o")) == "uvw_small"  # 32 pairs: cached weights
+    assert fam(o3.FullyConnectedTensorProduct("12x0e", "4x0e", "32x0e")) == "uvw_small"  # multiplicity not a multiple of 8
+    assert fam(o3.FullyConnectedTensorProduct("64x0e", "4x0e", "64x0e", shared_weights=False, internal_weights=False)) == "uvw_small"
+    assert fam(ks.cfg5(), torch.bfloat16) == "uvw_mfma"
+
+
+def test_radial_message_kernel_is_offered_only_for_what_it_takes():
+    """forward_gather_scatter_radial: two-layer network ending in the product's per-edge weights, all-uvu instructions
+    with multiplicity 32; everything else is declined (None / False) so that callers run the two kernels."""
+    from e3nn_amd import nn
+
+    tp = ks.cfg3(merged=True)
+    good = nn.FullyConnectedNet([8, 64, tp.weight_numel], torch.nn.functional.silu)
+    assert tp._radial_description(good) == (8, 64, 1, pytest.approx(1.679, abs=2e-3), 1.0, 1.0)
+    assert tp.prepare_gather_scatter_radial(good)  # builds (or finds) the kernel without a GPU
+    assert tp._radial_description(nn.FullyConnectedNet([8, 64, 64, tp.weight_numel], torch.tanh)) is None  # three layers
+    assert tp._radial_description(nn.FullyConnectedNet([8, 64, tp.weight_numel], torch.tanh, out_act=True)) is None
+    assert tp._radial_description(nn.FullyConnectedNet([8, 64, tp.weight_numel + 32], torch.tanh)) is None  # other width
+    assert not tp.prepare_gather_scatter_radial(nn.FullyConnectedNet([8, 24, tp.weight_numel], torch.tanh))  # hidden % 16
+    assert not tp.prepare_gather_scatter_radial(nn.FullyConnectedNet([100, 64, tp.weight_numel], torch.tanh))  # inputs > 64
+    other = ks.cfg4("A")  # multiplicities other than 32
+    assert not other.prepare_gather_scatter_radial(nn.FullyConnectedNet([8, 16, other.weight_numel], torch.tanh))
+    shared = ks.golden_tp("uvu_shared_v2")  # shared weights: nothing per edge to compute
+    assert shared._radial_description(nn.FullyConnectedNet([8, 16, shared.weight_numel], torch.tanh)) is None
