@@ -323,7 +323,9 @@ def bench_radial_network(args, dev, ctx):
     out_bytes = E * (8 + 352) * 4
     return {"edges": E, "ms_one_kernel": ms1, "ms_layer_by_layer": msl, "tflops_one_kernel": flop / (ms1 * 1e-3) / 1e12,
             "frac_fp32_mfma_peak": flop / (ms1 * 1e-3) / 1e12 / 157.3, "hbm_gbs_one_kernel": out_bytes / (ms1 * 1e-3) / 1e9,
-            "frac_hbm_peak": out_bytes / (ms1 * 1e-3) / 1e9 / HBM_PEAK_GBS}  # fmt: skip
+            "frac_hbm_peak": out_bytes / (ms1 * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "arithmetic": "layer 64->352: six bf16 MFMA products of three-way split operands, fp32 accumulation (fp32-accurate); "
+                          "tflops / frac_fp32_mfma_peak count the 2*m*n*k flops of the fp32 product"}  # fmt: skip
 
 
 def bench_radial_message(args, dev, ctx):

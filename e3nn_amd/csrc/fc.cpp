@@ -32,7 +32,8 @@ struct e3x_fc_plan {
   bool epilogue = false;  // outputs are multiplied by an activation derivative of a caller-supplied tensor
   int input_act = 0;      // the rows given are pre-activations: the network starts from input_cst * act(x)
   double input_cst = 1.0;
-  int64_t packed_numel = 0;
+  int64_t packed_numel = 0;   // floats of the packed network (a split layer takes 1.5 per weight)
+  int64_t logical_numel = 0;  // weights of the padded network
   std::string key, hsaco;
   std::mutex mu;
   hipModule_t module[kMaxDevices] = {nullptr};
@@ -58,6 +59,11 @@ std::string fstr(double v) {
 }
 
 int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+bool env_split() {
+  const char* v = std::getenv("E3X_FC_SPLIT");
+  return !(v && v[0] == '0');
+}
 
 int load_functions(e3x_fc_plan* P, int dev) {
   std::lock_guard<std::mutex> lock(P->mu);
@@ -101,9 +107,24 @@ extern "C" int e3x_fc_plan_create_fused(const int32_t* hs, int32_t n_hs, int32_t
     P->hs.push_back(hs[i]);
     P->hp.push_back(round_up(hs[i], i == 0 ? 8 : 32));
   }
-  for (int l = 0; l < NL; ++l) P->packed_numel += (int64_t)P->hp[l] * P->hp[l + 1];
+  for (int l = 0; l < NL; ++l) P->logical_numel += (int64_t)P->hp[l] * P->hp[l + 1];
+  P->packed_numel = P->logical_numel;
   if (P->packed_numel * 4 > kMaxPackedBytes)
     return fail(E3X_ERR_INVALID, "e3x_fc_plan_create: the weights of the network do not fit the LDS of a compute unit");
+  // Layers with a narrow input (<= 64, the three bf16 images of the input cost 3/4 of its width in registers) and at
+  // least four output tiles run as six bf16 matrix products (fp32-accurate, 3/8 of the matrix time) while the packed
+  // network (6 bytes per weight of such a layer) still fits the LDS; the widest first.
+  std::vector<int> split(NL, 0);
+  if (env_split()) {
+    std::vector<int> order;
+    for (int l = 0; l < NL; ++l)
+      if (P->hp[l] % 16 == 0 && P->hp[l] >= 32 && P->hp[l] <= 64 && P->hp[l + 1] >= 128) order.push_back(l);
+    std::sort(order.begin(), order.end(), [&](int a, int b) { return (int64_t)P->hp[a] * P->hp[a + 1] > (int64_t)P->hp[b] * P->hp[b + 1]; });
+    for (int l : order) {
+      const int64_t extra = (int64_t)P->hp[l] * P->hp[l + 1] / 2;
+      if ((P->packed_numel + extra) * 4 <= kMaxPackedBytes) split[l] = 1, P->packed_numel += extra;
+    }
+  }
 
   // e3nn/nn/_fc.py:70-88: every layer but the last is followed by act (unit second moment: cst * act) and has
   // var_out = 1; the last has var_out = variance_out and act only with out_act.  _fc.py:38-48: with act,
@@ -152,6 +173,8 @@ extern "C" int e3x_fc_plan_create_fused(const int32_t* hs, int32_t n_hs, int32_t
   for (int i = 0; i <= NL; ++i) s << (i ? ", " : "") << P->hp[i];
   s << "};\nconstexpr int ACT[NL] = {";
   for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << acts[l];
+  s << "};\nconstexpr bool SPLITL[NL] = {";
+  for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << (split[l] ? "true" : "false");
   s << "};\nconstexpr float WSCALE[NL] = {";
   for (int l = 0; l < NL; ++l) s << (l ? ", " : "") << fstr(wscale[l]);
   s << "};\nconstexpr float OUT_POST = " << fstr(out_post) << ";\n";
@@ -264,7 +287,7 @@ extern "C" int e3x_fc_forward_epilogue(e3x_fc_plan* P, const void* x, const void
   hipStream_t st = (hipStream_t)stream;
   {
     void* args[] = {&ptrs, &workspace};
-    hipError_t err = hipModuleLaunchKernel(P->fn_pack[dev], (unsigned)((P->packed_numel + 255) / 256), 1, 1, 256, 1, 1, 0, st,
+    hipError_t err = hipModuleLaunchKernel(P->fn_pack[dev], (unsigned)((P->logical_numel + 255) / 256), 1, 1, 256, 1, 1, 0, st,
                                            args, nullptr);
     if (err != hipSuccess) return fail(E3X_ERR_HIP, std::string("e3x_fc_forward: pack launch failed: ") + hipGetErrorString(err));
   }
