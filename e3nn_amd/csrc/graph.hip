@@ -96,6 +96,21 @@ __global__ __launch_bounds__(kBlock) void order_score_kernel(const int* __restri
   if (hits) atomicAdd(score, hits);
 }
 
+// One more level of the row key for graphs whose sources and destinations are the same node set:
+// level[n] <- key[level[n]] (the smallest source of the row's current key node), and its value for the rows in
+// their current order
+__global__ __launch_bounds__(kBlock) void level_key_kernel(const int* __restrict__ order, const unsigned* __restrict__ keys,
+                                                           unsigned* __restrict__ level, unsigned* __restrict__ by_position,
+                                                           long long N, int first) {
+  for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < N; i += (long long)gridDim.x * kBlock) {
+    const int n = order[i];
+    const unsigned prev = first ? keys[n] : level[n];  // each row appears once in `order`: no other thread touches level[n]
+    const unsigned next = prev < (unsigned)N ? keys[prev] : 0xffffffffu;
+    level[n] = next;
+    by_position[i] = next;
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void fill_zero_kernel(int* p, int n) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -210,7 +225,7 @@ extern "C" size_t e3x_row_order_workspace_bytes(int64_t num_nodes) {
   size_t temp = 0;
   (void)rocprim::radix_sort_pairs(nullptr, temp, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr, (int*)nullptr,
                                   (size_t)(num_nodes > 0 ? num_nodes : 1), 0, 32, (hipStream_t)0);
-  return 256 + 4 * n4 + align_up(temp, 256);  // score | keys_in | keys_out | ids_in | second | rocPRIM temp
+  return 256 + 6 * n4 + align_up(temp, 256);  // score | keys_in | keys_out | ids_in | second | level | level keys | rocPRIM temp
 }
 
 extern "C" int e3x_row_order_build(const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm, int64_t E,
@@ -232,8 +247,10 @@ extern "C" int e3x_row_order_build(const void* src, int idx_bits, const int32_t*
   unsigned* keys_out = (unsigned*)(ws + 256 + n4);
   int* ids_in = (int*)(ws + 256 + 2 * n4);
   unsigned* second = (unsigned*)(ws + 256 + 3 * n4);
-  void* temp = ws + 256 + 4 * n4;
-  size_t temp_bytes = workspace_bytes - 256 - 4 * n4;
+  unsigned* level = (unsigned*)(ws + 256 + 4 * n4);
+  unsigned* level_keys = (unsigned*)(ws + 256 + 5 * n4);
+  void* temp = ws + 256 + 6 * n4;
+  size_t temp_bytes = workspace_bytes - 256 - 6 * n4;
   hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(kBlock), 0, st, score, 1);
   if (idx_bits == 64)
     hipLaunchKernelGGL((rowkey_kernel<long long>), dim3(grid_for(num_nodes, kBlock)), dim3(kBlock), 0, st, (const long long*)src,
@@ -245,6 +262,22 @@ extern "C" int e3x_row_order_build(const void* src, int idx_bits, const int32_t*
   // stable: rows with the same key keep their numbering
   hipError_t err = rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, ids_in, row_order, (size_t)num_nodes, 0, 32, st);
   if (err != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_row_order_build: radix sort failed");
+  // Sources and destinations numbered alike (one node set): two more levels, key of the key.  Rows are then grouped
+  // by (smallest source of the smallest source of their smallest source, ..., smallest source), which puts groups of
+  // rows with neighbouring key nodes next to each other as well.  Two stable sorts, the most significant level last.
+  if (num_src_nodes == num_nodes && num_nodes > 1) {
+    int* cur = row_order;
+    int* other = ids_in;
+    for (int lev = 0; lev < 2; ++lev) {
+      hipLaunchKernelGGL(level_key_kernel, dim3(grid_for(num_nodes, kBlock)), dim3(kBlock), 0, st, cur, keys_in, level, level_keys,
+                         (long long)num_nodes, lev == 0 ? 1 : 0);
+      if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_row_order_build: launch failed");
+      err = rocprim::radix_sort_pairs(temp, temp_bytes, level_keys, keys_out, cur, other, (size_t)num_nodes, 0, 32, st);
+      if (err != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_row_order_build: radix sort failed");
+      std::swap(cur, other);
+    }
+    // two sorts: the result is back in row_order
+  }
   if (shared_pairs) {
     hipLaunchKernelGGL(order_score_kernel, dim3(grid_for(num_nodes, kBlock)), dim3(kBlock), 0, st, row_order, keys_in, second,
                        (long long)num_nodes, score);

@@ -177,7 +177,9 @@ int e3x_tp_plan_prepare_radial(e3x_plan* plan, int32_t n_in, int32_t n_hidden, i
                                double variance_in, double variance_out);
 
 /* Processing order of the output rows for e3x_tp_gather_scatter_ordered: row_order[num_nodes] (int32 device array owned
- * by the caller) is the permutation of the rows sorted, stably, by the smallest source row among their in-edges.  Rows
+ * by the caller) is the permutation of the rows sorted, stably, by the smallest source row among their in-edges (with
+ * num_src_nodes == num_nodes, one node set, the sort key is (k3, k2, k1): k1 the smallest source of the row, k2 = k1 of
+ * node k1, k3 = k1 of node k2).  Rows
  * that share their smallest source share most of their sources (a one-permutation min-hash of the neighbour sets), so
  * rows processed next to each other gather the same rows of the node table and find them in L2, whatever the
  * caller's node numbering; the results are bit-identical to the unordered call.  No counterpart in the reference

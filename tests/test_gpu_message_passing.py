@@ -106,8 +106,9 @@ def test_run_to_run_bit_reproducible_and_prebuilt_edges():
 
 @pytest.mark.parametrize("idx", [torch.int32, torch.int64])
 def test_row_processing_order(idx):
-    """The rows are walked in the order of their smallest source row (stable), rows without edges last; the order
-    changes which row a wavefront takes, not what it computes: outputs are bit-identical with and without it."""
+    """The rows are walked in the order of their smallest source row (and, on one node set, of that node's own key, twice
+    over; stable), rows without edges last; the order changes which row a wavefront takes, not what it computes: outputs
+    are bit-identical with and without it."""
     tp = ks.cfg3(True)
     N, E = 900, 15_000
     src, dst = random_graph(N, E, seed=5, dtype=idx)
@@ -119,8 +120,16 @@ def test_row_processing_order(idx):
     assert sorted(order.tolist()) == list(range(N))
     key = np.full(N, 2**32 - 1, dtype=np.int64)
     np.minimum.at(key, dst.long().numpy(), (src.long().numpy() % N))
-    assert np.array_equal(order, np.argsort(key, kind="stable"))
-    assert (key[order[-5:]] == 2**32 - 1).all()  # the test graph has more than five empty rows
+    # sources and destinations are one node set here: rows are grouped by (k3, k2, k1) with k1 the smallest source of the
+    # row, k2 = k1 of node k1, k3 = k1 of node k2 -- three stable sorts, the most significant key last
+    big = 2**32 - 1
+    k2 = np.where(key < N, key[np.minimum(key, N - 1)], big)
+    k3 = np.where(k2 < N, key[np.minimum(k2, N - 1)], big)
+    want = np.argsort(key, kind="stable")
+    want = want[np.argsort(k2[want], kind="stable")]
+    want = want[np.argsort(k3[want], kind="stable")]
+    assert np.array_equal(order, want)
+    assert (key[order[-5:]] == big).all()  # the test graph has more than five empty rows
     plain = DstSortedEdges(src.to(DEV), dst.to(DEV), N, locality_order=False)
     assert plain.row_order is None
     a = tp.forward_gather_scatter(node_x, attr, w, edges=edges)
