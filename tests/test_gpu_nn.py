@@ -112,6 +112,30 @@ def test_fully_connected_net_one_kernel(case):
     assert_close(out.reshape(-1, hs[-1]), want, what="one-kernel fc, batch dims")
 
 
+def test_split_operand_layer_is_as_accurate_as_the_fp32_product():
+    """The 64 -> 352 layer runs as six bf16 matrix products of three-way split operands accumulated in fp32.  Against the
+    float64 product its error is that of an fp32 matrix product (here: torch's), not that of bf16 arithmetic, also for
+    operands with a wide spread of magnitudes."""
+    from e3nn_amd.nn.fc import _FusedPlan
+
+    plan = _FusedPlan([64, 352], "identity", False, 1, 1)
+    assert plan.handle is not None and plan.workspace_bytes == 64 * 352 * 6  # three bf16 planes: the split path
+    g = torch.Generator().manual_seed(7)
+    Z = 4099
+    x = torch.randn(Z, 64, generator=g) * torch.exp(3.0 * torch.randn(Z, 64, generator=g))  # magnitudes over several decades
+    w = torch.randn(64, 352, generator=g) * torch.exp(2.0 * torch.randn(64, 352, generator=g))
+    exact = (x.double() @ w.double()) / 8.0
+    got = plan.forward(x.to(DEV), [w.to(DEV)]).cpu().double()
+    fp32 = ((x.to(DEV) @ w.to(DEV)) / 8.0).cpu().double()
+    scale = (x.double().abs() @ w.double().abs()) / 8.0  # what an error of one rounding per product is measured against
+    err_split = ((got - exact).abs() / scale).max().item()
+    err_fp32 = ((fp32 - exact).abs() / scale).max().item()
+    # (errors relative to sum |x||w|: fp32 accumulation of 64 terms alone gives a few 1e-7)
+    assert err_split < 2e-6, err_split  # bf16 arithmetic would sit near 4e-3, two-way splits near 2e-5
+    assert err_split < 4 * err_fp32 + 2e-7, (err_split, err_fp32)
+    print(f"split-operand product: {err_split:.2e}, fp32 product: {err_fp32:.2e}")
+
+
 @pytest.mark.parametrize("case", range(len(ks.FUSED_FC_CASES)))
 def test_fully_connected_net_gradients(case):
     """Under autograd the dense layers run on the one-layer kernels (x @ W, g @ W^T, x^T g): every gradient against
