@@ -48,6 +48,8 @@ _SIGNATURES = {
     "e3x_tp_forward_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_size_t, c_void_p]),
     "e3x_csr_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "e3x_csr_build": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "e3x_csr_static_scratch_bytes": (c_size_t, []),
+    "e3x_csr_build_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),
     "e3x_index_check": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p]),
     "e3x_tp_gather_scatter": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_int64, c_int64, c_int64, c_void_p]),

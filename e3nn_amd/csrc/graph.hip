@@ -7,7 +7,9 @@
 // permutation (and therefore the summation order) is unique for a given edge list.
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include <rocprim/rocprim.hpp>
 
@@ -18,6 +20,31 @@ namespace {
 constexpr int kBlock = 256;
 
 __device__ int d_flag[4];  // range-check result of e3x_index_check (one copy per device)
+
+// Sort buffers of e3x_csr_build_static.  Every device the library runs on holds its own copy of this array at its
+// own address for the life of the process; host code must use the address hipGetSymbolAddress reports for the
+// current device (static_scratch() below), never the array's name.
+constexpr size_t kStaticScratchBytes = 64u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+// device address of `scratch` on the current device, looked up once per device
+int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return e3x::fail(E3X_ERR_HIP, "e3x_csr_build_static: no current HIP device");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p)
+      return e3x::fail(E3X_ERR_HIP, "e3x_csr_build_static: hipGetSymbolAddress failed");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return E3X_OK;
+}
 
 template <typename IdxT>
 __global__ __launch_bounds__(kBlock) void keys_kernel(const IdxT* __restrict__ dst, long long E, long long N,
@@ -173,6 +200,28 @@ extern "C" size_t e3x_csr_workspace_bytes(int64_t E, int64_t num_nodes) {
   // flags | keys_in | keys_out | ids_in | rocPRIM temp
   return 256 + 3 * e4 + align_up(sort_temp_bytes(E > 0 ? E : 1, num_nodes > 1 ? num_nodes : 2), 256);
 }
+
+extern "C" int e3x_csr_build_static(const void* dst, int idx_bits, int64_t E, int64_t num_nodes, int32_t* rowptr,
+                                    int32_t* perm, void* stream) {
+  if (E < 0 || num_nodes < 0 || E >= (1LL << 31) || num_nodes >= (1LL << 31))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_csr_build_static: E and num_nodes must fit in int32");
+  const size_t need = e3x_csr_workspace_bytes(E, num_nodes);
+  if (need > kStaticScratchBytes) {
+    char msg[200];
+    snprintf(msg, sizeof msg,
+             "e3x_csr_build_static: %lld edges need %zu bytes of sort buffers, the static buffer holds %zu "
+             "(use e3x_csr_build with a workspace)", (long long)E, need, kStaticScratchBytes);
+    return e3x::fail(E3X_ERR_INVALID, msg);
+  }
+  void* ws = nullptr;
+  if (E > 0) {  // E == 0 touches no scratch
+    const int rc = static_scratch(&ws);
+    if (rc != E3X_OK) return rc;
+  }
+  return e3x_csr_build(dst, idx_bits, E, num_nodes, rowptr, perm, ws, kStaticScratchBytes, stream);
+}
+
+extern "C" size_t e3x_csr_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 extern "C" int e3x_csr_build(const void* dst, int idx_bits, int64_t E, int64_t num_nodes, int32_t* rowptr,
                              int32_t* perm, void* workspace, size_t workspace_bytes, void* stream) {
