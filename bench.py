@@ -25,8 +25,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # L2-miss traffic of one e3x_uvu_fused launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt): 3374122 KiB fetched + 56251 KiB written
-NEQUIP_TRAFFIC_BYTES = (3374122 + 56251) * 1024
+# scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt), keyed by the code object the counters were read
+# on: a kernel that has changed since reports no traffic instead of a stale figure.
+NEQUIP_TRAFFIC_BYTES = {
+    "uvu_77a1034ede7bf763fa3ae452": (3374122 + 56251) * 1024,  # 3374122 KiB fetched + 56251 KiB written
+}
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 
@@ -43,6 +46,22 @@ def event_time_ms(fn, steps, warmup):
     end.record()
     torch.cuda.synchronize()
     return beg.elapsed_time(end) / steps
+
+
+def event_times_ms(fn, steps, warmup):
+    """(mean, median, min) duration of fn() over `steps` launches: one HIP event between consecutive launches on the
+    current stream, the mean taken from the first to the last event (exactly `steps` launches)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    ev[0].record()
+    for i in range(steps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    each = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
+    return ev[0].elapsed_time(ev[steps]) / steps, each[len(each) // 2], each[0]
 
 
 def bench_copy(args, dev):
@@ -89,7 +108,7 @@ def radial_weights(r, cutoff, weight_numel, gen, dev):
 def bench_nequip(args, dev):
     from e3nn_amd import o3
     from e3nn_amd.nn import DstSortedEdges
-    from tests import kernel_sets as ks
+    from e3nn_amd import kernel_sets as ks
 
     N, side, cutoff = 50_000, 86.8, 5.0
     pos, src, dst = radius_graph(N, side, cutoff)
@@ -115,13 +134,14 @@ def bench_nequip(args, dev):
     def step():
         out[0] = tp.forward_gather_scatter(node_x, attr, w, edges=edges)
 
-    ms = event_time_ms(step, args.steps, args.warmup)
+    ms, ms_median, ms_min = event_times_ms(step, args.steps, args.warmup)
     # algorithmic bytes: per edge weights + SH + two int64 indices, node table read once, output written once
     bytes_algo = E * (4 * tp.weight_numel + 4 * 9 + 2 * 8) + N * 4 * (tp.irreps_in1.dim + tp.irreps_out.dim)
     gbs = bytes_algo / (ms * 1e-3) / 1e9
     res = {
-        "edges": E, "nodes": N, "ms": ms, "edges_per_s": E / (ms * 1e-3), "bytes_per_launch": bytes_algo,
-        "achieved_gbs": gbs, "edge_sort_ms_per_graph": sort_ms,
+        "edges": E, "nodes": N, "ms": ms, "ms_median": ms_median, "ms_min": ms_min, "edges_per_s": E / (ms * 1e-3),
+        "bytes_per_launch": bytes_algo, "achieved_gbs": gbs, "edge_sort_ms_per_graph": sort_ms,
+        "kernel_key": tp._plan(torch.float32).key,
         "edges_per_s_incl_sort": E / ((ms + sort_ms) * 1e-3),
     }  # fmt: skip
     ctx = dict(tp=tp, node_x=node_x, attr=attr, w=w, src=src_t, dst=dst_t, N=N, out=out[0])
@@ -161,11 +181,13 @@ def bench_nequip(args, dev):
 
 def cpu_baseline_nequip(ctx, n_edges=200_000, reps=3):
     """The reference's CPU path (torch einsum graph + index + scatter_add_) on a slice of the same workload."""
+    from oracle import tensor_product as otp
     from oracle.torch_cpu import tp_gather_scatter_torch
-    from tests.helpers import oracle_spec
 
     torch.set_num_threads(os.cpu_count())
-    spec = oracle_spec(ctx["tp"])
+    tp = ctx["tp"]
+    ins = [(t.i_in1, t.i_in2, t.i_out, t.connection_mode, t.has_weight) for t in tp.instructions]
+    spec = otp.make_spec(str(tp.irreps_in1), str(tp.irreps_in2), str(tp.irreps_out), ins, shared_weights=tp.shared_weights)
     E = min(n_edges, ctx["src"].shape[0])
     node_x = ctx["node_x"].cpu()
     attr, w = ctx["attr"][:E].cpu(), ctx["w"][:E].cpu()
@@ -202,7 +224,7 @@ def bench_sh(args, dev):
 def bench_mace(args, dev, dtype=torch.float32, variant="A"):
     """MACE-style uvu (L=3): variant A keeps 0e,1o,2e,3o outputs (23 paths), B every l <= 3 of either parity (34)."""
     from e3nn_amd.nn import DstSortedEdges
-    from tests import kernel_sets as ks
+    from e3nn_amd import kernel_sets as ks
 
     N, E = 20_000, 500_000
     gen = torch.Generator().manual_seed(0)
@@ -225,7 +247,7 @@ def bench_mace(args, dev, dtype=torch.float32, variant="A"):
 
 def bench_uvw(args, dev, dtype=torch.float32):
     """Dense uvw: FCTP(128x0e+128x1o+128x2e x same -> same), 65536 rows, shared weights N(0, 1/fan_in)."""
-    from tests import kernel_sets as ks
+    from e3nn_amd import kernel_sets as ks
 
     tp = ks.cfg5().to(dev)
     Z = 65536
@@ -248,7 +270,7 @@ def bench_nequip_cube40(args, dev):
     """The headline configuration as literally stated: 50 000 nodes in a 40 A cube, 5 A cutoff (degree ~354)."""
     from e3nn_amd import o3
     from e3nn_amd.nn import DstSortedEdges
-    from tests import kernel_sets as ks
+    from e3nn_amd import kernel_sets as ks
 
     N, side, cutoff = 50_000, 40.0, 5.0
     pos, src, dst = radius_graph(N, side, cutoff)
@@ -277,7 +299,7 @@ def bench_convolution(args, dev, ctx):
     """One whole interaction block (reference e3nn/nn/models/v2106/points_convolution.py:99-113) on the headline
     graph: radial network 8 -> 64 -> 352, self-connection, lin1, fused message, lin2, alpha; 4 species."""
     from e3nn_amd.nn import DstSortedEdges
-    from tests import kernel_sets as ks
+    from e3nn_amd import kernel_sets as ks
 
     conv = ks.conv_wide().to(dev)
     N, E = ctx["N"], ctx["src"].shape[0]
@@ -388,7 +410,7 @@ def bench_nequip_backward(args, dev, ctx):
 def bench_uvw_backward(args, dev):
     """Dense uvw (fp32), forward + backward with respect to both inputs and the shared weights, and the
     weight-gradient kernel alone against the matrix-core peak."""
-    from tests import kernel_sets as ks
+    from e3nn_amd import kernel_sets as ks
 
     tp = ks.cfg5().to(dev)
     Z = 65536
@@ -468,6 +490,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": neq["ms"],
+        "ms_per_step_median": neq["ms_median"],
+        "ms_per_step_min": neq["ms_min"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -480,7 +504,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": neq["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": neq["achieved_gbs"] / HBM_PEAK_GBS, "traffic": NEQUIP_TRAFFIC_BYTES, "kernel": "e3x_uvu_fused",
+            "frac": neq["achieved_gbs"] / HBM_PEAK_GBS, "traffic": NEQUIP_TRAFFIC_BYTES.get(neq["kernel_key"]), "kernel": "e3x_uvu_fused",
             "algorithmic_bytes": neq["bytes_per_launch"],
         },
         "other": other,

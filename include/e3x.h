@@ -21,6 +21,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the library is built with hidden visibility: only what this header declares is exported */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
 
 #define E3X_OK 0
 #define E3X_ERR_INVALID (-1)     /* bad argument / unsupported instruction set */
@@ -304,6 +308,9 @@ int e3x_fc_backward_w(e3x_fc_plan* plan, const void* x, const void* grad_out, vo
  * for bandwidth counters (known traffic: n_bytes read + n_bytes written). */
 int e3x_copy_bytes(const void* src, void* dst, size_t n_bytes, void* stream);
 
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

@@ -1,292 +1,9 @@
-"""Every instruction set the GPU tests, the smoke check and the benchmark run.
-
-One place, so that the build step can compile all of their kernels into the in-tree
-cache before anything runs on a GPU.
-"""
-import json
+"""The package's instruction-set list with the golden cases of tests/golden switched on."""
 import os
 
-import torch
+from e3nn_amd import kernel_sets as _ks
 
-from e3nn_amd import o3
-from e3nn_amd.nn.message import message_tensor_product
+_ks.use_golden(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
 
-GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-
-SH2 = str(o3.Irreps.spherical_harmonics(2))
-SH3 = str(o3.Irreps.spherical_harmonics(3))
-
-GOLDEN_GPU_CASES = [
-    "fctp_cfg1", "fctp_small_cfg5_like", "fctp_per_sample_weights", "fctp_norm_path",
-    "uvu_merged_cfg3_like_mul4", "uvu_builder_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2",
-    "uvu_builderB_cfg4_like_mul2", "uvu_shared_v2", "uvu_mixed_weightless", "empty_path_and_missing_output",
-    "modes_uuu_uvuv_uuw_uvv", "modes_triangular", "conv_small",
-]  # fmt: skip
-
-
-def golden_meta():
-    with open(os.path.join(GOLDEN, "tp_cases.json")) as f:
-        return json.load(f)
-
-
-# backward pass in bf16 storage: a matrix-core uvw set, shared uvu weights, per-edge uvu weights
-BACKWARD_BF16_CASES = ["mfma_small", "uvu_shared_v2", "cfg3_merged"]
-
-
-def tp_from_meta(m, **extra):
-    upw = m.get("user_path_weights", [1.0] * len(m["instructions"]))
-    ins = [tuple(t[:5]) + (pw,) for t, pw in zip(m["instructions"], upw)]
-    kw = {}
-    if m.get("irrep_normalization"):
-        kw = dict(irrep_normalization=m["irrep_normalization"], path_normalization=m["path_normalization"])
-    return o3.TensorProduct(
-        m["irreps_in1"], m["irreps_in2"], m["irreps_out"], ins,
-        internal_weights=m["internal_weights"], shared_weights=m["shared_weights"], **kw, **extra,
-    )  # fmt: skip
-
-
-def golden_tp(name, meta=None, **extra):
-    m = dict((meta or golden_meta())[name])
-    if name == "fctp_norm_path":
-        m.update(irrep_normalization="norm", path_normalization="path")
-    return tp_from_meta(m, **extra)
-
-
-def cfg1():
-    return o3.FullyConnectedTensorProduct("16x0e+16x1o", "0e+1o+2e", "16x0e+16x1o+16x2e")
-
-
-def cfg3(merged=True):
-    f = "32x0e+32x1o+32x2e"
-    return message_tensor_product(f, SH2, irreps_out=f) if merged else message_tensor_product(f, SH2, keep="0e+1o+2e")
-
-
-def cfg4(variant="A"):
-    f = "128x0e+128x1o+128x2e+128x3o"
-    keep = "0e+1o+2e+3o" if variant == "A" else "0e+0o+1e+1o+2e+2o+3e+3o"
-    return message_tensor_product(f, SH3, keep=keep)
-
-
-def cfg5():
-    f = "128x0e+128x1o+128x2e"
-    return o3.FullyConnectedTensorProduct(f, f, f)
-
-
-def mfma_small():
-    # smallest shapes the matrix-core uvw kernel takes: multiplicities 32 / 64, three output irreps
-    return o3.FullyConnectedTensorProduct("64x0e+32x1o", "32x0e+32x1o+32x2e", "64x0e+64x1o+64x1e+64x2e")
-
-
-def node_fctp():
-    # node-wise step of a convolution: features x a few scalar node attributes (one-hot species), the GEMM K index is
-    # the feature multiplicity and the attribute index is a short outer loop (reference
-    # e3nn/nn/models/v2106/points_convolution.py:56-58)
-    return o3.FullyConnectedTensorProduct("128x0e+64x1o+32x2e", "4x0e", "128x0e+64x1o+96x2e")
-
-
-def node_wide_out():
-    # scalar second input with several 32-channel output tiles per irrep, l = 3 and a pseudoscalar attribute: the
-    # shape of an input gradient of a node-wise layer (few channels in, many out)
-    return o3.FullyConnectedTensorProduct("32x0e+32x1o+32x3o", "3x0e+2x0o", "96x0e+64x1o+64x1e+32x3o+32x3e")
-
-
-def node_narrow():
-    # scalar second input, channel counts that are not multiples of 4 (weight rows read float by float, a partly
-    # filled 32-channel tile) and multiplicities 8 / 24 / 40: the shape of the per-node mixing coefficient of a
-    # convolution (reference e3nn/nn/models/v2106/points_convolution.py:92-97) with two more irreps
-    return o3.FullyConnectedTensorProduct("96x0e+40x1o+8x2e", "4x0e", "1x0e+23x1o+9x2e")
-
-
-def node_partial_tile():
-    # channel counts that are multiples of 4 but not of 32: 16-byte weight pieces inside and outside the last tile
-    return o3.FullyConnectedTensorProduct("64x0e+16x1o", "3x0e", "48x0e+20x1o")
-
-
-def outer_split():
-    # 32-channel output tiles with several outer indices and a second input that is not scalar: the matrix-core
-    # kernel gives its second wave column every other outer index
-    return o3.FullyConnectedTensorProduct("64x0e+32x1o", "4x0e+2x1o", "32x1o+32x1e+32x2e")
-
-
-def wide_k():
-    # GEMM K extents above 128 (256 and 160): the K operand is resident in LDS in blocks of 128, restaged per outer index
-    return o3.FullyConnectedTensorProduct("256x0e+160x1o", "32x0e+32x1o", "64x0e+64x1o")
-
-
-def radial_layer():
-    # one dense layer of a radial network written as a tensor product of scalars: 64 -> 352 (= 5.5 tiles of 64
-    # channels: the last tile is half full), second input "0e"
-    return o3.FullyConnectedTensorProduct("64x0e", "0e", "352x0e")
-
-
-def mixed_modes(**extra):
-    # uvu and uvw paths into the same output irrep plus an elementwise and an unweighted path: the general kernel
-    ins = [(0, 0, 0, "uvu", True), (1, 1, 0, "uvw", True), (1, 0, 1, "uvu", False), (1, 1, 2, "uvv", True),
-           (0, 0, 3, "uuu", True), (1, 2, 4, "uuw", False)]  # fmt: skip
-    return o3.TensorProduct("4x0e+4x1o", "4x0e+3x1o+4x1e", "4x0e+4x1o+3x1e+4x0e+1x0o", ins, shared_weights=False, **extra)
-
-
-def scalar_exact():
-    # 1x1 Clebsch-Gordan, path weight 1: products and sums of small integers are exact in fp32
-    return message_tensor_product("32x0e", "0e", irreps_out="32x0e")
-
-
-def odd_mul():
-    # multiplicities that are no multiple of the lane-group width, several chunks
-    return message_tensor_product("80x0e+24x1o+5x2e", SH2, keep="0e+1o+2e")
-
-
-def all_tensor_products():
-    """(name, TensorProduct, dtypes) for everything that must be in the kernel cache."""
-    meta = golden_meta()
-    out = [(n, golden_tp(n, meta), (torch.float32,)) for n in GOLDEN_GPU_CASES]
-    out += [
-        ("cfg1", cfg1(), (torch.float32,)),
-        ("cfg3_merged", cfg3(True), (torch.float32, torch.bfloat16)),
-        ("cfg3_builder", cfg3(False), (torch.float32,)),
-        ("cfg4_A", cfg4("A"), (torch.float32, torch.bfloat16)),
-        ("cfg4_B", cfg4("B"), (torch.float32,)),
-        ("cfg5", cfg5(), (torch.float32, torch.bfloat16)),
-        ("mfma_small", mfma_small(), (torch.float32,)),
-        ("node_fctp", node_fctp(), (torch.float32,)),
-        ("radial_layer", radial_layer(), (torch.float32,)),
-        ("wide_k", wide_k(), (torch.float32,)),
-        ("outer_split", outer_split(), (torch.float32,)),
-        ("node_wide_out", node_wide_out(), (torch.float32,)),
-        ("node_narrow", node_narrow(), (torch.float32,)),
-        ("node_partial_tile", node_partial_tile(), (torch.float32,)),
-        ("mixed_modes", mixed_modes(), (torch.float32,)),
-        ("scalar_exact", scalar_exact(), (torch.float32,)),
-        ("odd_mul", odd_mul(), (torch.float32,)),
-    ]
-    return out
-
-
-# instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
-BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
-                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
-                  "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
-
-
-def nn_golden():
-    import numpy as np
-
-    with open(os.path.join(GOLDEN, "nn_cases.json")) as f:
-        meta = json.load(f)
-    return np.load(os.path.join(GOLDEN, "nn_cases.npz")), meta
-
-
-def nn_modules():
-    """(name, module) for the node-wise blocks the GPU tests run; every TensorProduct inside needs its kernels."""
-    from e3nn_amd import nn
-
-    _, meta = nn_golden()
-    out = []
-    for name in ("linear_mixed", "linear_path_norm", "linear_bias"):
-        m = meta[name]
-        out.append((name, o3.Linear(m["irreps_in"], m["irreps_out"], **m["kwargs"])))
-    out.append(("linear_wide", o3.Linear("128x0e+128x1o+64x2e", "128x0e+64x1o+32x1o")))
-    out.append(("fc_golden", nn.FullyConnectedNet(meta["fc"]["hs"], torch.nn.functional.silu)))
-    out.append(("fc_radial", nn.FullyConnectedNet([8, 64, 352], torch.nn.functional.silu)))
-    # a hidden layer too wide for the one-kernel path and its one-layer specialisations: tensor-product kernels throughout
-    out.append(("fc_wide_hidden", nn.FullyConnectedNet([8, 512, 16], torch.nn.functional.silu)))
-    a = meta["conv"]["args"]
-    out.append(("conv_golden", nn.Convolution(a[0], a[1], a[2], a[3], a[4], a[5])))
-    out.append(("conv_wide", conv_wide()))
-    return out
-
-
-# (hs, act, out_act, variance_in, variance_out) of the networks the one-kernel path is tested on: the radial network of
-# the benchmark block; three layers with a 96-wide output; widths that are multiples of nothing (scalar input loads,
-# zero-padded hidden layer, a partial last column tile); one layer with an output activation and variances; no activation
-FUSED_FC_CASES = [
-    ([8, 64, 352], "silu", False, 1, 1),
-    ([8, 64, 64, 96], "tanh", False, 1, 1),
-    ([5, 100, 50], "silu", False, 1, 1),
-    ([16, 40], "sigmoid", True, 2, 3),
-    ([12, 32, 32], None, False, 1, 2),
-    ([128, 128, 128, 8], "relu", True, 1, 1),
-]
-
-
-def fused_fc_nets():
-    from e3nn_amd import nn
-
-    torch.manual_seed(20240611)  # the weights are drawn at construction
-    return [nn.FullyConnectedNet(hs, act, variance_in=vi, variance_out=vo, out_act=oa) for hs, act, oa, vi, vo in FUSED_FC_CASES]
-
-
-def radial_message_cases():
-    """(name, all-uvu TensorProduct, two-layer radial network) for the message kernel with the network inside."""
-    from e3nn_amd import nn
-
-    torch.manual_seed(20240612)  # the weights are drawn at construction
-    tp = cfg3(merged=True)
-    small = o3.TensorProduct("32x0e+32x1o", "0e+1o", "32x0e+32x1o+32x1e", [(0, 0, 0, "uvu", True), (0, 1, 1, "uvu", True), (1, 0, 1, "uvu", True),
-                             (1, 1, 0, "uvu", True), (1, 1, 2, "uvu", True)], shared_weights=False, internal_weights=False)  # fmt: skip
-    return [
-        ("nequip_silu", tp, nn.FullyConnectedNet([8, 64, tp.weight_numel], torch.nn.functional.silu)),
-        ("small_tanh", small, nn.FullyConnectedNet([5, 32, small.weight_numel], torch.tanh, variance_in=2, variance_out=3)),
-        ("small_linear", small, nn.FullyConnectedNet([12, 16, small.weight_numel], None)),
-    ]
-
-
-def conv_wide():
-    # one interaction block at NequIP-like width: 32 channels per irrep, 4 species, 8 radial basis functions
-    from e3nn_amd import nn
-
-    f = "32x0e+32x1o+32x2e"
-    return nn.Convolution(f, "4x0e", SH2, f, [8, 64], 37.5)
-
-
-def prebuild(verbose=True, workers=6):
-    """Builds every kernel the tests and the benchmark use.  Plan creation spends its time in the HIP compiler (a child
-    process, the calling thread waits with the GIL released), so a few threads build several kernels at once."""
-    from concurrent.futures import ThreadPoolExecutor
-
-    from e3nn_amd import nn
-
-    jobs = []
-    for name, mod in nn_modules() + [(f"fused_fc{i}", net) for i, net in enumerate(fused_fc_nets())]:
-        for sub in mod.modules():
-            inner = sub.__dict__.get("_tp")  # Linear and the dense layers keep theirs out of the module tree
-            for tp in (sub, inner):
-                if isinstance(tp, o3.TensorProduct):
-                    jobs.append((f"module {name}", tp, (torch.float32,), True))
-            if isinstance(sub, nn.FullyConnectedNet):
-                jobs.append((f"module {name} (one kernel)", sub, None, False))
-    for name, tp, dtypes in all_tensor_products():
-        jobs.append((f"kernel {name}", tp, dtypes, name in BACKWARD_CASES))
-    for name, tp, net in radial_message_cases():
-        jobs.append((f"radial {name}", tp, net, False))
-    for name, mod in nn_modules():
-        if isinstance(mod, nn.Convolution):  # the block runs its radial network inside the message kernel when it can
-            jobs.append((f"radial {name}", mod.tp, mod.fc, False))
-
-    def build(job):
-        name, tp, dtypes, backward = job
-        if name.startswith("radial "):
-            plan = dtypes.fused_plan()  # the network on its own, which the tests run beside the fused kernel
-            return name, ["built" if tp.prepare_gather_scatter_radial(dtypes) else "(separate kernels)", plan.key or ""]
-        if dtypes is None:
-            plan = tp.fused_plan()
-            keys = [plan.key or "(layer by layer: " + plan.reason + ")"]
-            for layer in tp:
-                fwd, bwd = layer.dense_plans()
-                keys += [fwd.key, bwd.key] if fwd else ["(tensor-product kernels)"]
-            layers = list(tp)
-            for prev, layer in zip(layers, layers[1:]):  # input gradient through the activation in one kernel
-                pair = layer.act_dense_plans(prev) if prev.act is not None else None
-                keys += [pair[0].key, pair[1].key] if pair is not None else []
-            return name, keys
-        keys = [tp._plan(dt).key for dt in dtypes]
-        if backward:
-            tp.compile_backward(torch.float32)
-        if name.replace("kernel ", "") in BACKWARD_BF16_CASES:
-            tp.compile_backward(torch.bfloat16)
-        return name, keys
-
-    with ThreadPoolExecutor(max_workers=workers) as pool:
-        for name, keys in pool.map(build, jobs):
-            if verbose:
-                print(f"{name:40s} {' '.join(keys)}", flush=True)
+from e3nn_amd.kernel_sets import *  # noqa: E402,F401,F403
+from e3nn_amd.kernel_sets import GOLDEN_GPU_CASES, BACKWARD_CASES, BACKWARD_BF16_CASES, FUSED_FC_CASES, SH2, SH3  # noqa: E402,F401

@@ -26,6 +26,12 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(handle, name), f"{name} declared in e3x.h but not exported"
     assert declared == set(_lib._SIGNATURES), "ctypes signatures out of sync with e3x.h"
+    # ... and nothing else: internal C++ symbols stay inside the library
+    import subprocess
+
+    syms = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = {line.split()[-1] for line in syms.splitlines() if line.strip()}
+    assert exported == declared, sorted(exported ^ declared)
     assert _lib.lib().e3x_version() >= 100
 
 
