@@ -20,6 +20,7 @@ namespace {
 constexpr int kBlock = 256;
 
 __device__ int d_flag[4];  // range-check result of e3x_index_check (one copy per device)
+std::mutex g_flag_mutex;   // one check at a time: concurrent callers would share the flag
 
 // Sort buffers of e3x_csr_build_static.  Every device the library runs on holds its own copy of this array at its
 // own address for the life of the process; host code must use the address hipGetSymbolAddress reports for the
@@ -342,6 +343,8 @@ extern "C" int e3x_index_check(const void* idx, int idx_bits, int64_t E, int64_t
   if (E == 0) return E3X_OK;
   if (!idx) return e3x::fail(E3X_ERR_INVALID, "e3x_index_check: null pointer");
   hipStream_t st = (hipStream_t)stream;
+  // zero, launch and read-back form one critical section (it ends with a stream synchronisation anyway)
+  std::lock_guard<std::mutex> lock(g_flag_mutex);
   int* flag = nullptr;
   if (hipGetSymbolAddress((void**)&flag, HIP_SYMBOL(d_flag)) != hipSuccess)
     return e3x::fail(E3X_ERR_HIP, "e3x_index_check: hipGetSymbolAddress failed");

@@ -533,6 +533,21 @@ int build_uvw_node_source(e3x_plan& P, std::string* src) {
   return E3X_OK;
 }
 
+// The matrix-core weight-gradient kernel reads 8 multiplicity indices of the M operand and of the output gradient
+// with 16-byte loads: every irrep offset it starts from and both row lengths must be multiples of 4 floats.  Plans
+// that do not fit (an odd total dimension, an irrep of odd size in front of the operand) take the vector-ALU kernel.
+bool mfma_dw_fits(const e3x_plan& P) {
+  for (const auto& p : P.paths) {
+    const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2];
+    const bool okU = a.mul % 32 == 0 && a.mul <= k_cap(P.dtype), okV = b.mul % 32 == 0 && b.mul <= k_cap(P.dtype);
+    const bool m_is_x2 = okV && (!okU || b.l < a.l);
+    const int moff = m_is_x2 ? P.off2[p.in2] : P.off1[p.in1];
+    const int64_t mdim = m_is_x2 ? P.in2_dim : P.in1_dim;
+    if ((moff | P.offo[p.out] | mdim | P.out_dim) & 3) return false;
+  }
+  return true;
+}
+
 // Tables of the matrix-core weight-gradient kernel: per path the M operand is the input with the smaller l.
 
 int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
@@ -541,16 +556,8 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
   if (env_int("E3X_DW_ZC", 0)) s << "#define E3X_DW_ZC " << env_int("E3X_DW_ZC", 0) << "\n";
   int n_nz = 0, n_path = 0, dkmax = 1, drmax = 1;
   long long tiles = 0;
-  // the kernel reads 8 multiplicity indices of the M operand and of the output gradient with 16-byte loads
-  for (const auto& p : P.paths) {
-    const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2];
-    const bool okU = a.mul % 32 == 0 && a.mul <= k_cap(P.dtype), okV = b.mul % 32 == 0 && b.mul <= k_cap(P.dtype);
-    const bool m_is_x2 = okV && (!okU || b.l < a.l);
-    const int moff = m_is_x2 ? P.off2[p.in2] : P.off1[p.in1];
-    const int64_t mdim = m_is_x2 ? P.in2_dim : P.in1_dim;
-    if ((moff | P.offo[p.out] | mdim | P.out_dim) & 3)
-      return fail(E3X_ERR_INVALID, "weight gradient on the matrix cores: irrep offsets and row lengths must be multiples of 4");
-  }
+  if (!mfma_dw_fits(P))
+    return fail(E3X_ERR_INVALID, "weight gradient on the matrix cores: irrep offsets and row lengths must be multiples of 4");
   for (const auto& p : P.paths) {
     const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2], &c = P.out[p.out];
     const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1, d3 = 2 * c.l + 1;
@@ -620,9 +627,15 @@ int load_dw_function(e3x_plan* P, int dev) {
   return E3X_OK;
 }
 
-// A uvw_node plan that the matrix-core gradient kernel does not take (multiplicities that are not multiples of 32)
-// gets its weight gradient from the vector-ALU family: that code object is built on first use.
-bool node_dw_on_valu(const e3x_plan* P) { return P->family == "uvw_node" && !uvw_mfma_eligible(*P); }
+// A uvw_node or uvw_mfma plan that the matrix-core gradient kernel does not take (multiplicities that are not
+// multiples of 32, operands that are not 16-byte aligned within their rows) gets its weight gradient from the
+// vector-ALU family: that code object is built on first use.  Decided from the plan alone, so that
+// e3x_tp_plan_prepare_backward_w and e3x_tp_backward_w_uvw agree.
+bool node_dw_on_valu(const e3x_plan* P) {
+  if (P->family == "uvw_node") return !uvw_mfma_eligible(*P) || !mfma_dw_fits(*P);
+  if (P->family == "uvw_mfma") return !mfma_dw_fits(*P);
+  return false;
+}
 
 int prepare_valu_dw(e3x_plan* P) {
   std::lock_guard<std::mutex> lock(P->mu);
@@ -1183,6 +1196,10 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
 
 extern "C" int e3x_tp_plan_prepare_backward_w(e3x_plan* P) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: null plan");
+  if (P->family == "uvw_small")
+    for (const auto& q : P->paths)
+      if (q.mode != E3X_MODE_UVW)
+        return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: no weight-gradient kernel for connection modes other than uvu / uvw");
   if (node_dw_on_valu(P)) return prepare_valu_dw(P);
   if (P->family == "uvw_mfma" || P->family == "uvw_node") {
     if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_backward_w: fp32 storage only");
@@ -1197,6 +1214,9 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null plan");
   if (P->family != "uvw_small" && P->family != "uvw_mfma" && P->family != "uvw_node")
     return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: the plan must be all-uvw");
+  // the general vector-ALU family also holds the other connection modes, whose weight blocks are not [U, V, W]
+  for (const auto& q : P->paths)
+    if (q.mode != E3X_MODE_UVW) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: the plan must be all-uvw");
   if (P->dtype != E3X_F32) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: fp32 storage only");
   if (Z < 0) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: negative batch");
   if (P->weight_numel == 0) return E3X_OK;
@@ -1205,7 +1225,7 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
   int dev, rc;
   if ((rc = current_device(&dev))) return rc;
   // the node-wise family has no gradient kernel of its own: the matrix-core one where its tiling fits, else the vector-ALU one
-  const bool mfma = P->family == "uvw_mfma" || (P->family == "uvw_node" && !node_dw_on_valu(P));
+  const bool mfma = (P->family == "uvw_mfma" || P->family == "uvw_node") && !node_dw_on_valu(P);
   if (Z == 0) return P->shared_weights ? e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st) : E3X_OK;
   if (!grad_out || (P->in1_dim && !x1) || (P->in2_dim && !x2)) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_uvw: null pointer");
   long long n_rows = Z;

@@ -126,6 +126,17 @@ def wide_k():
     return o3.FullyConnectedTensorProduct("256x0e+160x1o", "32x0e+32x1o", "64x0e+64x1o")
 
 
+def unaligned_mfma():
+    # matrix-core forward, but an irrep no output reaches (3x2e) makes the input row 175 floats long: the matrix-core
+    # weight-gradient kernel needs 16-byte aligned operands within a row, so the gradient runs on the vector-ALU kernel
+    return o3.FullyConnectedTensorProduct("64x0e+32x1o+3x2e", "0e", "64x0e+32x1o")
+
+
+def unaligned_offsets():
+    # a 5-float irrep in front of the tiled one: operand offset 5
+    return o3.FullyConnectedTensorProduct("1x2e+32x0e", "0e", "32x0e")
+
+
 def radial_layer():
     # one dense layer of a radial network written as a tensor product of scalars: 64 -> 352 (= 5.5 tiles of 64
     # channels: the last tile is half full), second input "0e"
@@ -170,6 +181,8 @@ def all_tensor_products():
         ("node_wide_out", node_wide_out(), (torch.float32,)),
         ("node_narrow", node_narrow(), (torch.float32,)),
         ("node_partial_tile", node_partial_tile(), (torch.float32,)),
+        ("unaligned_mfma", unaligned_mfma(), (torch.float32,)),
+        ("unaligned_offsets", unaligned_offsets(), (torch.float32,)),
         ("mixed_modes", mixed_modes(), (torch.float32,)),
         ("scalar_exact", scalar_exact(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),
@@ -180,7 +193,7 @@ def all_tensor_products():
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
                   "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
-                  "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
+                  "unaligned_mfma", "unaligned_offsets", "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
 
 
 def nn_golden():

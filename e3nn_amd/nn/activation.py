@@ -7,6 +7,7 @@ import ctypes
 from typing import List
 
 import torch
+from torch.autograd.function import once_differentiable
 
 from .. import _lib
 from ..o3.irreps import Irrep, Irreps
@@ -97,6 +98,7 @@ class _GateFn(torch.autograd.Function):
         return mod._launch(x, None)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, g):
         (x,) = ctx.saved_tensors
         return ctx.mod._launch(x, g.contiguous()), None

@@ -32,7 +32,10 @@ class DstSortedEdges:
         """The same edges with source and destination exchanged (grouped by ``edge_src``); the backward
         pass with respect to the node features scatters onto the sources.  Built once, cached."""
         if self._transposed is None:
-            self._transposed = DstSortedEdges(self.edge_dst, self.edge_src, self.num_src_nodes, self.num_nodes, self._locality_order)
+            # the sources become scatter destinations, which do not wrap: negative source indices (valid for the
+            # gather, like torch advanced indexing) are normalised first
+            src = torch.where(self.edge_src < 0, self.edge_src + self.num_src_nodes, self.edge_src)
+            self._transposed = DstSortedEdges(self.edge_dst, src, self.num_src_nodes, self.num_nodes, self._locality_order)
             self._transposed._transposed = self
         return self._transposed
 

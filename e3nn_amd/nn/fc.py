@@ -13,6 +13,7 @@ Two device paths, both HIP kernels of this package:
 import ctypes
 
 import torch
+from torch.autograd.function import once_differentiable
 
 from .. import _lib
 from ..o3.tensor_product import TensorProduct
@@ -29,6 +30,7 @@ class _DenseFn(torch.autograd.Function):
         return layer._fwd.forward(x, [w.contiguous()])
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, g):
         x, w = ctx.saved_tensors
         layer = ctx.layer
@@ -63,6 +65,7 @@ class _ActDenseFn(torch.autograd.Function):
         return ctx.plans[0].forward(z, [w.contiguous()])
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, g):
         z, w = ctx.saved_tensors
         fwd, bwd = ctx.plans

@@ -7,6 +7,7 @@ import ctypes
 from typing import Any, List, Union
 
 import torch
+from torch.autograd.function import once_differentiable
 
 from .. import _lib
 from .irreps import Irreps
@@ -39,6 +40,7 @@ class _SphericalHarmonicsFn(torch.autograd.Function):
         return out.reshape(batch + (n_out,))
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, g):
         (xyz,) = ctx.saved_tensors
         ls, normalize, normalization, batch = ctx.cfg

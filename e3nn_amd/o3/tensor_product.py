@@ -19,6 +19,7 @@ from math import prod, sqrt
 from typing import List, Optional, Union
 
 import torch
+from torch.autograd.function import once_differentiable
 
 from .. import _lib, get_optimization_defaults
 from .irreps import Irreps
@@ -198,6 +199,7 @@ class _TensorProductFn(torch.autograd.Function):
         return tp._plan(x1.dtype).forward(x1, x2, w)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, g):
         tp = ctx.tp
         x1, x2, w = ctx.saved_tensors
@@ -248,6 +250,7 @@ class _GatherScatterFn(torch.autograd.Function):
         return tp._plan(node_x.dtype).gather_scatter(node_x, edge_attr, w, edges.edge_src, edges, node_x.shape[0])
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, g):
         tp, edges = ctx.tp, ctx.edges
         node_x, edge_attr, w = ctx.saved_tensors

@@ -32,3 +32,23 @@ def golden_tp():
         meta = json.load(f)
     arrays = dict(np.load(os.path.join(GOLDEN, "tp_cases.npz")))
     return meta, arrays
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Raw error figures of every comparison against the oracle made in this session (max abs, max relative),
+    beside the pass / fail of the tolerance checks; also written to gpurun_out/parity_errors.json when that
+    directory exists."""
+    from tests.helpers import ERROR_LOG
+
+    if not ERROR_LOG:
+        return
+    tr = terminalreporter
+    tr.section("raw errors against the oracle")
+    tr.write_line(f"{'comparison':60s} {'n':>9s} {'max|err|':>10s} {'max|ref|':>10s} {'max rel':>10s} {'err/tol':>8s}")
+    for r in ERROR_LOG:
+        tr.write_line(f"{r['what'][:60]:60s} {r['n']:9d} {r['max_abs_err']:10.3e} {r['max_abs_ref']:10.3e} "
+                      f"{r['max_rel_err']:10.3e} {r['worst_err_over_tol']:8.3f}")  # fmt: skip
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "parity_errors.json"), "w") as f:
+            json.dump(ERROR_LOG, f, indent=1)

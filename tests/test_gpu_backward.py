@@ -69,6 +69,20 @@ def test_fused_message_gradients(maker, N, E, idx):
     a2, c2 = node_x.to(DEV).requires_grad_(True), w.to(DEV)
     tp.forward_gather_scatter(a2, attr.to(DEV), c2, edges=edges).backward(cot.to(DEV))
     assert torch.equal(a2.grad, a.grad)
+    # negative source indices wrap in the gather; the gradient scatters onto the wrapped rows
+    neg = torch.where(torch.arange(E) % 3 == 0, src - N, src)
+    a3 = node_x.to(DEV).requires_grad_(True)
+    tp.forward_gather_scatter(a3, attr.to(DEV), c2, edges=DstSortedEdges(neg.to(idx).to(DEV), dst.to(idx).to(DEV), N)).backward(cot.to(DEV))
+    assert torch.equal(a3.grad, a.grad)
+
+
+def test_second_derivatives_raise_instead_of_dropping_terms():
+    # the backward passes are kernels on fresh buffers (no graph): double backward must fail loudly
+    tp = ks.cfg1().to(DEV)
+    x1, x2 = seeded(8, 64).to(DEV).requires_grad_(True), seeded(8, 9).to(DEV)
+    (g,) = torch.autograd.grad(tp(x1, x2).square().sum(), x1, create_graph=True)
+    with pytest.raises(RuntimeError, match="once_differentiable"):
+        g.sum().backward()
 
 
 @pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.mfma_small, 70),
@@ -92,7 +106,7 @@ def test_uvw_input_gradients(maker, Z):
 @pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.cfg1, 4099),
                                      (lambda: ks.golden_tp("fctp_per_sample_weights"), 5), (ks.mfma_small, 70),
                                      (ks.mfma_small, 1500), (ks.node_fctp, 700), (ks.radial_layer, 513), (ks.node_wide_out, 300), (ks.node_narrow, 260),
-                                     (ks.node_partial_tile, 100)])  # fmt: skip
+                                     (ks.node_partial_tile, 100), (ks.unaligned_mfma, 300), (ks.unaligned_offsets, 129)])  # fmt: skip
 def test_uvw_weight_gradients(maker, Z):
     tp = maker().to(DEV)
     spec = oracle_spec(tp)

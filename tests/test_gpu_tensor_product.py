@@ -210,16 +210,57 @@ def test_uvw_full_size_dense_configuration():
     assert torch.equal(tp(x1[1000:1100], x2[1000:1100]), out[1000:1100])
 
 
-def test_uvw_bf16_storage():
+def _bf16_uvw(seed_w=0):
     tp = ks.cfg5().to(DEV)
-    w = _fan_in_weights(tp)
-    Z = 40
-    x1, x2 = seeded(Z, 1152, seed=31), seeded(Z, 1152, seed=32)
+    w = _fan_in_weights(tp, seed=seed_w)
     tpb = ks.cfg5().to(DEV).to(torch.bfloat16)
     with torch.no_grad():
         tpb.weight.copy_(w.to(torch.bfloat16))
+    return tp, tpb, tpb.weight.detach().float().cpu().numpy()
+
+
+def _oracle_chunks(spec, x1, x2, w, chunk=48):
+    return np.concatenate([otp.tp_forward(spec, x1[b : b + chunk], x2[b : b + chunk], w) for b in range(0, x1.shape[0], chunk)])
+
+
+def test_uvw_bf16_storage():
+    # two full 128-row workgroup tiles and a ragged tail of 77 rows; outputs have standard deviation 1/128, so the
+    # tolerance is tied to the output scale: atol = 1e-2 max|ref| (a dropped path of the 11 shifts outputs by ~0.5 sigma,
+    # ten times this), rtol 1e-2 for the single bf16 rounding of the output
+    tp, tpb, wq = _bf16_uvw()
+    Z = 333
+    x1, x2 = seeded(Z, 1152, seed=31), seeded(Z, 1152, seed=32)
     xb, yb = x1.to(DEV).to(torch.bfloat16), x2.to(DEV).to(torch.bfloat16)
     out = tpb(xb, yb)
     assert out.dtype == torch.bfloat16
-    ref = otp.tp_forward(oracle_spec(tp), xb.float().cpu().numpy(), yb.float().cpu().numpy(), tpb.weight.detach().float().cpu().numpy())
-    assert_close(out, ref, atol=2e-2, rtol=1e-2, what="bf16 uvw")
+    ref = _oracle_chunks(oracle_spec(tp), xb.float().cpu().numpy(), yb.float().cpu().numpy(), wq)
+    scale = float(np.abs(ref).max())
+    assert 0.02 < scale < 0.08
+    assert_close(out, ref, atol=1e-2 * scale, rtol=1e-2, what="bf16 uvw, Z = 333")
+    # every path matters at this tolerance: the oracle without the last instruction fails it
+    spec = oracle_spec(tp)
+    short = otp.make_spec(str(tp.irreps_in1), str(tp.irreps_in2), str(tp.irreps_out),
+                          [(t.i_in1, t.i_in2, t.i_out, t.connection_mode, t.has_weight, 0.0 if n == 10 else 1.0) for n, t in enumerate(tp.instructions)],
+                          shared_weights=True)  # fmt: skip
+    assert len(spec.instructions) == 11
+    miss = _oracle_chunks(short, xb[:48].float().cpu().numpy(), yb[:48].float().cpu().numpy(), wq)
+    assert (np.abs(out[:48].detach().float().cpu().numpy() - miss) > 1e-2 * scale + 1e-2 * np.abs(miss)).any()
+
+
+def test_uvw_bf16_storage_full_size():
+    # batch 65536: rows from both ends, tile boundaries and the middle against the oracle; slices give the same rows
+    tp, tpb, wq = _bf16_uvw()
+    Z = 65536
+    g = torch.Generator(device=DEV).manual_seed(0)
+    xb = torch.randn(Z, 1152, device=DEV, generator=g).to(torch.bfloat16)
+    yb = torch.randn(Z, 1152, device=DEV, generator=g).to(torch.bfloat16)
+    out = tpb(xb, yb)
+    rows = torch.tensor([0, 127, 128, 32767, 32768, 40001, 65408, 65535])
+    ref = otp.tp_forward(oracle_spec(tp), xb[rows].float().cpu().numpy(), yb[rows].float().cpu().numpy(), wq)
+    scale = float(np.abs(ref).max())
+    assert_close(out[rows], ref, atol=1e-2 * scale, rtol=1e-2, what="bf16 uvw, 8 rows of Z = 65536")
+    # a batch slice gives the same rows up to the accumulation order (workgroups start at different outer-index
+    # blocks depending on their position in the grid): within one bf16 rounding step of the output
+    part = tpb(xb[4096 : 4096 + 256], yb[4096 : 4096 + 256]).float()
+    assert (part - out[4096 : 4096 + 256].float()).abs().max().item() <= 2.0**-7 * scale
+    assert abs(out.float().var().item() * 16384 - 1.0) < 0.1

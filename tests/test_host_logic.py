@@ -303,3 +303,26 @@ def test_radial_message_kernel_is_offered_only_for_what_it_takes():
     assert not other.prepare_gather_scatter_radial(nn.FullyConnectedNet([8, 16, other.weight_numel], torch.tanh))
     shared = ks.golden_tp("uvu_shared_v2")  # shared weights: nothing per edge to compute
     assert shared._radial_description(nn.FullyConnectedNet([8, 16, shared.weight_numel], torch.tanh)) is None
+
+
+def test_weight_gradient_of_matrix_core_plans_with_unaligned_rows_builds():
+    # legal reference configurations whose rows are not multiples of 4 floats (an irrep no output reaches, an odd
+    # total dimension): forward on the matrix cores, weight gradient on the vector-ALU kernel, decided at plan level
+    for tp in (ks.unaligned_mfma(), ks.unaligned_offsets(), o3.FullyConnectedTensorProduct("32x0e+1x1o", "0e", "32x0e")):
+        plan = tp._plan(torch.float32)
+        assert plan.family in ("uvw_mfma", "uvw_node")
+        tp.compile_backward()
+        assert _lib.lib().e3x_tp_plan_prepare_backward_w(plan.handle) == 0
+    lin = o3.Linear("1x2e+32x0e", "32x0e")
+    lin._tp.compile_backward()
+
+
+def test_weight_gradient_entry_point_rejects_other_connection_modes():
+    tp = ks.mixed_modes()
+    plan = tp._plan(torch.float32)
+    assert plan.family == "uvw_small"
+    L = _lib.lib()
+    assert L.e3x_tp_plan_prepare_backward_w(plan.handle) == _lib.ERR_INVALID
+    one = ctypes.c_void_p(16)  # never dereferenced: the mode check comes first
+    assert L.e3x_tp_backward_w_uvw(plan.handle, one, one, one, one, 4, None) == _lib.ERR_INVALID
+    assert b"all-uvw" in L.e3x_last_error()

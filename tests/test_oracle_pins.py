@@ -268,6 +268,89 @@ def test_conv_matches_reference_golden(golden_tp):
     assert not out[-1].any()
 
 
+# ---------------------------------------------------------------- torch-CPU restatement (timed baseline, backward oracle)
+TORCH_CASES = [  # every golden case whose instructions are all weighted uvu / uvw, the modes the restatement covers
+    "fctp_cfg1", "fctp_small_cfg5_like", "fctp_per_sample_weights", "fctp_norm_path", "uvu_merged_cfg3_like_mul4",
+    "uvu_builder_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_builderB_cfg4_like_mul2", "uvu_shared_v2",
+]  # fmt: skip
+
+
+@pytest.mark.parametrize("name", TORCH_CASES)
+def test_torch_restatement_matches_reference_golden(golden_tp, name):
+    import torch
+
+    from oracle.torch_cpu import tp_forward_torch
+
+    meta, arr = golden_tp
+    kw = dict(irrep_normalization="norm", path_normalization="path") if name == "fctp_norm_path" else {}
+    spec = spec_from_meta(meta[name], **kw)
+    x1, x2, w = (torch.from_numpy(arr[f"{name}/{k}"]) for k in ("x1", "x2", "w"))
+    assert x1.dtype == torch.float64
+    out = tp_forward_torch(spec, x1, x2, w).numpy()
+    assert out.shape == arr[name + "/out"].shape
+    np.testing.assert_allclose(out, arr[name + "/out"], atol=1e-12, rtol=1e-12)
+
+
+def test_torch_restatement_matches_numpy_oracle_on_the_benchmark_sets():
+    # the instruction sets of the benchmark at reduced multiplicity, all five l-specialisations of the einsum strings
+    import torch
+
+    from oracle.torch_cpu import tp_forward_torch
+
+    rng = np.random.default_rng(3)
+    sh3 = "0e+1o+2e+3o"
+    mid, ins = otp.convolution_instructions("6x0e+6x1o+6x2e+6x3o", sh3, lambda l, p: p == (-1) ** l and l <= 3)
+    uvu = otp.make_spec("6x0e+6x1o+6x2e+6x3o", sh3, ir_.to_str(mid), ins, shared_weights=False)
+    assert len(ins) == 23
+    f = "5x0e+5x1o+5x2e"
+    uvw = otp.make_spec(f, f, f, otp.fully_connected_instructions(f, f, f), shared_weights=True)
+    for spec in (uvu, uvw):
+        Z = 7
+        x1 = rng.standard_normal((Z, ir_.dim(spec.irreps_in1)))
+        x2 = rng.standard_normal((Z, ir_.dim(spec.irreps_in2)))
+        w = rng.standard_normal((spec.weight_numel,) if spec.shared_weights else (Z, spec.weight_numel))
+        ref = otp.tp_forward(spec, x1, x2, w)
+        got = tp_forward_torch(spec, torch.from_numpy(x1), torch.from_numpy(x2), torch.from_numpy(w)).numpy()
+        np.testing.assert_allclose(got, ref, atol=1e-12, rtol=1e-12)
+        assert np.abs(ref).max() > 0.5  # not a comparison of zeros
+
+
+def test_torch_gather_scatter_matches_reference_golden(golden_tp):
+    import torch
+
+    from oracle.torch_cpu import scatter_torch, tp_gather_scatter_torch
+
+    meta, arr = golden_tp
+    spec = spec_from_meta(meta["conv_small"])
+    g = {k.split("/")[1]: v for k, v in arr.items() if k.startswith("conv_small/")}
+    t = {k: torch.from_numpy(v) for k, v in g.items()}
+    N = g["node_x"].shape[0]
+    out = tp_gather_scatter_torch(spec, t["node_x"], t["attr"], t["w"], t["src"].long(), t["dst"].long(), N).numpy()
+    np.testing.assert_allclose(out, g["out"], atol=1e-12)
+    # int32 destinations are widened; integer payloads sum exactly
+    msg = torch.arange(40, dtype=torch.float64).reshape(10, 4)
+    dst = torch.tensor([3, 0, 3, 1, 0, 0, 4, 3, 1, 0], dtype=torch.int32)
+    ref = np.zeros((6, 4))
+    np.add.at(ref, dst.numpy(), msg.numpy())
+    assert (scatter_torch(msg, dst.long(), 6).numpy() == ref).all()
+
+
+def test_torch_spherical_harmonics_match_reference_golden(golden_sh):
+    import torch
+
+    from oracle.torch_cpu import spherical_harmonics_torch
+
+    pts = torch.from_numpy(golden_sh["points"])
+    for lmax in (1, 2, 3):
+        n = (lmax + 1) ** 2
+        for normalize in (True, False):
+            ref = golden_sh[f"lmax8_{int(normalize)}_component"][:, :n]
+            got = spherical_harmonics_torch(lmax, pts, normalize).numpy()
+            assert (np.abs(got - ref) / np.maximum(1.0, np.abs(ref))).max() < 1e-12
+    zero = spherical_harmonics_torch(3, torch.zeros(2, 3, dtype=torch.float64), True).numpy()
+    assert (zero[:, 0] == 1).all() and not zero[:, 1:].any()  # reference _spherical_harmonics.py:96
+
+
 # ---------------------------------------------------------------- rotations (equivariance tooling)
 def test_wigner_D_is_a_representation_and_w3j_is_invariant():
     from oracle.rotation import irreps_D, random_rotation, wigner_D
