@@ -13,6 +13,7 @@ from ..o3.irreps import Irrep, Irreps
 from ..o3.tensor_product import FullyConnectedTensorProduct, TensorProduct
 from .edges import DstSortedEdges
 from .fc import FullyConnectedNet
+from .message import message_instructions
 
 
 class Convolution(torch.nn.Module):
@@ -23,42 +24,34 @@ class Convolution(torch.nn.Module):
         self, irreps_node_input, irreps_node_attr, irreps_edge_attr, irreps_node_output, fc_neurons, num_neighbors
     ) -> None:
         super().__init__()
-        self.irreps_node_input = Irreps(irreps_node_input)
-        self.irreps_node_attr = Irreps(irreps_node_attr)
-        self.irreps_edge_attr = Irreps(irreps_edge_attr)
-        self.irreps_node_output = Irreps(irreps_node_output)
+        self.irreps_node_input, self.irreps_node_attr = Irreps(irreps_node_input), Irreps(irreps_node_attr)
+        self.irreps_edge_attr, self.irreps_node_output = Irreps(irreps_edge_attr), Irreps(irreps_node_output)
         self.num_neighbors = num_neighbors
 
-        self.sc = FullyConnectedTensorProduct(self.irreps_node_input, self.irreps_node_attr, self.irreps_node_output)
-        self.lin1 = FullyConnectedTensorProduct(self.irreps_node_input, self.irreps_node_attr, self.irreps_node_input)
+        def node_wise(features, out):  # features (x) node attributes -> out, shared weights
+            return FullyConnectedTensorProduct(features, self.irreps_node_attr, out)
 
-        irreps_mid, instructions = [], []
-        for i, (mul, ir_in) in enumerate(self.irreps_node_input):
-            for j, (_, ir_edge) in enumerate(self.irreps_edge_attr):
-                for ir_out in ir_in * ir_edge:
-                    if ir_out in self.irreps_node_output or ir_out == Irrep(0, 1):
-                        k = len(irreps_mid)
-                        irreps_mid.append((mul, ir_out))
-                        instructions.append((i, j, k, "uvu", True))
-        irreps_mid = Irreps(irreps_mid)
-        irreps_mid, p, _ = irreps_mid.sort()
-        assert irreps_mid.dim > 0, (
-            f"irreps_node_input={self.irreps_node_input} time irreps_edge_attr={self.irreps_edge_attr} produces nothing "
-            f"in irreps_node_output={self.irreps_node_output}"
-        )
-        instructions = [(i_1, i_2, p[i_out], mode, train) for i_1, i_2, i_out, mode, train in instructions]
-        tp = TensorProduct(
+        # messages carry every irrep the output asks for, plus scalars for the per-node mixing coefficient `alpha`
+        wanted = {ir for _, ir in self.irreps_node_output} | {Irrep(0, 1)}
+        irreps_mid, instructions = message_instructions(self.irreps_node_input, self.irreps_edge_attr, wanted)
+        if irreps_mid.dim == 0:
+            raise AssertionError(
+                f"no product of an input irrep ({self.irreps_node_input}) with an edge irrep ({self.irreps_edge_attr}) "
+                f"lies in the output irreps ({self.irreps_node_output}): there is no message to send"
+            )
+        # submodules in the reference's registration order (state_dict keys and the random stream of the initial weights)
+        self.sc = node_wise(self.irreps_node_input, self.irreps_node_output)
+        self.lin1 = node_wise(self.irreps_node_input, self.irreps_node_input)
+        message = TensorProduct(
             self.irreps_node_input, self.irreps_edge_attr, irreps_mid, instructions, internal_weights=False, shared_weights=False
         )
-        self.fc = FullyConnectedNet(list(fc_neurons) + [tp.weight_numel], torch.nn.functional.silu)
-        self.tp = tp
-        self.lin2 = FullyConnectedTensorProduct(irreps_mid, self.irreps_node_attr, self.irreps_node_output)
-        self.alpha = FullyConnectedTensorProduct(irreps_mid, self.irreps_node_attr, "0e")
-        with torch.no_grad():
-            self.alpha.weight.zero_()
-        assert (
-            self.alpha.output_mask[0] == 1.0
-        ), f"irreps_mid={irreps_mid} and irreps_node_attr={self.irreps_node_attr} are not able to generate scalars"
+        self.fc = FullyConnectedNet([*fc_neurons, message.weight_numel], torch.nn.functional.silu)
+        self.tp = message
+        self.lin2 = node_wise(irreps_mid, self.irreps_node_output)
+        self.alpha = node_wise(irreps_mid, "0e")
+        torch.nn.init.zeros_(self.alpha.weight)  # the block starts as its self-connection
+        if self.alpha.output_mask[0] != 1.0:
+            raise AssertionError(f"the messages ({irreps_mid}) and the node attributes ({self.irreps_node_attr}) cannot produce a scalar for alpha")
 
     def forward(self, node_input, node_attr, edge_src, edge_dst, edge_attr, edge_scalars, edges=None) -> torch.Tensor:
         node_self_connection = self.sc(node_input, node_attr)

@@ -6,24 +6,24 @@
 blocks sorted by irrep.  ``merged_instructions`` instead sums all paths with the same
 output irrep into one block of a given ``irreps_out``.
 """
+import itertools
+
 from ..o3.irreps import Irrep, Irreps
 from ..o3.tensor_product import TensorProduct
 
 
 def message_instructions(irreps_node_input, irreps_edge_attr, keep):
-    """Returns ``(irreps_mid, instructions)``; ``keep`` is an Irreps / list of irreps to retain."""
-    irreps_node_input, irreps_edge_attr = Irreps(irreps_node_input), Irreps(irreps_edge_attr)
-    keep = {ir for _, ir in Irreps(keep)} if not callable(keep) else keep
-    wanted = keep if callable(keep) else (lambda ir: ir in keep)
-    mid, ins = [], []
-    for i, (mul, ir_in) in enumerate(irreps_node_input):
-        for j, (_, ir_edge) in enumerate(irreps_edge_attr):
-            for ir_out in ir_in * ir_edge:
-                if wanted(ir_out):
-                    ins.append((i, j, len(mid), "uvu", True))
-                    mid.append((mul, ir_out))
-    mid, p, _ = Irreps(mid).sort()
-    return mid, [(a, b, p[c], mode, train) for a, b, c, mode, train in ins]
+    """Returns ``(irreps_mid, instructions)``; ``keep`` is an Irreps, a collection of irreps or a predicate on an irrep."""
+    nodes, edges = Irreps(irreps_node_input), Irreps(irreps_edge_attr)
+    if callable(keep):
+        wanted = keep
+    else:
+        kept = {Irrep(ir) for ir in (Irreps(keep) if isinstance(keep, str) else keep)}
+        wanted = kept.__contains__
+    # one path per (node irrep, edge irrep, allowed product irrep), in that nesting; path n writes output block n
+    paths = [(i, j, mul, ir) for (i, (mul, a)), (j, (_, b)) in itertools.product(enumerate(nodes), enumerate(edges)) for ir in a * b if wanted(ir)]
+    blocks, position, _ = Irreps([(mul, ir) for _, _, mul, ir in paths]).sort()  # ... then the blocks are sorted by irrep
+    return blocks, [(i, j, position[n], "uvu", True) for n, (i, j, _, _) in enumerate(paths)]
 
 
 def merged_instructions(irreps_node_input, irreps_edge_attr, irreps_out):

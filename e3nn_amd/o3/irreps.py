@@ -1,125 +1,137 @@
 """Irreducible representations of O(3) and direct sums of them.
 
-Same public behaviour as the reference's ``e3nn.o3.Irrep`` / ``e3nn.o3.Irreps``
+Public behaviour of the reference's ``e3nn.o3.Irrep`` / ``e3nn.o3.Irreps``
 (e3nn/o3/_irreps.py:14-264, :301-806) for everything the tensor-product hot path
-needs: parsing, layout (``dim``, ``slices``), the selection rule ``ir1 * ir2``,
-``sort`` / ``simplify`` / ``regroup`` / ``filter`` and ``randn``.  The rotation-matrix
-constructors (``D_from_*``) are not part of the hot path and are not provided.
+needs: the string grammar, the feature layout (``dim``, ``slices``), the selection rule
+``ir1 * ir2``, ``sort`` / ``simplify`` / ``regroup`` / ``filter`` and ``randn``.  The
+rotation-matrix constructors (``D_from_*``) are not part of the hot path and are not provided.
+
+Grammar:  irreps := term ("+" term)* | ""      term := [mul "x"] irrep      irrep := l ("e" | "o" | "y")
+where "y" is the parity of the spherical harmonics, (-1)^l.
 """
-import collections
 import itertools
+import re
+from collections import namedtuple
 from typing import List, Union
 
 import torch
 
+_IRREP_NAME = re.compile(r"\s*(\d+)\s*([eoy])\s*")
+_TERM = re.compile(r"\s*(?:(\d+)\s*x)?\s*(\d+\s*[eoy])\s*")
+_SortResult = namedtuple("sort", ["irreps", "p", "inv"])
+
+
+def _parse_irrep_name(text: str):
+    m = _IRREP_NAME.fullmatch(text)
+    if m is None:
+        raise ValueError(f'unable to convert string "{text.strip()}" into an Irrep')
+    degree = int(m.group(1))
+    parity = {"e": 1, "o": -1, "y": -1 if degree % 2 else 1}[m.group(2)]
+    return degree, parity
+
+
+def _not_a_sequence(self, *_args):
+    # Irrep and (mul, irrep) pairs are tuples only for hashing, ordering and unpacking
+    raise NotImplementedError
+
 
 class Irrep(tuple):
-    """Irreducible representation ``(l, p)``; ``Irrep("1o")``, ``Irrep(2, 1)``, ``Irrep("3y")``."""
+    """Irreducible representation ``(l, p)``; ``Irrep("1o")``, ``Irrep(2, 1)``, ``Irrep("3y")``.
+
+    Ordered as the pair ``(l, p)``: at equal ``l`` the odd irrep comes first."""
 
     def __new__(cls, l, p=None):
-        if p is None:
-            if isinstance(l, Irrep):
+        if p is None:  # one argument: an Irrep, a (mul, irrep) pair of an Irreps, a name, or an (l, p) pair
+            if type(l) is Irrep:
                 return l
-            if isinstance(l, _MulIr):
-                return l.ir
-            if isinstance(l, str):
-                name = l.strip()
-                try:
-                    deg = int(name[:-1])
-                    if deg < 0:
-                        raise ValueError
-                    p = {"e": 1, "o": -1, "y": (-1) ** deg}[name[-1]]
-                    l = deg
-                except Exception:
-                    raise ValueError(f'unable to convert string "{name}" into an Irrep')
-            elif isinstance(l, tuple):
-                l, p = l
-        if not isinstance(l, int) or l < 0:
-            raise ValueError(f"l must be positive integer, got {l}")
-        if p not in (-1, 1):
-            raise ValueError(f"parity must be on of (-1, 1), got {p}")
-        return super().__new__(cls, (l, p))
+            if type(l) is _MulIr:
+                return l[1]
+            l, p = _parse_irrep_name(l) if isinstance(l, str) else tuple(l)
+        if isinstance(l, bool) or not isinstance(l, int) or l < 0:
+            raise ValueError(f"the degree l must be a non-negative integer, got {l!r}")
+        if p != 1 and p != -1:
+            raise ValueError(f"the parity p must be 1 or -1, got {p!r}")
+        return tuple.__new__(cls, (l, int(p)))
 
-    @property
-    def l(self) -> int:  # noqa: E743
-        return self[0]
-
-    @property
-    def p(self) -> int:
-        return self[1]
-
-    @property
-    def dim(self) -> int:
-        return 2 * self.l + 1
+    l = property(lambda self: self[0], doc="degree")  # noqa: E741
+    p = property(lambda self: self[1], doc="parity, 1 (even) or -1 (odd)")
+    dim = property(lambda self: 2 * self[0] + 1, doc="dimension 2l + 1")
 
     def is_scalar(self) -> bool:
-        return self.l == 0 and self.p == 1
+        return self == (0, 1)
 
     def __repr__(self) -> str:
-        return f"{self.l}{'e' if self.p == 1 else 'o'}"
+        return f"{self[0]}{'o' if self[1] < 0 else 'e'}"
 
     @classmethod
     def iterator(cls, lmax=None):
-        for l in itertools.count():
-            yield Irrep(l, (-1) ** l)
-            yield Irrep(l, -((-1) ** l))
-            if l == lmax:
-                break
+        """0e, 0o, 1o, 1e, 2e, 2o, ...: for every l the parity of the spherical harmonics first."""
+        degrees = itertools.count() if lmax is None else range(lmax + 1)
+        for l in degrees:
+            natural = -1 if l % 2 else 1
+            yield cls(l, natural)
+            yield cls(l, -natural)
 
     def __mul__(self, other):
-        # selection rule: |l1 - l2| <= l <= l1 + l2, parities multiply
+        """Irreps of the product: ``|l1 - l2| <= l <= l1 + l2``, parities multiply."""
         other = Irrep(other)
-        for l in range(abs(self.l - other.l), self.l + other.l + 1):
-            yield Irrep(l, self.p * other.p)
+        lo, hi = abs(self[0] - other[0]), self[0] + other[0]
+        return (Irrep(l, self[1] * other[1]) for l in range(lo, hi + 1))
 
-    def __rmul__(self, other):
-        assert isinstance(other, int)
-        return Irreps([(other, self)])
+    def __rmul__(self, mul):
+        assert isinstance(mul, int)
+        return Irreps([(mul, self)])
 
     def __add__(self, other):
-        return Irreps(self) + Irreps(other)
+        return Irreps([self]) + other
 
-    def count(self, _value):
-        raise NotImplementedError
-
-    def index(self, _value):
-        raise NotImplementedError
-
-    def __contains__(self, _object):
-        raise NotImplementedError
-
-    def __len__(self):
-        raise NotImplementedError
+    count = index = __contains__ = __len__ = _not_a_sequence
 
 
 class _MulIr(tuple):
+    """``mul`` copies of one irrep."""
+
     def __new__(cls, mul, ir=None):
         if ir is None:
             mul, ir = mul
-        assert isinstance(mul, int)
-        assert isinstance(ir, Irrep)
-        return super().__new__(cls, (mul, ir))
+        assert isinstance(mul, int) and isinstance(ir, Irrep)
+        return tuple.__new__(cls, (mul, ir))
 
-    @property
-    def mul(self) -> int:
-        return self[0]
-
-    @property
-    def ir(self) -> Irrep:
-        return self[1]
-
-    @property
-    def dim(self) -> int:
-        return self.mul * self.ir.dim
+    mul = property(lambda self: self[0])
+    ir = property(lambda self: self[1])
+    dim = property(lambda self: self[0] * self[1].dim)
 
     def __repr__(self) -> str:
-        return f"{self.mul}x{self.ir}"
+        return f"{self[0]}x{self[1]!r}"
 
-    def count(self, _value):
-        raise NotImplementedError
+    count = index = _not_a_sequence
 
-    def index(self, _value):
-        raise NotImplementedError
+
+def _terms_of_string(text: str):
+    if not text.strip():
+        return []
+    terms = []
+    for piece in text.split("+"):
+        m = _TERM.fullmatch(piece)
+        if m is None:
+            raise ValueError(f'Unable to convert string "{text}" into an Irreps')
+        terms.append(_MulIr(int(m.group(1) or 1), Irrep(m.group(2))))
+    return terms
+
+
+def _term_of_item(item):
+    """One element of a list given to ``Irreps``: "1o", Irrep, (mul, irrep-like) or a ``_MulIr``."""
+    if isinstance(item, _MulIr):
+        return item
+    if isinstance(item, (str, Irrep)):
+        return _MulIr(1, Irrep(item))
+    try:
+        mul, ir = item
+    except (TypeError, ValueError):
+        raise ValueError(f'Unable to interpret "{item}" as an irrep.') from None
+    if isinstance(mul, bool) or not isinstance(mul, int) or mul < 0:
+        raise ValueError(f'Unable to interpret "{item}" as an irrep.')
+    return _MulIr(mul, Irrep(ir))
 
 
 class Irreps(tuple):
@@ -131,156 +143,134 @@ class Irreps(tuple):
 
     def __new__(cls, irreps=None):
         if isinstance(irreps, Irreps):
-            return super().__new__(cls, irreps)
-        out = []
-        if isinstance(irreps, Irrep):
-            out.append(_MulIr(1, Irrep(irreps)))
-        elif isinstance(irreps, str):
-            try:
-                if irreps.strip() != "":
-                    for term in irreps.split("+"):
-                        if "x" in term:
-                            mul, ir = term.split("x")
-                            mul, ir = int(mul), Irrep(ir)
-                        else:
-                            mul, ir = 1, Irrep(term)
-                        assert isinstance(mul, int) and mul >= 0
-                        out.append(_MulIr(mul, ir))
-            except Exception:
-                raise ValueError(f'Unable to convert string "{irreps}" into an Irreps')
+            terms = irreps
         elif irreps is None:
-            pass
+            terms = ()
+        elif isinstance(irreps, Irrep):
+            terms = (_MulIr(1, irreps),)
+        elif isinstance(irreps, str):
+            terms = _terms_of_string(irreps)
         else:
-            for mul_ir in irreps:
-                mul, ir = None, None
-                if isinstance(mul_ir, str):
-                    mul, ir = 1, Irrep(mul_ir)
-                elif isinstance(mul_ir, Irrep):
-                    mul, ir = 1, mul_ir
-                elif isinstance(mul_ir, _MulIr):
-                    mul, ir = mul_ir
-                elif len(mul_ir) == 2:
-                    mul, ir = mul_ir
-                    ir = Irrep(ir)
-                if not (isinstance(mul, int) and mul >= 0 and ir is not None):
-                    raise ValueError(f'Unable to interpret "{mul_ir}" as an irrep.')
-                out.append(_MulIr(mul, ir))
-        return super().__new__(cls, out)
+            terms = [_term_of_item(item) for item in irreps]
+        return tuple.__new__(cls, terms)
 
     @staticmethod
     def spherical_harmonics(lmax: int, p: int = -1) -> "Irreps":
-        return Irreps([(1, (l, p**l)) for l in range(lmax + 1)])
+        """``0e + 1o + 2e + ...`` up to ``lmax`` (``p = 1``: all even)."""
+        return Irreps([_MulIr(1, Irrep(l, p**l)) for l in range(lmax + 1)])
 
-    def slices(self):
-        out, i = [], 0
-        for mul_ir in self:
-            out.append(slice(i, i + mul_ir.dim))
-            i += mul_ir.dim
-        return out
-
-    def randn(self, *size, normalization="component", requires_grad=False, dtype=None, device=None):
-        di = size.index(-1)
-        lsize, rsize = size[:di], size[di + 1 :]
-        if normalization == "component":
-            return torch.randn(*lsize, self.dim, *rsize, requires_grad=requires_grad, dtype=dtype, device=device)
-        if normalization == "norm":
-            x = torch.zeros(*lsize, self.dim, *rsize, requires_grad=requires_grad, dtype=dtype, device=device)
-            with torch.no_grad():
-                for s, (mul, ir) in zip(self.slices(), self):
-                    r = torch.randn(*lsize, mul, ir.dim, *rsize, dtype=dtype, device=device)
-                    r.div_(r.norm(2, dim=di + 1, keepdim=True))
-                    x.narrow(di, s.start, mul * ir.dim).copy_(r.reshape(*lsize, -1, *rsize))
-            return x
-        raise ValueError("Normalization needs to be 'norm' or 'component'")
-
-    def __getitem__(self, i):
-        x = super().__getitem__(i)
-        return Irreps(x) if isinstance(i, slice) else x
-
-    def __contains__(self, ir) -> bool:
-        ir = Irrep(ir)
-        return any(ir == irrep for _, irrep in self)
-
-    def count(self, ir) -> int:
-        ir = Irrep(ir)
-        return sum(mul for mul, irrep in self if ir == irrep)
-
-    def index(self, _object):
-        raise NotImplementedError
-
-    def __add__(self, irreps) -> "Irreps":
-        return Irreps(super().__add__(Irreps(irreps)))
-
-    def __mul__(self, other) -> "Irreps":
-        if isinstance(other, Irreps):
-            raise NotImplementedError("Use o3.TensorProduct for this, see the documentation")
-        return Irreps(super().__mul__(other))
-
-    def __rmul__(self, other) -> "Irreps":
-        return Irreps(super().__rmul__(other))
-
-    def simplify(self) -> "Irreps":
-        out = []
-        for mul, ir in self:
-            if out and out[-1][1] == ir:
-                out[-1] = (out[-1][0] + mul, ir)
-            elif mul > 0:
-                out.append((mul, ir))
-        return Irreps(out)
-
-    def remove_zero_multiplicities(self) -> "Irreps":
-        return Irreps([(mul, ir) for mul, ir in self if mul > 0])
-
-    def sort(self):
-        """Stable sort by ``(l, p)`` (odd before even at equal ``l``); returns ``(irreps, p, inv)``."""
-        Ret = collections.namedtuple("sort", ["irreps", "p", "inv"])
-        keyed = sorted((ir, i, mul) for i, (mul, ir) in enumerate(self))
-        inv = tuple(i for _, i, _ in keyed)
-        p = tuple(inv.index(i) for i in range(len(inv)))
-        return Ret(Irreps([(mul, ir) for ir, _, mul in keyed]), p, inv)
-
-    def regroup(self) -> "Irreps":
-        return self.sort().irreps.simplify()
-
-    def filter(self, keep=None, *, drop=None, lmax: int = None) -> "Irreps":
-        if keep is None and drop is None and lmax is None:
-            return self
-        if sum(v is not None for v in (keep, drop, lmax)) > 1:
-            raise ValueError("Cannot specify more than one of keep, drop and lmax")
-        if lmax is not None:
-            return Irreps([(mul, ir) for mul, ir in self if ir.l <= lmax])
-        sel, want = (keep, True) if keep is not None else (drop, False)
-        if callable(sel):
-            return Irreps([mul_ir for mul_ir in self if bool(sel(mul_ir)) == want])
-        if isinstance(sel, str):
-            sel = Irreps(sel)
-        if isinstance(sel, Irrep):
-            sel = [sel]
-        if isinstance(sel, _MulIr):
-            sel = [sel.ir]
-        sel = {Irrep(ir) for ir in sel}
-        return Irreps([(mul, ir) for mul, ir in self if (ir in sel) == want])
-
+    # ---- layout -------------------------------------------------------------------------------------------------
     @property
     def dim(self) -> int:
-        return sum(mul * ir.dim for mul, ir in self)
+        return sum(term.dim for term in self)
 
     @property
     def num_irreps(self) -> int:
-        return sum(mul for mul, _ in self)
+        return sum(term.mul for term in self)
 
     @property
     def ls(self) -> List[int]:
-        return [l for mul, (l, p) in self for _ in range(mul)]
+        return [term.ir.l for term in self for _ in range(term.mul)]
 
     @property
     def lmax(self) -> int:
-        if len(self) == 0:
-            raise ValueError("Cannot get lmax of empty Irreps")
-        return max(self.ls)
+        if not self:
+            raise ValueError("an empty Irreps has no lmax")
+        return max(term.ir.l for term in self)
+
+    def slices(self):
+        """Column range of every block in a feature vector."""
+        ends = list(itertools.accumulate(term.dim for term in self))
+        return [slice(end - term.dim, end) for term, end in zip(self, ends)]
+
+    def randn(self, *size, normalization="component", requires_grad=False, dtype=None, device=None):
+        """Random features; the ``-1`` in ``size`` stands for the irreps axis.  ``"component"``: every component
+        N(0, 1); ``"norm"``: every irrep copy uniformly on the unit sphere of its 2l+1 components."""
+        axis = size.index(-1)
+        before, after = size[:axis], size[axis + 1 :]
+        if normalization == "component":
+            return torch.randn(*before, self.dim, *after, requires_grad=requires_grad, dtype=dtype, device=device)
+        if normalization != "norm":
+            raise ValueError(f"normalization must be 'component' or 'norm', got {normalization!r}")
+        blocks = []
+        for term in self:
+            v = torch.randn(*before, term.mul, term.ir.dim, *after, dtype=dtype, device=device)
+            v = v / v.norm(dim=axis + 1, keepdim=True)
+            blocks.append(v.reshape(*before, term.dim, *after))
+        x = torch.cat(blocks, dim=axis) if blocks else torch.zeros(*before, 0, *after, dtype=dtype, device=device)
+        return x.requires_grad_(requires_grad)
+
+    # ---- tuple protocol -------------------------------------------------------------------------------------------
+    def __getitem__(self, i):
+        got = tuple.__getitem__(self, i)
+        return Irreps(got) if isinstance(i, slice) else got
+
+    def __contains__(self, ir) -> bool:
+        wanted = Irrep(ir)
+        return any(term.ir == wanted for term in self)
+
+    def count(self, ir) -> int:
+        """Total multiplicity of ``ir``."""
+        wanted = Irrep(ir)
+        return sum(term.mul for term in self if term.ir == wanted)
+
+    index = _not_a_sequence
+
+    def __add__(self, irreps) -> "Irreps":
+        return Irreps(tuple(self) + tuple(Irreps(irreps)))
+
+    def __mul__(self, n) -> "Irreps":
+        if isinstance(n, Irreps):
+            raise NotImplementedError("Irreps * Irreps is not defined: build an o3.TensorProduct")
+        return Irreps(tuple(self) * n)
+
+    __rmul__ = __mul__
 
     def __repr__(self) -> str:
-        return "+".join(f"{mul_ir}" for mul_ir in self)
+        return "+".join(map(repr, self))
+
+    # ---- rearrangements -------------------------------------------------------------------------------------------
+    def remove_zero_multiplicities(self) -> "Irreps":
+        return Irreps([term for term in self if term.mul > 0])
+
+    def simplify(self) -> "Irreps":
+        """Merges neighbouring blocks of the same irrep and drops empty ones (the order is kept)."""
+        merged = []
+        for ir, run in itertools.groupby(self.remove_zero_multiplicities(), key=lambda term: term.ir):
+            merged.append((sum(term.mul for term in run), ir))
+        return Irreps(merged)
+
+    def sort(self):
+        """Stable sort by ``(l, p)``; returns ``(irreps, p, inv)`` with ``sorted[p[i]] = self[i]`` and
+        ``sorted[j] = self[inv[j]]``."""
+        inv = tuple(sorted(range(len(self)), key=lambda i: (self[i].ir, i, self[i].mul)))
+        p = [0] * len(inv)
+        for new, old in enumerate(inv):
+            p[old] = new
+        return _SortResult(Irreps([self[i] for i in inv]), tuple(p), inv)
+
+    def regroup(self) -> "Irreps":
+        """Sorted, with equal irreps merged."""
+        ordered, _, _ = self.sort()
+        return ordered.simplify()
+
+    def filter(self, keep=None, *, drop=None, lmax: int = None) -> "Irreps":
+        """Blocks selected by ``keep`` (irreps or a predicate on ``(mul, ir)``), by ``drop`` (the complement) or by
+        ``lmax``; at most one of the three."""
+        given = [name for name, v in (("keep", keep), ("drop", drop), ("lmax", lmax)) if v is not None]
+        if not given:
+            return self
+        if len(given) > 1:
+            raise ValueError("Cannot specify more than one of keep, drop and lmax")
+        if lmax is not None:
+            return Irreps([term for term in self if term.ir.l <= lmax])
+        selector, wanted = (keep, True) if keep is not None else (drop, False)
+        if callable(selector):
+            return Irreps([term for term in self if bool(selector(term)) is wanted])
+        if isinstance(selector, (str, Irrep, _MulIr)):
+            selector = [Irrep(selector)] if not isinstance(selector, str) else [term.ir for term in Irreps(selector)]
+        chosen = {Irrep(ir) for ir in selector}
+        return Irreps([term for term in self if (term.ir in chosen) is wanted])
 
 
 IrrepsLike = Union[str, Irreps, Irrep, list, tuple]
