@@ -442,6 +442,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--locality-variants", action="store_true", help="time the headline graph with sorted edges / Morton node ids also when --only is given")
+    ap.add_argument("--no-headline", action="store_true", help="profiling aid: run only the sections of --only (those that do not build on the headline graph) and print their results, so that a profile holds the launches of one configuration only")
     ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_b,mace_bf16,nequip40,uvw,uvw_bf16,conv,radial,nequip_bwd,uvw_bwd (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -450,6 +451,17 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.no_headline:
+        sections = {"copy": lambda: bench_copy(args, dev), "sh": lambda: bench_sh(args, dev), "mace": lambda: bench_mace(args, dev),
+                    "mace_b": lambda: bench_mace(args, dev, variant="B"), "mace_bf16": lambda: bench_mace(args, dev, torch.bfloat16),
+                    "nequip40": lambda: bench_nequip_cube40(args, dev), "uvw": lambda: bench_uvw(args, dev),
+                    "uvw_bf16": lambda: bench_uvw(args, dev, torch.bfloat16), "uvw_bwd": lambda: bench_uvw_backward(args, dev)}  # fmt: skip
+        names = [n for n in args.only.split(",") if n]
+        if not names or any(n not in sections for n in names):
+            sys.exit("bench.py --no-headline needs --only with sections out of: " + ",".join(sections))
+        print(json.dumps({"sections_only": {n: sections[n]() for n in names}}))
+        return
 
     neq, ctx = bench_nequip(args, dev)
     other = {"nequip_uvu": neq}
