@@ -8,6 +8,7 @@ namespace e3x {
 extern const char* const kTplCommon;
 extern const char* const kTplUvu;
 extern const char* const kTplUvuFc;
+extern const char* const kTplUvuMfma;
 extern const char* const kTplUvwSmall;
 extern const char* const kTplUvwMfma;
 extern const char* const kTplUvwMfmaBf16;

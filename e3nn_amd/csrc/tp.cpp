@@ -61,6 +61,10 @@ struct e3x_plan {
   std::string radial_desc;
   std::mutex mu;
   std::vector<std::unique_ptr<SubKernel>> subs;
+  // uvu, bf16 storage: the message kernel (gather + product + scatter) with the contraction on the matrix cores,
+  // when the instruction set fits it; the plain product keeps the kernels of `subs`
+  std::unique_ptr<SubKernel> msg_mfma;
+  int msg_groups = 0;  // wavefronts per output row
   // uvw_mfma: the weight-gradient kernel is a code object of its own, built on first use
   std::unique_ptr<SubKernel> dw;
   long long dw_tiles = 0;  // grid.x: the largest tile count of a path
@@ -287,6 +291,119 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only 
   s << "}  // namespace cfg\n";
   *src = s.str() + e3x::kTplCommon + (tpl ? tpl : e3x::kTplUvu);
   return E3X_OK;
+}
+
+
+// ---- uvu message kernel on the matrix cores -----------------------------------------------------------------
+// Tables of templates/uvu_mfma.inc.  Returns false (and builds nothing) when the instruction set does not fit:
+// bf16 storage, per-edge weights on every instruction, multiplicity 1 on the second input, one multiplicity U = 128
+// on the first input and the output, at most 16 components per multiplicity index on the first input, split over
+// the two halves of the K range without cutting an irrep, and exactly one instruction per output irrep (the
+// per-path output blocks that the reference's convolution builds, e3nn/nn/models/v2106/points_convolution.py:60-76).
+bool build_uvu_msg_mfma_source(e3x_plan& P, SubKernel& K, std::string* src) {
+  if (P.dtype != E3X_BF16 || P.shared_weights || P.paths.empty() || P.in2_dim > 16 || P.in2_dim == 0) return false;
+  const int U = 128, UT = U / 32;
+  std::vector<char> used1(P.in1.size(), 0);
+  std::vector<int> n_out(P.out.size(), 0);
+  for (const auto& p : P.paths) {
+    if (p.mode != E3X_MODE_UVU || !p.has_w || P.in2[p.in2].mul != 1 || P.in1[p.in1].mul != U || P.out[p.out].mul != U)
+      return false;
+    used1[p.in1] = 1;
+    if (++n_out[p.out] > 1) return false;
+  }
+  if (P.in1_dim % 8 || P.weight_numel % 8 || P.in2_dim % 8) return false;  // rows are read in 16-byte pieces
+  // K slots: first-fit of the input irreps, largest first, into two halves of 8
+  std::vector<int> order;
+  for (size_t a = 0; a < P.in1.size(); ++a) if (used1[a]) order.push_back((int)a);
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return P.in1[a].l > P.in1[b].l; });
+  std::vector<int> half_of(P.in1.size(), -1), slot0(P.in1.size(), 0);
+  int fill[2] = {0, 0};
+  std::vector<int> runs[2];
+  for (int a : order) {
+    const int d = 2 * P.in1[a].l + 1;
+    const int h = fill[0] + d <= 8 ? 0 : (fill[1] + d <= 8 ? 1 : -1);
+    if (h < 0) return false;
+    half_of[a] = h, slot0[a] = fill[h], fill[h] += d;
+    runs[h].push_back(a);
+  }
+  std::ostringstream s;
+  emit_header(s, P);
+  int prefetch = env_int("E3X_UVUM_PREFETCH", 2), mblk = env_int("E3X_UVUM_MBLK", 8);
+  if (prefetch != 2 && prefetch != 4 && prefetch != 8) prefetch = 4;
+  if (mblk != 8 && mblk != 16 && mblk != 32) mblk = 8;
+  s << "constexpr int U = " << U << ", UT = " << UT << ", MBLK = " << mblk << ", PREFETCH = " << prefetch << ";\n";
+  s << "#define E3X_UVUM_OCC " << env_int("E3X_UVUM_OCC", 3) << "\n";
+  // K slot sl (0-7: first half, 8-15: second) of index u is component kslot_off[sl] + u * kslot_d[sl] of a source row
+  int ks_off[16], ks_d[16];
+  for (int i = 0; i < 16; ++i) ks_off[i] = 0, ks_d[i] = 0;
+  for (int h = 0; h < 2; ++h)
+    for (int a : runs[h]) {
+      const int d = 2 * P.in1[a].l + 1;
+      for (int i = 0; i < d; ++i) ks_off[8 * h + slot0[a] + i] = P.off1[a] + i, ks_d[8 * h + slot0[a] + i] = d;
+    }
+  s << "constexpr int kslot_off[16] = {";
+  for (int i = 0; i < 16; ++i) s << ks_off[i] << ", ";
+  s << "};\nconstexpr int kslot_d[16] = {";
+  for (int i = 0; i < 16; ++i) s << ks_d[i] << ", ";
+  s << "};\n";
+  // paths and their Clebsch-Gordan non-zeros (path weight folded in)
+  std::vector<int> all(P.paths.size());
+  for (size_t i = 0; i < all.size(); ++i) all[i] = (int)i;
+  NzList L = emit_nz(P, all);
+  s << "struct GPath { int x2off, d2, half, slot0, d1, woff, ooff, d3, nz_beg, nz_end; };\n";
+  s << "constexpr int NP = " << P.paths.size() << ";\nconstexpr GPath gpaths[NP] = {\n";
+  for (size_t i = 0; i < P.paths.size(); ++i) {
+    const auto& p = P.paths[i];
+    s << "  {" << P.off2[p.in2] << ", " << 2 * P.in2[p.in2].l + 1 << ", " << half_of[p.in1] << ", " << slot0[p.in1] << ", "
+      << 2 * P.in1[p.in1].l + 1 << ", " << p.woff << ", " << P.offo[p.out] << ", " << 2 * P.out[p.out].l + 1 << ", "
+      << L.beg[i] << ", " << L.end[i] << "},\n";
+  }
+  s << "};\n";
+  emit_nz_table(s, L);
+  // matrix rows: the columns (path, k) of the product in pairs (k, k + 1) of one path, 16 pairs per 32-row tile,
+  // two tiles per group (one wavefront per output row and group)
+  struct PairRow { int path, k0, k1; };
+  std::vector<PairRow> pr;
+  for (size_t i = 0; i < P.paths.size(); ++i) {
+    const int d3 = 2 * P.out[P.paths[i].out].l + 1;
+    for (int k = 0; k < d3; k += 2) pr.push_back({(int)i, k, k + 1 < d3 ? k + 1 : -1});
+  }
+  // tiles per group: one keeps a wavefront at 64 accumulators and three waves per SIMD
+  const int tiles = env_int("E3X_UVUM_TILES", 1) == 2 ? 2 : 1, ppg = 16 * tiles;
+  const int ng = ((int)pr.size() + ppg - 1) / ppg;
+  if (ng > 8) return false;  // one wavefront per group, one workgroup per output row
+  K.waves_per_block = ng;
+  while ((int)pr.size() < ng * ppg) pr.push_back({-1, -1, -1});
+  s << "constexpr int TILES = " << tiles << ", NG = " << ng << ";\nstruct Pair { int path, k0, k1; };\nconstexpr Pair pairs[NG * "
+    << ppg << "] = {\n";
+  for (const auto& q : pr) s << "  {" << q.path << ", " << q.k0 << ", " << q.k1 << "},\n";
+  s << "};\n";
+  std::ostringstream gb, ge, rv, rh;
+  int gw_max = 0;
+  for (int g = 0; g < ng; ++g) {
+    int lo = 1 << 30, hi = -1;
+    unsigned valid[2] = {0, 0}, half[2] = {0, 0};
+    for (int q = 0; q < ppg; ++q) {
+      const PairRow& r = pr[g * ppg + q];
+      if (r.path < 0) continue;
+      lo = std::min(lo, r.path), hi = std::max(hi, r.path);
+      const int tile = q / 16, row0 = 8 * ((q % 16) / 4) + (q % 16) % 4;
+      const unsigned hb = (unsigned)half_of[P.paths[r.path].in1];
+      valid[tile] |= 1u << row0, half[tile] |= hb << row0;
+      if (r.k1 >= 0) valid[tile] |= 1u << (row0 + 4), half[tile] |= hb << (row0 + 4);
+    }
+    gb << lo << ", ", ge << hi + 1 << ", ";
+    gw_max = std::max(gw_max, hi + 1 - lo);
+    rv << "{" << valid[0] << "u" << (tiles == 2 ? ", " + std::to_string(valid[1]) + "u" : "") << "}, ";
+    rh << "{" << half[0] << "u" << (tiles == 2 ? ", " + std::to_string(half[1]) + "u" : "") << "}, ";
+  }
+  s << "constexpr int gp_beg[NG] = {" << gb.str() << "};\nconstexpr int gp_end[NG] = {" << ge.str() << "};\n";
+  s << "constexpr int GW_MAX = " << gw_max << ";\n";
+  s << "constexpr unsigned row_valid[NG][TILES] = {" << rv.str() << "};\nconstexpr unsigned row_half[NG][TILES] = {" << rh.str() << "};\n";
+  s << "}  // namespace cfg\n";
+  P.msg_groups = ng;
+  *src = s.str() + e3x::kTplCommon + e3x::kTplUvuMfma;
+  return true;
 }
 
 // ---- uvw (lane <-> output multiplicity, VALU) ----------------------------------------
@@ -688,6 +805,17 @@ int load_functions(e3x_plan* P, int dev) {
     }
     K->module[dev] = mod;
   }
+  if (P->msg_mfma && !P->msg_mfma->module[dev]) {
+    SubKernel* K = P->msg_mfma.get();
+    hipModule_t mod = nullptr;
+    hipError_t err = hipModuleLoad(&mod, K->hsaco.c_str());
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, "hipModuleLoad(" + K->hsaco + ") failed: " + hipGetErrorString(err));
+    if (hipModuleGetFunction(&K->fn_fused[dev], mod, "e3x_uvu_mfma_fused") != hipSuccess ||
+        hipModuleGetFunction(&K->fn_pack[dev], mod, "e3x_uvu_mfma_pack_x1") != hipSuccess)
+      return fail(E3X_ERR_HIP, "kernel e3x_uvu_mfma_fused / e3x_uvu_mfma_pack_x1 missing from " + K->hsaco);
+    K->module[dev] = mod;
+  }
   return E3X_OK;
 }
 
@@ -832,6 +960,15 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
     P->key += (P->key.empty() ? "" : "+") + K->key;
     P->subs.push_back(std::move(K));
   }
+  if (P->family == "uvu" && env_int("E3X_UVU_MFMA", 1)) {
+    std::unique_ptr<SubKernel> K(new SubKernel);
+    std::string src;
+    if (build_uvu_msg_mfma_source(*P, *K, &src)) {
+      if ((rc = e3x::get_code_object("uvu_mfma", src, &K->key, &K->hsaco))) return rc;
+      P->key += "+" + K->key;
+      P->msg_mfma = std::move(K);
+    }
+  }
   *out = P.release();
   return E3X_OK;
 }
@@ -948,6 +1085,19 @@ extern "C" int e3x_tp_gather_scatter_ordered(e3x_plan* P, const void* node_x, co
                                              const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
                                              const int32_t* row_order, void* out, int64_t E, int64_t num_src_nodes,
                                              int64_t num_out_nodes, void* stream) {
+  return e3x_tp_gather_scatter_ws(P, node_x, edge_attr, w, src, idx_bits, rowptr, perm, row_order, out, E, num_src_nodes,
+                                  num_out_nodes, nullptr, 0, stream);
+}
+
+extern "C" size_t e3x_tp_gather_scatter_workspace_bytes(const e3x_plan* P, int64_t num_src_nodes) {
+  if (!P || !P->msg_mfma || num_src_nodes <= 0) return 0;
+  return (size_t)num_src_nodes * 128 * 32;  // the node table in operand order: 16 bf16 per multiplicity index
+}
+
+extern "C" int e3x_tp_gather_scatter_ws(e3x_plan* P, const void* node_x, const void* edge_attr, const void* w,
+                                        const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
+                                        const int32_t* row_order, void* out, int64_t E, int64_t num_src_nodes,
+                                        int64_t num_out_nodes, void* workspace, size_t workspace_bytes, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: null plan");
   if (P->family != "uvu") return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: the plan must be all-uvu");
   if (P->shared_weights && P->weight_numel)
@@ -969,6 +1119,30 @@ extern "C" int e3x_tp_gather_scatter_ordered(e3x_plan* P, const void* node_x, co
   long long n_rows = num_out_nodes, n_src = num_src_nodes;
   void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&w,         (void*)&out,    (void*)&src,  (void*)&idx64,
                   (void*)&rowptr, (void*)&perm,      (void*)&row_order, (void*)&n_rows, (void*)&n_src};
+  // the matrix-core message kernel: needs the workspace for the node table in operand order, 8-byte aligned weight
+  // rows and a 16-byte aligned workspace; without them the vector-ALU kernels below run
+  if (P->msg_mfma && E > 0 && workspace && workspace_bytes >= e3x_tp_gather_scatter_workspace_bytes(P, num_src_nodes) &&
+      !(((uintptr_t)w | (uintptr_t)edge_attr) & 15) && !((uintptr_t)workspace & 15)) {
+    SubKernel* K = P->msg_mfma.get();
+    {
+      const long long pblocks = n_src;  // a workgroup per node
+      void* pargs[] = {(void*)&node_x, (void*)&workspace, (void*)&n_src};
+      hipError_t perr = hipModuleLaunchKernel(K->fn_pack[dev], (unsigned)pblocks, 1, 1, 256, 1, 1, 0, st, pargs, nullptr);
+      if (perr != hipSuccess)
+        return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(perr));
+    }
+    void* margs[] = {(void*)&workspace, (void*)&edge_attr, (void*)&w,         (void*)&out,    (void*)&src,  (void*)&idx64,
+                     (void*)&rowptr,    (void*)&perm,      (void*)&row_order, (void*)&n_rows, (void*)&n_src};
+    const long long items = n_rows * P->msg_groups;
+    long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
+    blocks = (blocks + 7) / 8 * 8;
+    if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
+    hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1, 0,
+                                           st, margs, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
+    return E3X_OK;
+  }
   for (auto& K : P->subs) {
     const long long items = n_rows * K->chunks;
     long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;

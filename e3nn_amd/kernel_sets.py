@@ -171,7 +171,7 @@ def all_tensor_products():
         ("cfg3_merged", cfg3(True), (torch.float32, torch.bfloat16)),
         ("cfg3_builder", cfg3(False), (torch.float32,)),
         ("cfg4_A", cfg4("A"), (torch.float32, torch.bfloat16)),
-        ("cfg4_B", cfg4("B"), (torch.float32,)),
+        ("cfg4_B", cfg4("B"), (torch.float32, torch.bfloat16)),
         ("cfg5", cfg5(), (torch.float32, torch.bfloat16)),
         ("mfma_small", mfma_small(), (torch.float32,)),
         ("node_fctp", node_fctp(), (torch.float32,)),

@@ -115,12 +115,17 @@ class _Plan:
     def gather_scatter(self, table, edge_attr, w, gather_idx, edges, num_table_rows):
         """``out[n] = sum_{e: edges groups e under n} TP(table[gather_idx[e]], edge_attr[e], w[e])``."""
         out = torch.empty(edges.num_nodes, self.out_dim, dtype=table.dtype, device=table.device)
+        L = _lib.lib()
         with torch.cuda.device(table.device):
+            # scratch of the matrix-core message kernel (the node table in operand order); 0 for every other plan
+            ws_bytes = L.e3x_tp_gather_scatter_workspace_bytes(self.handle, num_table_rows)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=table.device) if ws_bytes else None
             _lib.check(
-                _lib.lib().e3x_tp_gather_scatter_ordered(
+                L.e3x_tp_gather_scatter_ws(
                     self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(gather_idx),
                     gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(edges.row_order),
-                    _lib.ptr(out), edges.num_edges, num_table_rows, edges.num_nodes, _lib.stream_ptr(table.device),
+                    _lib.ptr(out), edges.num_edges, num_table_rows, edges.num_nodes, _lib.ptr(ws), ws_bytes,
+                    _lib.stream_ptr(table.device),
                 )  # fmt: skip
             )
         return out

@@ -213,6 +213,21 @@ int e3x_tp_gather_scatter_ordered(e3x_plan* plan, const void* node_x, const void
                                   const int32_t* row_order, void* out, int64_t E, int64_t num_src_nodes,
                                   int64_t num_out_nodes, void* stream);
 
+/* e3x_tp_gather_scatter_ordered with caller-owned device scratch.  Plans in bf16 storage whose instruction set fits
+ * the matrix-core message kernel (per-edge weights on every instruction, multiplicity 128 on the first input and
+ * the output, 1 on the second, at most 16 components per multiplicity index, one instruction per output irrep:
+ * what the reference's convolution builds, e3nn/nn/models/v2106/points_convolution.py:60-76) take that kernel
+ * when given e3x_tp_gather_scatter_workspace_bytes(plan, num_src_nodes) bytes (16-byte aligned; the call writes a
+ * copy of the node table in matrix-operand order there); the Clebsch-Gordan contraction then runs in bf16 on the
+ * matrix cores with fp32 accumulation (the per-edge matrices are rounded to bf16 once more than in the other
+ * kernels).  Every other plan needs no workspace (the function returns 0) and runs as e3x_tp_gather_scatter_ordered;
+ * so does a call without workspace. */
+size_t e3x_tp_gather_scatter_workspace_bytes(const e3x_plan* plan, int64_t num_src_nodes);
+int e3x_tp_gather_scatter_ws(e3x_plan* plan, const void* node_x, const void* edge_attr, const void* w, const void* src,
+                             int idx_bits, const int32_t* rowptr, const int32_t* perm, const int32_t* row_order,
+                             void* out, int64_t E, int64_t num_src_nodes, int64_t num_out_nodes, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
 /* Gradients of the `uvu` product (plain: src = dst = NULL, row e of every table; fused: the edge lists
  * of e3x_tp_gather_scatter, unsorted) with respect to the per-sample weights and the second input:
  *   grad_w[E, weight_numel] (shared weights: one [weight_numel] vector summed over the edges with fp32 atomics),

@@ -178,18 +178,43 @@ def test_fused_matches_oracle(maker, N, E, idx):
     assert (out - unfused).abs().max().item() < 1e-4 * scale
 
 
-def test_fused_bf16_storage():
-    tp = ks.cfg4("A")
-    N, E = 50, 1000
-    src, dst = random_graph(N, E, seed=9, dtype=torch.int32)
-    node_x, attr, w = seeded(N, 2048, seed=1), seeded(E, 16, seed=2), seeded(E, 2944, seed=3)
+@pytest.mark.parametrize("variant,N,E,idx", [("A", 50, 1000, torch.int32), ("A", 7, 900, torch.int64), ("B", 40, 700, torch.int32),
+                                              ("A", 300, 5, torch.int64)])  # fmt: skip
+def test_fused_bf16_storage(variant, N, E, idx):
+    # bf16 storage of the 128-channel l <= 3 sets runs the message kernel with the contraction on the matrix cores
+    # (one workgroup per row, 4 or 6 wavefronts): rows longer than a block of 64 edges (E / N > 64), rows without
+    # edges, the per-edge matrices rounded to bf16 once more than in the other kernels
+    tp = ks.cfg4(variant)
+    assert "uvu_mfma" in tp._plan(torch.bfloat16).key
+    src, dst = random_graph(N, E, seed=9, dtype=idx)
+    dst = torch.where(dst == 2, dst + 1, dst)  # node 2 receives nothing
+    node_x, attr, w = seeded(N, 2048, seed=1), seeded(E, 16, seed=2), seeded(E, tp.weight_numel, seed=3)
     nb, ab, wb = (t.to(DEV).to(torch.bfloat16) for t in (node_x, attr, w))
     out = tp.forward_gather_scatter(nb, ab, wb, src.to(DEV), dst.to(DEV), N)
+    assert out.dtype == torch.bfloat16 and not out[2].any()
     ref = tp_gather_scatter(
         oracle_spec(tp), nb.float().cpu().numpy(), ab.float().cpu().numpy(), wb.float().cpu().numpy(), src.numpy(), dst.numpy(), N
     )
     scale = float(np.abs(ref).max())
-    assert_close(out, ref, atol=1e-2 * scale, rtol=1e-2, what="bf16 fused")
+    assert_close(out, ref, atol=1e-2 * scale / 4, rtol=1e-2, what=f"bf16 fused {variant} N={N} E={E}")
+    # bit-reproducible, and the same bits for an edge list already grouped by destination
+    assert torch.equal(tp.forward_gather_scatter(nb, ab, wb, src.to(DEV), dst.to(DEV), N), out)
+    order = torch.argsort(dst, stable=True)
+    od = order.to(DEV)
+    assert torch.equal(tp.forward_gather_scatter(nb, ab[od], wb[od], src[order].to(DEV), dst[order].to(DEV), N), out)
+    # without the workspace the C entry point runs the vector-ALU kernels: same result up to the rounding of the matrices
+    from e3nn_amd import _lib
+
+    plan = tp._plan(torch.bfloat16)
+    edges = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    plain = torch.empty_like(out)
+    s_d = src.to(DEV)
+    with torch.cuda.device(DEV):
+        _lib.check(_lib.lib().e3x_tp_gather_scatter_ordered(
+            plan.handle, _lib.ptr(nb), _lib.ptr(ab), _lib.ptr(wb), _lib.ptr(s_d), s_d.element_size() * 8, _lib.ptr(edges.rowptr),
+            _lib.ptr(edges.perm), None, _lib.ptr(plain), E, N, N, _lib.stream_ptr(torch.device(DEV))))  # fmt: skip
+    assert_close(plain, ref, atol=1e-2 * scale / 8, rtol=1e-2, what=f"bf16 fused {variant} without workspace")
+    assert (plain.float() - out.float()).abs().max().item() <= 1e-2 * scale / 2
 
 
 @pytest.mark.parametrize("case,N,E,idx", [
