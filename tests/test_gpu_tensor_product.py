@@ -264,3 +264,18 @@ def test_uvw_bf16_storage_full_size():
     part = tpb(xb[4096 : 4096 + 256], yb[4096 : 4096 + 256]).float()
     assert (part - out[4096 : 4096 + 256].float()).abs().max().item() <= 2.0**-7 * scale
     assert abs(out.float().var().item() * 16384 - 1.0) < 0.1
+
+
+def test_provider_binding_runs_the_same_kernels():
+    # e3x plans built by the provider from (Irreps, Instruction) data give the product's own results, with e3nn's
+    # broadcasting of leading dimensions
+    from e3nn_amd import provider
+
+    for tp, shared in ((ks.cfg1().to(DEV), True), (ks.cfg3(True), False)):
+        gm = provider.hip_provider(tp.irreps_in1, tp.irreps_in2, tp.irreps_out, tp.instructions, shared, True, True)
+        x1 = seeded(5, 1, tp.irreps_in1.dim, seed=1).to(DEV)
+        x2 = seeded(1, 3, tp.irreps_in2.dim, seed=2).to(DEV)
+        w = tp.weight.detach() if shared else seeded(5, 3, tp.weight_numel, seed=3).to(DEV)
+        got = gm(x1, x2, w)
+        ref = tp(x1, x2) if shared else tp(x1, x2, w)
+        assert got.shape == (5, 3, tp.irreps_out.dim) and torch.equal(got, ref)

@@ -326,3 +326,19 @@ def test_weight_gradient_entry_point_rejects_other_connection_modes():
     one = ctypes.c_void_p(16)  # never dereferenced: the mode check comes first
     assert L.e3x_tp_backward_w_uvw(plan.handle, one, one, one, one, 4, None) == _lib.ERR_INVALID
     assert b"all-uvw" in L.e3x_last_error()
+
+
+def test_provider_binding_builds_plans_from_constructor_data():
+    # the code-generation provider a reference maintainer would register: descriptor filled from Irreps + Instruction
+    from e3nn_amd import provider
+
+    for tp in (ks.cfg1(), ks.cfg3(True), ks.mixed_modes()):
+        gm = provider.hip_provider(tp.irreps_in1, tp.irreps_in2, tp.irreps_out, tp.instructions, tp.shared_weights, True, True)
+        assert isinstance(gm, torch.fx.GraphModule)
+        assert (gm.hip.weight_numel, gm.hip.in1_dim, gm.hip.out_dim) == (tp.weight_numel, tp.irreps_in1.dim, tp.irreps_out.dim)
+    empty = o3.TensorProduct("0x0e", "0e", "0e", [(0, 0, 0, "uvw", True)])
+    assert provider.hip_provider(empty.irreps_in1, empty.irreps_in2, empty.irreps_out, empty.instructions, True, True, True) is None
+    hooks = ["einsum code generator"]
+    provider.register(hooks)
+    provider.register(hooks)
+    assert hooks == [provider.hip_provider, "einsum code generator"]
