@@ -287,6 +287,22 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only 
   // - 2 % on the 128-channel l <= 3 set in fp32, whose operands alone take ~150 registers.
   const bool loads_first = P.dtype == E3X_BF16 || upl * (accregs + x1regs + wregs) + (int)P.in2_dim <= 140;
   if (env_int("E3X_UVU_SCHED", loads_first ? 1 : 0) == 0) s << "#define E3X_UVU_SCHED 0\n";
+  // The source row through LDS (see fetch_x1 / stage_x1 in the template): when a lane owns several indices of irreps
+  // with d > 1, whose runs make the direct 16-byte loads touch d lines per lane group.  Needs whole 16-byte pieces.
+  {
+    const int epp = P.dtype == E3X_BF16 ? 8 : 4;
+    bool whole = !bwd_only && !tpl && !prefetch && upl * (P.dtype == E3X_BF16 ? 2 : 4) % 16 == 0 && P.in1_dim % (epp * K.lanes) == 0;
+    bool wide = false;
+    for (size_t a = 0; a < P.in1.size(); ++a) {
+      const int d = 2 * P.in1[a].l + 1;
+      if (!used1[a] && P.in1[a].mul > 0) whole = false;  // split kernels gather only their own slice of the row
+      if (used1[a] && (P.off1[a] % epp || (upl * d) % epp || P.in1[a].mul % upl || P.in1[a].mul > K.lanes * upl * K.chunks)) whole = false;
+      wide = wide || (used1[a] && d > 1);
+    }
+    const long long lds = (long long)K.waves_per_block * (64 / K.lanes) * P.in1_dim * (P.dtype == E3X_BF16 ? 2 : 4);
+    if (env_int("E3X_UVU_X1_LDS", (whole && wide && K.chunks == 1 && lds <= 49152) ? 1 : 0) && whole && K.chunks == 1 && lds <= 65536)
+      s << "#define E3X_UVU_X1_LDS 1\n";
+  }
   if (extra_cfg) s << *extra_cfg;
   s << "}  // namespace cfg\n";
   *src = s.str() + e3x::kTplCommon + (tpl ? tpl : e3x::kTplUvu);
