@@ -72,6 +72,17 @@ __global__ __launch_bounds__(kBlock) void range_kernel(const IdxT* __restrict__ 
   if (bad) atomicOr(&flags[0], 1);
 }
 
+// src_rows[k] = source row of the edge at position k of the destination-sorted list, negative values wrapped
+template <typename IdxT>
+__global__ __launch_bounds__(kBlock) void src_rows_kernel(const IdxT* __restrict__ src, const int* __restrict__ perm,
+                                                          long long E, long long n_src, int* __restrict__ src_rows) {
+  for (long long k = (long long)blockIdx.x * kBlock + threadIdx.x; k < E; k += (long long)gridDim.x * kBlock) {
+    long long s = (long long)src[perm ? perm[k] : k];
+    if (s < 0) s += n_src;
+    src_rows[k] = (int)s;
+  }
+}
+
 // rowptr[n] = first position k with sorted_key[k] >= n   (n = 0..N)
 __global__ __launch_bounds__(kBlock) void rowptr_kernel(const unsigned* __restrict__ sorted, long long E,
                                                         long long N, int* __restrict__ rowptr) {
@@ -336,6 +347,23 @@ extern "C" int e3x_row_order_build(const void* src, int idx_bits, const int32_t*
       return e3x::fail(E3X_ERR_HIP, "e3x_row_order_build: reading back the score failed");
   }
   return E3X_OK;
+}
+
+extern "C" int e3x_src_rows_build(const void* src, int idx_bits, const int32_t* perm, int64_t E, int64_t num_src_nodes,
+                                   int32_t* src_rows, void* stream) {
+  if (idx_bits != 32 && idx_bits != 64) return e3x::fail(E3X_ERR_INVALID, "e3x_src_rows_build: idx_bits must be 32 or 64");
+  if (E < 0 || num_src_nodes < 0 || num_src_nodes >= (1LL << 31))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_src_rows_build: sizes must be in [0, 2^31)");
+  if (E == 0) return E3X_OK;
+  if (!src || !src_rows) return e3x::fail(E3X_ERR_INVALID, "e3x_src_rows_build: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  if (idx_bits == 64)
+    hipLaunchKernelGGL((src_rows_kernel<long long>), dim3(grid_for(E, kBlock)), dim3(kBlock), 0, st,
+                       (const long long*)src, perm, (long long)E, (long long)num_src_nodes, src_rows);
+  else
+    hipLaunchKernelGGL((src_rows_kernel<int>), dim3(grid_for(E, kBlock)), dim3(kBlock), 0, st, (const int*)src, perm,
+                       (long long)E, (long long)num_src_nodes, src_rows);
+  return hipGetLastError() == hipSuccess ? E3X_OK : e3x::fail(E3X_ERR_HIP, "e3x_src_rows_build: launch failed");
 }
 
 extern "C" int e3x_index_check(const void* idx, int idx_bits, int64_t E, int64_t num_nodes, void* stream) {

@@ -281,7 +281,8 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only 
   // coefficient folded into the edge attribute (see accumulate_edge); measured on one GPU, old -> new: 32 channels
   // l <= 2 at four indices per lane 0.637 -> 0.635 ms (degree 354: 4.91 -> 4.84), 128 channels l <= 3 in bf16 storage
   // 1.60 -> 1.48 ms, in fp32 at two indices per lane 1.68 -> 1.77 ms
-  if (env_int("E3X_UVU_FOLD", (upl == 4 || P.dtype == E3X_BF16) ? 1 : 0)) s << "#define E3X_UVU_FOLD 1\n";
+  const bool fold = env_int("E3X_UVU_FOLD", (upl == 4 || P.dtype == E3X_BF16) ? 1 : 0) != 0;
+  if (fold) s << "#define E3X_UVU_FOLD 1\n";
   // All loads of an edge ahead of its first product (a scheduling barrier in the edge loop) while the operands of an
   // edge leave room for three waves per SIMD; measured: + 3 % on the 32-channel l <= 2 set, + 13 % in bf16 storage,
   // - 2 % on the 128-channel l <= 3 set in fp32, whose operands alone take ~150 registers.
@@ -302,6 +303,19 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only 
     const long long lds = (long long)K.waves_per_block * (64 / K.lanes) * P.in1_dim * (P.dtype == E3X_BF16 ? 2 : 4);
     if (env_int("E3X_UVU_X1_LDS", (whole && wide && K.chunks == 1 && lds <= 49152) ? 1 : 0) && whole && K.chunks == 1 && lds <= 65536)
       s << "#define E3X_UVU_X1_LDS 1\n";
+  }
+  // The partial sums of the lane groups combined through LDS and the row stored as whole 16-byte pieces (see
+  // reduce_store_row in the template): fp32, four indices per lane, several groups per wavefront, and a kernel that
+  // owns the whole output row.  Measured on the 32-channel l <= 2 set: the shuffle butterfly and the 128-byte stores
+  // it replaces were 15 % of the kernel.
+  {
+    bool ok = !bwd_only && !tpl && P.dtype == E3X_F32 && upl == 4 && K.lanes < 64 && K.chunks == 1 && P.out_dim % 4 == 0;
+    for (size_t c = 0; c < P.out.size(); ++c) {
+      if (P.out[c].mul == 0) continue;
+      if (!usedo[c] || P.offo[c] % 4 || P.out[c].mul % 4 || P.out[c].mul > K.lanes * upl) ok = false;
+    }
+    const long long lds = (long long)K.waves_per_block * (64 / K.lanes) * P.out_dim * 4;
+    if (ok && lds <= 49152 && env_int("E3X_UVU_LDS_REDUCE", 1)) s << "#define E3X_UVU_LDS_REDUCE 1\n";
   }
   if (extra_cfg) s << *extra_cfg;
   s << "}  // namespace cfg\n";
@@ -1101,8 +1115,8 @@ extern "C" int e3x_tp_gather_scatter_ordered(e3x_plan* P, const void* node_x, co
                                              const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
                                              const int32_t* row_order, void* out, int64_t E, int64_t num_src_nodes,
                                              int64_t num_out_nodes, void* stream) {
-  return e3x_tp_gather_scatter_ws(P, node_x, edge_attr, w, src, idx_bits, rowptr, perm, row_order, out, E, num_src_nodes,
-                                  num_out_nodes, nullptr, 0, stream);
+  return e3x_tp_gather_scatter_ws(P, node_x, edge_attr, w, src, idx_bits, rowptr, perm, row_order, nullptr, out, E,
+                                  num_src_nodes, num_out_nodes, nullptr, 0, stream);
 }
 
 extern "C" size_t e3x_tp_gather_scatter_workspace_bytes(const e3x_plan* P, int64_t num_src_nodes) {
@@ -1112,8 +1126,9 @@ extern "C" size_t e3x_tp_gather_scatter_workspace_bytes(const e3x_plan* P, int64
 
 extern "C" int e3x_tp_gather_scatter_ws(e3x_plan* P, const void* node_x, const void* edge_attr, const void* w,
                                         const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
-                                        const int32_t* row_order, void* out, int64_t E, int64_t num_src_nodes,
-                                        int64_t num_out_nodes, void* workspace, size_t workspace_bytes, void* stream) {
+                                        const int32_t* row_order, const int32_t* src_rows, void* out, int64_t E,
+                                        int64_t num_src_nodes, int64_t num_out_nodes, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: null plan");
   if (P->family != "uvu") return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: the plan must be all-uvu");
   if (P->shared_weights && P->weight_numel)
@@ -1131,7 +1146,12 @@ extern "C" int e3x_tp_gather_scatter_ws(e3x_plan* P, const void* node_x, const v
     if (P->paths.empty()) return E3X_OK;
   }
   if ((rc = load_functions(P, dev))) return rc;
+  // index mode of the kernels: 0 / 1 = the caller's int32 / int64 list indexed by edge id, 2 = src_rows
   int idx64 = idx_bits == 64;
+  if (src_rows) {
+    src = src_rows;
+    idx64 = 2;
+  }
   long long n_rows = num_out_nodes, n_src = num_src_nodes;
   void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&w,         (void*)&out,    (void*)&src,  (void*)&idx64,
                   (void*)&rowptr, (void*)&perm,      (void*)&row_order, (void*)&n_rows, (void*)&n_src};

@@ -7,6 +7,7 @@ edges of each destination to be contiguous: ``DstSortedEdges`` validates both in
 arrays once and builds the row pointers and the stable permutation on the GPU.
 """
 import ctypes
+import os
 
 import torch
 
@@ -39,9 +40,28 @@ class DstSortedEdges:
             self._transposed._transposed = self
         return self._transposed
 
+    @property
+    def src_rows(self) -> torch.Tensor:
+        """``edge_src`` in the order of the destination-sorted list (int32, negative values wrapped): the fused
+        kernels read it sequentially, where ``edge_src[perm[k]]`` costs them a cache line per edge.  Built on first
+        use, once per graph."""
+        if self._src_rows is None and self.num_edges > 0 and os.environ.get("E3X_SRC_ROWS", "1") != "0":
+            dev = self.edge_src.device
+            rows = torch.empty(self.num_edges, dtype=torch.int32, device=dev)
+            with torch.cuda.device(dev):
+                _lib.check(
+                    _lib.lib().e3x_src_rows_build(
+                        _lib.ptr(self.edge_src), self.edge_src.element_size() * 8, _lib.ptr(self.perm), self.num_edges,
+                        self.num_src_nodes, _lib.ptr(rows), _lib.stream_ptr(dev),
+                    )  # fmt: skip
+                )
+            self._src_rows = rows
+        return self._src_rows
+
     def __init__(self, edge_src: torch.Tensor, edge_dst: torch.Tensor, num_nodes: int, num_src_nodes: int = None,
                  locality_order="auto"):
         self._transposed = None
+        self._src_rows = None
         self._locality_order = locality_order
         if not (edge_src.is_cuda and edge_dst.is_cuda):
             raise RuntimeError("DstSortedEdges needs index tensors on the GPU")

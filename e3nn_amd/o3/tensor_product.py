@@ -124,6 +124,7 @@ class _Plan:
                 L.e3x_tp_gather_scatter_ws(
                     self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(gather_idx),
                     gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(edges.row_order),
+                    _lib.ptr(edges.src_rows if gather_idx is edges.edge_src else None),
                     _lib.ptr(out), edges.num_edges, num_table_rows, edges.num_nodes, _lib.ptr(ws), ws_bytes,
                     _lib.stream_ptr(table.device),
                 )  # fmt: skip

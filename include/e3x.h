@@ -223,10 +223,19 @@ int e3x_tp_gather_scatter_ordered(e3x_plan* plan, const void* node_x, const void
  * kernels).  Every other plan needs no workspace (the function returns 0) and runs as e3x_tp_gather_scatter_ordered;
  * so does a call without workspace. */
 size_t e3x_tp_gather_scatter_workspace_bytes(const e3x_plan* plan, int64_t num_src_nodes);
+/* `src_rows` (may be NULL): the source rows in the order of the destination-sorted list, as e3x_src_rows_build writes
+ * them; the kernels then read it in place of `src` (which is still required).  Results are bit-identical. */
 int e3x_tp_gather_scatter_ws(e3x_plan* plan, const void* node_x, const void* edge_attr, const void* w, const void* src,
                              int idx_bits, const int32_t* rowptr, const int32_t* perm, const int32_t* row_order,
-                             void* out, int64_t E, int64_t num_src_nodes, int64_t num_out_nodes, void* workspace,
-                             size_t workspace_bytes, void* stream);
+                             const int32_t* src_rows, void* out, int64_t E, int64_t num_src_nodes,
+                             int64_t num_out_nodes, void* workspace, size_t workspace_bytes, void* stream);
+/* src_rows[k] = src[perm[k]] (perm NULL: src[k]) as int32, negative values wrapped by num_src_nodes: the gather
+ * indices of x[edge_src] (points_convolution.py:105) laid out in the order the fused kernels walk the edges.  Read
+ * through `perm`, an index costs the kernels a cache line of its own per edge; this list is read sequentially.  It
+ * depends on the graph only (built once per edge list, E * 4 bytes, caller-owned).  Indices must have been
+ * validated (e3x_index_check). */
+int e3x_src_rows_build(const void* src, int idx_bits, const int32_t* perm, int64_t E, int64_t num_src_nodes,
+                       int32_t* src_rows, void* stream);
 
 /* Gradients of the `uvu` product (plain: src = dst = NULL, row e of every table; fused: the edge lists
  * of e3x_tp_gather_scatter, unsorted) with respect to the per-sample weights and the second input:

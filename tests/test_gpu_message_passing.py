@@ -217,6 +217,40 @@ def test_fused_bf16_storage(variant, N, E, idx):
     assert (plain.float() - out.float()).abs().max().item() <= 1e-2 * scale / 2
 
 
+@pytest.mark.parametrize("idx", [torch.int32, torch.int64])
+def test_source_rows_in_sorted_order(idx):
+    # e3x_src_rows_build: the gather indices laid out in the order of the destination-sorted list, negative values
+    # wrapped; the message kernels (vector-ALU fp32, matrix-core bf16) give the same bits with and without the list
+    from e3nn_amd import _lib
+
+    N, E = 90, 4000
+    src, dst = random_graph(N, E, seed=21, dtype=idx)
+    src = torch.where(src % 3 == 0, src - N, src)  # a third of the sources as negative indices
+    edges = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    rows = edges.src_rows
+    assert rows.dtype == torch.int32 and rows.shape == (E,)
+    assert torch.equal(rows.cpu().long(), (src.long() % N)[edges.perm.cpu().long()])
+    L, st = _lib.lib(), _lib.stream_ptr(torch.device(DEV))
+    for tp, dtype, width in ((ks.cfg3(), torch.float32, 288), (ks.cfg4("A"), torch.bfloat16, 2048)):
+        plan = tp._plan(dtype)
+        node_x, attr, w = (seeded(n, d, seed=i).to(DEV).to(dtype) for i, (n, d) in
+                           enumerate(((N, width), (E, tp.irreps_in2.dim), (E, tp.weight_numel))))
+        outs = []
+        with torch.cuda.device(DEV):
+            ws_bytes = L.e3x_tp_gather_scatter_workspace_bytes(plan.handle, N)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=DEV)
+            s_d = edges.edge_src
+            for src_rows in (None, rows):
+                out = torch.empty(N, tp.irreps_out.dim, dtype=dtype, device=DEV)
+                _lib.check(L.e3x_tp_gather_scatter_ws(
+                    plan.handle, _lib.ptr(node_x), _lib.ptr(attr), _lib.ptr(w), _lib.ptr(s_d), s_d.element_size() * 8,
+                    _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), None, _lib.ptr(src_rows), _lib.ptr(out), E, N, N,
+                    _lib.ptr(ws) if ws_bytes else None, ws_bytes, st))  # fmt: skip
+                outs.append(out)
+        assert torch.equal(outs[0], outs[1])
+        assert torch.equal(tp.forward_gather_scatter(node_x, attr, w, edges=edges), outs[0])
+
+
 @pytest.mark.parametrize("case,N,E,idx", [
     ("nequip_silu", 400, 9_000, torch.int64), ("nequip_silu", 30, 3, torch.int32), ("nequip_silu", 5, 4_000, torch.int64),
     ("small_tanh", 200, 5_001, torch.int32), ("small_linear", 64, 777, torch.int64),
