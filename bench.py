@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt), keyed by the code object the counters were read
 # on: a kernel that has changed since reports no traffic instead of a stale figure.
 NEQUIP_TRAFFIC_BYTES = {
-    "uvu_77a1034ede7bf763fa3ae452": (3374122 + 56251) * 1024,  # 3374122 KiB fetched + 56251 KiB written
+    "uvu_c81958e38ae94d0c80d6d6a3": (2 * 1611962 + 56250) * 1024,  # FETCH_SIZE 1611962 x 2 KiB + WRITE_SIZE 56250 KiB
 }
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
@@ -80,6 +80,27 @@ def bench_copy(args, dev):
     ms = event_time_ms(step, max(3, args.steps // 5), 2)
     assert torch.equal(a[:4096], b[:4096])
     return {"bytes_read": n, "bytes_written": n, "ms": ms, "gbs": 2 * n / (ms * 1e-3) / 1e9}
+
+
+def bench_stream_rows(args, dev, n_rows, bytes_total, out_row_bytes):
+    """What this chip sustains on the memory traffic of the headline kernel alone: one wavefront per destination row
+    streams the row's share of the per-edge bytes (no gather, no arithmetic) and, in the second run, writes an
+    output row of the same size as the kernel's.  `bytes_total` is the headline's algorithmic byte count."""
+    from e3nn_amd import _lib
+
+    in_row = (bytes_total - n_rows * out_row_bytes) // n_rows // 16 * 16
+    a = torch.empty(n_rows * in_row, dtype=torch.uint8, device=dev).random_(0, 255)
+    b = torch.empty(n_rows * out_row_bytes, dtype=torch.uint8, device=dev)
+    L = _lib.lib()
+    res = {"rows": n_rows, "bytes_read_per_row": in_row, "bytes_written_per_row": out_row_bytes}
+    for name, out_bytes in (("read_only", 0), ("read_and_row_stores", out_row_bytes)):
+        def step():
+            _lib.check(L.e3x_stream_rows(_lib.ptr(a), in_row, n_rows, _lib.ptr(b), out_bytes, _lib.stream_ptr(dev)))
+
+        ms = event_time_ms(step, max(3, args.steps // 5), 2)
+        moved = n_rows * (in_row + out_bytes)
+        res[name] = {"ms": ms, "gbs": moved / (ms * 1e-3) / 1e9}
+    return res
 
 
 def radius_graph(n, side, cutoff, seed=0):
@@ -468,6 +489,7 @@ def main():
     want = set(args.only.split(",")) if args.only else {"copy", "sh", "mace", "mace_b", "mace_bf16", "nequip40", "uvw", "uvw_bf16", "conv", "radial", "nequip_bwd", "uvw_bwd"}
     if "copy" in want:
         other["copy_1GiB"] = bench_copy(args, dev)
+        other["stream_rows_headline_bytes"] = bench_stream_rows(args, dev, neq["nodes"], neq["bytes_per_launch"], 4 * ctx["tp"].irreps_out.dim)
     if "sh" in want:
         other["sh_lmax3_4M"] = bench_sh(args, dev)
     if "mace" in want:
@@ -516,8 +538,10 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": neq["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": neq["achieved_gbs"] / HBM_PEAK_GBS, "traffic": NEQUIP_TRAFFIC_BYTES.get(neq["kernel_key"]), "kernel": "e3x_uvu_fused",
+            "frac": neq["achieved_gbs"] / HBM_PEAK_GBS, "traffic": NEQUIP_TRAFFIC_BYTES.get(neq["kernel_key"].split("+")[0]), "kernel": "e3x_uvu_fused",
             "algorithmic_bytes": neq["bytes_per_launch"],
+            # the same bytes streamed by a kernel that does nothing else (e3x_stream_rows), measured in this run
+            "stream_same_bytes_gbs": other.get("stream_rows_headline_bytes", {}).get("read_and_row_stores", {}).get("gbs"),
         },
         "other": other,
     }  # fmt: skip

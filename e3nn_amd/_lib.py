@@ -90,6 +90,7 @@ _SIGNATURES = {
     "e3x_fc_plan_prepare_backward_w": (c_int, [c_void_p]),
     "e3x_fc_backward_w": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "e3x_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "e3x_stream_rows": (c_int, [c_void_p, c_size_t, c_int64, c_void_p, c_size_t, c_void_p]),
 }  # fmt: skip
 
 _lib = None

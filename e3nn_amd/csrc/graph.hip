@@ -162,6 +162,27 @@ __global__ __launch_bounds__(kBlock) void copy16_kernel(const uint4* __restrict_
   if (i < n16) dst[i] = src[i];
 }
 
+// One wavefront per row: reads the row's in16 16-byte pieces (consecutive rows are stored one after the other) with
+// non-temporal loads, eight 1 KB instructions in flight, folds them with XOR and writes out16 pieces of the fold.
+typedef unsigned stream_u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(kBlock) void stream_rows_kernel(const stream_u32x4* __restrict__ in, long long in16,
+                                                             long long n_rows, stream_u32x4* __restrict__ out, int out16) {
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * (kBlock / 64) + threadIdx.x / 64;
+  if (row >= n_rows) return;
+  const stream_u32x4* p = in + row * in16;
+  stream_u32x4 acc = {0u, 0u, 0u, 0u};
+  for (long long i = lane; i < in16; i += 64 * 8) {
+    stream_u32x4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      v[k] = i + 64 * k < in16 ? __builtin_nontemporal_load(p + i + 64 * k) : stream_u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc ^= v[k];
+  }
+  for (int q = lane; q < out16; q += 64) out[row * out16 + q] = acc;
+}
+
 __global__ __launch_bounds__(kBlock) void fill_zero_bytes_kernel(unsigned char* p, size_t n) {
   // 16-byte stores over the aligned middle, byte stores at the ragged ends
   const size_t head = (16 - ((uintptr_t)p & 15)) & 15;
@@ -400,4 +421,19 @@ extern "C" int e3x_copy_bytes(const void* src, void* dst, size_t n_bytes, void* 
   hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, (hipStream_t)stream, (const uint4*)src,
                      (uint4*)dst, n_bytes / 16);
   return hipGetLastError() == hipSuccess ? E3X_OK : e3x::fail(E3X_ERR_HIP, "e3x_copy_bytes: launch failed");
+}
+
+extern "C" int e3x_stream_rows(const void* in, size_t in_bytes_per_row, int64_t n_rows, void* out, size_t out_bytes_per_row,
+                               void* stream) {
+  if (in_bytes_per_row % 16 || out_bytes_per_row % 16 || ((uintptr_t)in % 16) || ((uintptr_t)out % 16) || n_rows < 0 ||
+      out_bytes_per_row > (1u << 20))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_stream_rows: sizes and pointers must be multiples of 16, rows of output at most 1 MiB");
+  if (n_rows == 0) return E3X_OK;
+  if (!in || (out_bytes_per_row && !out)) return e3x::fail(E3X_ERR_INVALID, "e3x_stream_rows: null pointer");
+  const int64_t blocks = (n_rows + kBlock / 64 - 1) / (kBlock / 64);
+  if (blocks > 0x7fffffffLL) return e3x::fail(E3X_ERR_INVALID, "e3x_stream_rows: too many rows for one launch");
+  hipLaunchKernelGGL(stream_rows_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, (hipStream_t)stream,
+                     (const stream_u32x4*)in, (long long)(in_bytes_per_row / 16), (long long)n_rows, (stream_u32x4*)out,
+                     (int)(out_bytes_per_row / 16));
+  return hipGetLastError() == hipSuccess ? E3X_OK : e3x::fail(E3X_ERR_HIP, "e3x_stream_rows: launch failed");
 }

@@ -331,6 +331,14 @@ int e3x_fc_backward_w(e3x_fc_plan* plan, const void* x, const void* grad_out, vo
 /* Plain device copy dst[i] = src[i], n_bytes multiple of 16: the calibration kernel
  * for bandwidth counters (known traffic: n_bytes read + n_bytes written). */
 int e3x_copy_bytes(const void* src, void* dst, size_t n_bytes, void* stream);
+/* The memory traffic of a fused message kernel without its arithmetic and without its gather: one wavefront per row
+ * reads in_bytes_per_row consecutive bytes (row r at in + r * in_bytes_per_row, non-temporal 16-byte loads) and
+ * writes out_bytes_per_row bytes (row r at out + r * out_bytes_per_row; 0: nothing is written).  Sizes are multiples
+ * of 16.  No counterpart in the reference: a calibration kernel like e3x_copy_bytes, for the rate this chip sustains
+ * on a read stream that carries a few per cent of row-sized writes (it is well below the rate of the read stream
+ * alone), against which the message kernels are to be read. */
+int e3x_stream_rows(const void* in, size_t in_bytes_per_row, int64_t n_rows, void* out, size_t out_bytes_per_row,
+                    void* stream);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop
