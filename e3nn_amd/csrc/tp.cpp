@@ -581,6 +581,8 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
     }
   }
   s << "constexpr int WT = " << wt << ", KMAX = " << kmax << ";\n";  // KMAX: the largest GEMM K extent
+  for (const char* knob : {"E3X_UVW16_OS", "E3X_UVW16_NBUF", "E3X_UVW16_LEAD"})
+    if (P.dtype == E3X_BF16 && std::getenv(knob)) s << "#define " << knob << " " << env_int(knob, 0) << "\n";
   s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
     << nzs.str() << "};\n";
   s << "constexpr int DKA = " << dka << ", DRMAX = " << drmax << ";\n";
