@@ -177,9 +177,9 @@ int e3x_tp_gather_scatter(e3x_plan* plan, const void* node_x, const void* edge_a
  * w2 [n_hidden, weight_numel] are the reference's layer0.weight / layer1.weight, edge_scalars [E, n_in].
  * For fp32 all-uvu plans with per-edge weights on every instruction, multiplicity 32 on the first input and the
  * output and 1 on the second, n_hidden a multiple of 16 (E3X_ERR_INVALID otherwise: run the network and
- * e3x_tp_gather_scatter instead).  `out` is fully overwritten.  Rows whose edges straddle the ranges of two of the
- * kernel's workers are summed with fp32 atomics: their last bits may differ between runs, all others are
- * reproducible.  The kernel is built on first use (one per network shape). */
+ * e3x_tp_gather_scatter instead).  `out` is fully overwritten.  Every row is summed in the order of the sorted
+ * edge list by one worker of the kernel: results are bit-reproducible.  The kernel is built on first use (one per
+ * network shape). */
 int e3x_tp_gather_scatter_radial(e3x_plan* plan, const void* node_x, const void* edge_attr, const void* edge_scalars,
                                  const void* w1, const void* w2, int32_t n_in, int32_t n_hidden, int32_t act,
                                  double act_cst, double variance_in, double variance_out, const void* src, int idx_bits,

@@ -282,10 +282,9 @@ def test_message_with_the_radial_network_inside(case, N, E, idx):
     with torch.no_grad():
         two = tp.forward_gather_scatter(node_x.to(DEV), attr, net(scalars.to(DEV)), edges=edges)
     assert (out - two).abs().max().item() < 1e-4 * scale
-    # rows that lie inside one worker's range are summed in a fixed order: a second run differs at most in the rows
-    # that straddle two ranges (fp32 atomics), and there only in the last bits
-    again = tp.forward_gather_scatter_radial(node_x.to(DEV), attr, scalars.to(DEV), net, edges)
-    assert (out - again).abs().max().item() <= 1e-5 * scale
+    # every row is summed by one worker of the kernel in the order of the sorted edge list: reruns give the same bits
+    for _ in range(3):
+        assert torch.equal(tp.forward_gather_scatter_radial(node_x.to(DEV), attr, scalars.to(DEV), net, edges), out)
 
 
 def test_message_with_the_radial_network_declines_what_it_does_not_take():
