@@ -300,3 +300,30 @@ def test_message_with_the_radial_network_declines_what_it_does_not_take():
     other_mul = ks.cfg4("A")  # multiplicities other than 32
     net = nn.FullyConnectedNet([8, 16, other_mul.weight_numel], torch.tanh).to(DEV)
     assert not other_mul.prepare_gather_scatter_radial(net)
+
+
+def test_calibration_kernels_move_the_bytes_they_claim():
+    # e3x_copy_bytes and e3x_stream_rows are what the profiler counters and the bandwidth figures are scaled by:
+    # the copy is exact, the row streamer writes the XOR of the 16-byte pieces of a row, lane by lane
+    from e3nn_amd import _lib
+
+    L, st = _lib.lib(), _lib.stream_ptr(torch.device(DEV))
+    g = torch.Generator().manual_seed(3)
+    a = torch.randint(0, 2**31 - 1, (4096 + 5 * 4,), generator=g, dtype=torch.int32).to(DEV)
+    b = torch.zeros_like(a)
+    with torch.cuda.device(DEV):
+        _lib.check(L.e3x_copy_bytes(_lib.ptr(a), _lib.ptr(b), a.numel() * 4, st))
+    assert torch.equal(a, b)
+    rows, pieces_in, pieces_out = 7, 150, 70  # ragged against the 64 lanes and the 8 loads in flight
+    x = torch.randint(0, 2**31 - 1, (rows, pieces_in, 4), generator=g, dtype=torch.int32).to(DEV)
+    out = torch.zeros(rows, pieces_out, 4, dtype=torch.int32, device=DEV)
+    with torch.cuda.device(DEV):
+        _lib.check(L.e3x_stream_rows(_lib.ptr(x), pieces_in * 16, rows, _lib.ptr(out), pieces_out * 16, st))
+    fold = torch.zeros(rows, 64, 4, dtype=torch.int32)
+    xc = x.cpu()
+    for i in range(pieces_in):
+        fold[:, i % 64] ^= xc[:, i]
+    assert torch.equal(out.cpu(), fold[:, torch.arange(pieces_out) % 64])
+    with pytest.raises(RuntimeError):
+        with torch.cuda.device(DEV):
+            _lib.check(L.e3x_stream_rows(_lib.ptr(x), 24, rows, _lib.ptr(out), 16, st))
