@@ -703,6 +703,7 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
   std::ostringstream s, nzs, ps;
   emit_header(s, P);
   if (env_int("E3X_DW_ZC", 0)) s << "#define E3X_DW_ZC " << env_int("E3X_DW_ZC", 0) << "\n";
+  if (std::getenv("E3X_DW_SYNTH")) s << "#define E3X_DW_SYNTH " << env_int("E3X_DW_SYNTH", 1) << "\n";
   int n_nz = 0, n_path = 0, dkmax = 1, drmax = 1;
   long long tiles = 0;
   if (!mfma_dw_fits(P))
