@@ -42,8 +42,9 @@ class Linear(torch.nn.Module):
     ) -> None:
         super().__init__()
         assert path_normalization in ["element", "path"]
-        if f_in is not None or f_out is not None:
-            raise NotImplementedError("Linear: f_in / f_out have no kernel")
+        if (f_in is None) != (f_out is None):
+            raise ValueError("Linear: f_in and f_out come together")
+        self.f_in, self.f_out = f_in, f_out
         irreps_in, irreps_out = Irreps(irreps_in), Irreps(irreps_out)
         if instructions is None:
             instructions = [
@@ -62,6 +63,7 @@ class Linear(torch.nn.Module):
 
         def alpha(i_in, i_out) -> float:
             x = sum(irreps_in[a if path_normalization == "element" else i_in].mul for a, b in instructions if b == i_out)
+            x *= 1 if f_in is None else f_in  # every input channel feeds every output channel (_linear.py:158-159)
             return 1.0 if x == 0 else x
 
         self.instructions = [
@@ -92,21 +94,38 @@ class Linear(torch.nn.Module):
         # the same map as a tensor product with "0e": the reference's own normalisation formula for TensorProduct
         # (component / element or path) reproduces alpha^(-1/2) once the delta / sqrt(2l+1) of the 3j tensor is counted
         # (kept out of the module tree: the reference's Linear has no such submodule in its state_dict)
+        # With f_in / f_out the features are [..., f_in, irreps_in.dim] -> [..., f_out, irreps_out.dim] and the weights
+        # [f_in, f_out, weight_numel] (_linear.py:226, :445-448): the same product on f_in * mul copies of every input
+        # irrep and f_out * mul copies of every output irrep, once the columns are regrouped irrep by irrep.
+        fi, fo = (1, 1) if f_in is None else (f_in, f_out)
+        wide_in = Irreps([(fi * mul, ir) for mul, ir in irreps_in])
+        wide_out = Irreps([(fo * mul, ir) for mul, ir in irreps_out])
         object.__setattr__(self, "_tp", TensorProduct(
-            irreps_in, "0e", irreps_out, [(i, 0, o, "uvw", True) for i, o in instructions],
+            wide_in, "0e", wide_out, [(i, 0, o, "uvw", True) for i, o in instructions],
             path_normalization=path_normalization, internal_weights=False, shared_weights=shared_weights,
         ))  # fmt: skip
-        self.weight_numel = self._tp.weight_numel
+        if f_in is not None:
+            def regroup(irreps, f):  # position in the wide row -> position in the flattened [f, irreps.dim] features
+                cols = [c * irreps.dim + sl.start + j for sl in irreps.slices() for c in range(f) for j in range(sl.stop - sl.start)]
+                return torch.tensor(cols, dtype=torch.long)
+
+            self.register_buffer("_cols_in", regroup(irreps_in, f_in), persistent=False)
+            cols_out = regroup(irreps_out, f_out)
+            self.register_buffer("_cols_out", torch.argsort(cols_out), persistent=False)
+        self.weight_numel = self._tp.weight_numel // (fi * fo)
         self.bias_numel = sum(sl.stop - sl.start for sl in self._bias_slices)
         if internal_weights and self.weight_numel > 0:
-            self.weight = torch.nn.Parameter(torch.randn(self.weight_numel))
+            self.weight = torch.nn.Parameter(torch.randn(*(() if f_in is None else (f_in, f_out)), self.weight_numel))
         else:
             self.register_buffer("weight", torch.Tensor())
         if internal_weights and self.bias_numel > 0:
-            self.bias = torch.nn.Parameter(torch.zeros(self.bias_numel))
+            self.bias = torch.nn.Parameter(torch.zeros(*(() if f_out is None else (f_out,)), self.bias_numel))
         else:
             self.register_buffer("bias", torch.Tensor())
-        self.register_buffer("output_mask", self._tp.output_mask.clone())
+        mask = self._tp.output_mask.clone()
+        if f_in is not None:  # the reference's mask is that of one output channel
+            mask = torch.cat([mask[f_out * sl.start : f_out * sl.start + (sl.stop - sl.start)] for sl in irreps_out.slices()]) if len(irreps_out) else mask[:0]
+        self.register_buffer("output_mask", mask)
 
     def __repr__(self) -> str:
         return f"{self.__class__.__name__}({self.irreps_in} -> {self.irreps_out} | {self.weight_numel} weights)"
@@ -120,8 +139,34 @@ class Linear(torch.nn.Module):
             if self.bias_numel > 0 and not self.internal_weights:
                 raise RuntimeError("Biases must be provided when internal_weights = False")
             bias = self.bias
+        if self.f_in is not None:
+            return self._forward_channels(features, weight, bias)
         ones = features.new_ones(features.shape[:-1] + (1,))
         out = self._tp(features, ones, weight)
+        if self.bias_numel > 0:
+            off = 0
+            out = out.clone()
+            for sl in self._bias_slices:
+                n = sl.stop - sl.start
+                out[..., sl] += bias[..., off : off + n]
+                off += n
+        return out
+
+    def _forward_channels(self, features, weight, bias):
+        f_in, f_out = self.f_in, self.f_out
+        lead = features.shape[:-2]
+        x = features.reshape(*lead, f_in * self.irreps_in.dim)[..., self._cols_in]
+        # weights [..., f_in, f_out, numel] -> per instruction [f_in * U, f_out * W], row-major, instruction after instruction
+        blocks, off = [], 0
+        for ins in self.instructions:
+            if ins.i_in == -1:
+                continue
+            U, W = ins.path_shape
+            blk = weight[..., off : off + U * W].reshape(*weight.shape[:-3], f_in, f_out, U, W)
+            blocks.append(blk.transpose(-3, -2).reshape(*weight.shape[:-3], f_in * U * f_out * W))
+            off += U * W
+        wide_w = torch.cat(blocks, dim=-1) if blocks else weight.new_zeros(*weight.shape[:-3], 0)
+        out = self._tp(x, x.new_ones(*lead, 1), wide_w)[..., self._cols_out].reshape(*lead, f_out, self.irreps_out.dim)
         if self.bias_numel > 0:
             off = 0
             out = out.clone()

@@ -51,6 +51,44 @@ def test_linear_on_the_matrix_cores():
     assert float((lin.weight.grad.cpu().double().numpy() * dw).sum()) == pytest.approx(fd, rel=2e-4)
 
 
+@pytest.mark.parametrize("norm", ["element", "path"])
+def test_linear_with_input_and_output_channels(norm):
+    # f_in / f_out (e3nn/o3/_linear.py:117-118): features [..., f_in, irreps_in.dim] -> [..., f_out, irreps_out.dim], weights
+    # [f_in, f_out, weight_numel], every path weight 1 / sqrt(f_in * fan-in) (:152-161), einsum "xyuw,zxui->zywi" (:448);
+    # checked against that einsum written out in float64
+    f_in, f_out = 3, 2
+    irreps_in, irreps_out = o3.Irreps("4x0e+3x1o+2x0e"), o3.Irreps("5x0e+2x1o")
+    lin = o3.Linear(irreps_in, irreps_out, f_in=f_in, f_out=f_out, biases=True, path_normalization=norm).to(DEV)
+    assert lin.weight.shape == (f_in, f_out, lin.weight_numel) and lin.bias.shape == (f_out, 5)
+    assert lin.weight_numel == 4 * 5 + 2 * 5 + 3 * 2 and lin.output_mask.shape == (irreps_out.dim,) and bool(lin.output_mask.all())
+    with torch.no_grad():
+        lin.bias.copy_(seeded(f_out, 5, seed=3))
+    x = seeded(7 * f_in, irreps_in.dim, seed=1).reshape(7, f_in, irreps_in.dim)
+    w = lin.weight.detach().cpu().double().numpy()
+    xs, ref = x.double().numpy(), np.zeros((7, f_out, irreps_out.dim))
+    off = 0
+    for ins in lin.instructions:
+        if ins.i_in == -1:
+            continue
+        U, W = ins.path_shape
+        sl_in, sl_out = irreps_in.slices()[ins.i_in], irreps_out.slices()[ins.i_out]
+        d = irreps_in[ins.i_in].ir.dim
+        fan = sum(irreps_in[i.i_in if norm == "element" else ins.i_in].mul for i in lin.instructions if i.i_in != -1 and i.i_out == ins.i_out)
+        assert ins.path_weight == pytest.approx((f_in * fan) ** -0.5)
+        blk = w[:, :, off : off + U * W].reshape(f_in, f_out, U, W)
+        ref[:, :, sl_out] += ins.path_weight * np.einsum("xyuw,zxui->zywi", blk, xs[:, :, sl_in].reshape(7, f_in, U, d)).reshape(7, f_out, W * d)
+        off += U * W
+    ref[:, :, :5] += lin.bias.detach().cpu().double().numpy()
+    xd = x.to(DEV).requires_grad_(True)
+    out = lin(xd)
+    assert out.shape == (7, f_out, irreps_out.dim)
+    assert_close(out, ref, what=f"Linear f_in f_out {norm}")
+    out.square().sum().backward()  # gradients reach the input and the [f_in, f_out, numel] parameter
+    assert xd.grad.shape == x.shape and lin.weight.grad.shape == lin.weight.shape and bool(lin.weight.grad.abs().sum() > 0)
+    with pytest.raises(ValueError):
+        o3.Linear(irreps_in, irreps_out, f_in=3)
+
+
 def test_activation_and_gate_against_reference_fixtures():
     arr, meta = ks.nn_golden()
     acts = {"silu": torch.nn.functional.silu, "tanh": torch.tanh, "sigmoid": torch.sigmoid, "abs": torch.abs, "relu": torch.relu}
