@@ -204,6 +204,10 @@ def nn_golden():
     return np.load(os.path.join(GOLDEN, "nn_cases.npz")), meta
 
 
+def linear_channels(norm="element"):
+    return o3.Linear("4x0e+3x1o+2x0e", "5x0e+2x1o", f_in=3, f_out=2, biases=True, path_normalization=norm)
+
+
 def nn_modules():
     """(name, module) for the node-wise blocks the GPU tests run; every TensorProduct inside needs its kernels."""
     from e3nn_amd import nn
@@ -216,6 +220,8 @@ def nn_modules():
             m = meta[name]
             out.append((name, o3.Linear(m["irreps_in"], m["irreps_out"], **m["kwargs"])))
     out.append(("linear_wide", o3.Linear("128x0e+128x1o+64x2e", "128x0e+64x1o+32x1o")))
+    for norm in ("element", "path"):  # input and output channels: the product on f_in / f_out copies of every irrep
+        out.append((f"linear_channels_{norm}", linear_channels(norm)))
     if meta is not None:
         out.append(("fc_golden", nn.FullyConnectedNet(meta["fc"]["hs"], torch.nn.functional.silu)))
     out.append(("fc_radial", nn.FullyConnectedNet([8, 64, 352], torch.nn.functional.silu)))

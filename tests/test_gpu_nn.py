@@ -57,8 +57,8 @@ def test_linear_with_input_and_output_channels(norm):
     # [f_in, f_out, weight_numel], every path weight 1 / sqrt(f_in * fan-in) (:152-161), einsum "xyuw,zxui->zywi" (:448);
     # checked against that einsum written out in float64
     f_in, f_out = 3, 2
-    irreps_in, irreps_out = o3.Irreps("4x0e+3x1o+2x0e"), o3.Irreps("5x0e+2x1o")
-    lin = o3.Linear(irreps_in, irreps_out, f_in=f_in, f_out=f_out, biases=True, path_normalization=norm).to(DEV)
+    lin = ks.linear_channels(norm).to(DEV)
+    irreps_in, irreps_out = lin.irreps_in, lin.irreps_out
     assert lin.weight.shape == (f_in, f_out, lin.weight_numel) and lin.bias.shape == (f_out, 5)
     assert lin.weight_numel == 4 * 5 + 2 * 5 + 3 * 2 and lin.output_mask.shape == (irreps_out.dim,) and bool(lin.output_mask.all())
     with torch.no_grad():
