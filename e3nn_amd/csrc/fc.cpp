@@ -210,6 +210,7 @@ extern "C" int e3x_fc_plan_prepare_backward_w(e3x_fc_plan* P) {
   if (const char* v = std::getenv("E3X_FCDW_KU")) s << "#define E3X_FCDW_KU " << std::atoi(v) << "\n";
   if (const char* v = std::getenv("E3X_FCDW_OCC")) s << "#define E3X_FCDW_OCC " << std::atoi(v) << "\n";
   if (const char* v = std::getenv("E3X_FCDW_SPLIT")) s << "#define E3X_FCDW_SPLIT " << std::atoi(v) << "\n";
+  if (const char* v = std::getenv("E3X_FCDW_SHARE")) s << "#define E3X_FCDW_SHARE " << std::atoi(v) << "\n";
   s << "namespace cfg {\n";
   s << "constexpr int H_IN = " << P->hs[0] << ", H_OUT = " << P->hs[1] << ", NTW = " << ntw << ";\n";
   s << "constexpr float SCALE = " << fstr(P->scale0) << ";\n";
