@@ -65,6 +65,11 @@ bool env_split() {
   return !(v && v[0] == '0');
 }
 
+bool env_split_wide() {
+  const char* v = std::getenv("E3X_FC_SPLIT_WIDE");
+  return !(v && v[0] == '0');
+}
+
 int load_functions(e3x_fc_plan* P, int dev) {
   std::lock_guard<std::mutex> lock(P->mu);
   if (P->module[dev]) return E3X_OK;
@@ -119,6 +124,9 @@ extern "C" int e3x_fc_plan_create_fused(const int32_t* hs, int32_t n_hs, int32_t
     std::vector<int> order;
     for (int l = 0; l < NL; ++l)
       if (P->hp[l] % 16 == 0 && P->hp[l] >= 32 && P->hp[l] <= 64 && P->hp[l + 1] >= 128) order.push_back(l);
+    // a last layer from a wide input to at most 64 outputs (the input gradient of the layers above): its input is
+    // split 16 columns at a time inside the loop, so the register cost does not grow with the width
+    if (env_split_wide() && P->hp[NL - 1] % 16 == 0 && P->hp[NL - 1] > 64 && P->hp[NL] <= 64) order.push_back(NL - 1);
     std::sort(order.begin(), order.end(), [&](int a, int b) { return (int64_t)P->hp[a] * P->hp[a + 1] > (int64_t)P->hp[b] * P->hp[b + 1]; });
     for (int l : order) {
       const int64_t extra = (int64_t)P->hp[l] * P->hp[l + 1] / 2;
