@@ -184,13 +184,21 @@ def _w3j_swap_sign(tp, t):
 
 
 def _permuted_weights(tp, w, perm):
-    """Per-instruction ``[..., U, V, W]`` weight blocks of a ``uvw`` product with their last three axes permuted."""
+    """Per-instruction ``[..., U, V, W]`` weight blocks of a ``uvw`` product with their last three axes permuted: one
+    gather along the weight axis through an index list built once per product, permutation and device."""
     if tp.weight_numel == 0:
         return w
-    batch = w.shape[:-1]
-    nb = len(batch)
-    blocks = [v.permute(*range(nb), *(nb + p for p in perm)).reshape(batch + (-1,)) for v in tp.weight_views(w)]
-    return torch.cat(blocks, dim=-1).contiguous()
+    key = ("weight permutation", perm, w.device)  # kept with the plans: dropped by copies and pickles alike
+    index = tp._plans.get(key)
+    if index is None:
+        blocks, offset = [], 0
+        for t in tp.instructions:
+            if t.has_weight:
+                n = prod(t.path_shape)
+                blocks.append(torch.arange(offset, offset + n).view(t.path_shape).permute(*perm).reshape(-1))
+                offset += n
+        index = tp._plans[key] = torch.cat(blocks).to(w.device)
+    return w.index_select(-1, index)
 
 
 class _TensorProductFn(torch.autograd.Function):
