@@ -39,6 +39,8 @@ struct SubKernel {
   hipFunction_t fn_plain[kMaxDevices] = {nullptr};
   hipFunction_t fn_fused[kMaxDevices] = {nullptr};
   hipFunction_t fn_bwd_edge[kMaxDevices] = {nullptr};
+  hipFunction_t fn_bwd_edge_lds[kMaxDevices] = {nullptr};  // the variant with every row through LDS, when generated
+  bool bwd_lds = false;
   hipFunction_t fn_dw[kMaxDevices] = {nullptr};
   hipFunction_t fn_pack[kMaxDevices] = {nullptr};
   // uvu: the edge-parallel backward kernel is a code object of its own (other lane layout), built on first use
@@ -278,6 +280,16 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only 
   K.waves_per_block = env_int("E3X_UVU_WAVES_PER_BLOCK", 4);
   s << "#define E3X_WAVES_PER_BLOCK " << K.waves_per_block << "\n";
   if (bwd_only) s << "#define E3X_UVU_BWD_ONLY 1\n";
+  if (bwd_only) {
+    // second kernel of the code object: the rows of an edge through LDS in 16-byte pieces (see the template); one
+    // kernel and one chunk must cover the instruction set so that the group writes the whole weight-gradient row
+    const int groups = 64 / K.lanes;
+    const int64_t lds = (int64_t)K.waves_per_block * groups * (P.in1_dim + P.out_dim + P.weight_numel) * 4;
+    K.bwd_lds = P.dtype == E3X_F32 && !P.shared_weights && K.chunks == 1 && K.path_ids.size() == P.paths.size() &&
+                P.weight_numel > 0 && P.in1_dim > 0 && P.in1_dim % 4 == 0 && P.out_dim % 4 == 0 && P.weight_numel % 4 == 0 &&
+                lds <= 64 * 1024 && env_int("E3X_UVU_BWD_LDS", 1) != 0;
+    if (K.bwd_lds) s << "#define E3X_UVU_BWD_LDS 1\n";
+  }
   // coefficient folded into the edge attribute (see accumulate_edge); measured on one GPU, old -> new: 32 channels
   // l <= 2 at four indices per lane 0.637 -> 0.635 ms (degree 354: 4.91 -> 4.84), 128 channels l <= 3 in bf16 storage
   // 1.60 -> 1.48 ms, in fp32 at two indices per lane 1.68 -> 1.77 ms
@@ -878,6 +890,8 @@ int load_uvu_bwd_functions(e3x_plan* P, int dev) {
     if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + B->hsaco + ") failed: " + hipGetErrorString(err));
     if (hipModuleGetFunction(&B->fn_bwd_edge[dev], mod, "e3x_uvu_bwd_edge") != hipSuccess)
       return fail(E3X_ERR_HIP, "kernel e3x_uvu_bwd_edge missing from " + B->hsaco);
+    if (B->bwd_lds && hipModuleGetFunction(&B->fn_bwd_edge_lds[dev], mod, "e3x_uvu_bwd_edge_lds") != hipSuccess)
+      return fail(E3X_ERR_HIP, "kernel e3x_uvu_bwd_edge_lds missing from " + B->hsaco);
     B->module[dev] = mod;
   }
   return E3X_OK;
@@ -1399,8 +1413,10 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
     const long long items = (E + groups - 1) / groups * K->chunks;
     const long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
     if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: too many edges for one launch");
-    hipError_t err =
-        hipModuleLaunchKernel(K->fn_bwd_edge[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1, 0, st, args, nullptr);
+    // rows in 16-byte pieces need aligned rows (their lengths are multiples of four by construction of the variant)
+    const bool staged = K->bwd_lds && grad_w && !(((uintptr_t)x1 | (uintptr_t)w | (uintptr_t)grad_out | (uintptr_t)grad_w) & 15);
+    hipError_t err = hipModuleLaunchKernel(staged ? K->fn_bwd_edge_lds[dev] : K->fn_bwd_edge[dev], (unsigned)blocks, 1, 1,
+                                           64 * K->waves_per_block, 1, 1, 0, st, args, nullptr);
     if (err != hipSuccess)
       return fail(E3X_ERR_HIP, std::string("e3x_tp_backward_w_x2: launch failed: ") + hipGetErrorString(err));
   }
