@@ -199,7 +199,8 @@ def test_fully_connected_plans_need_no_gpu_and_reject_what_the_kernel_cannot_hol
     assert plan.handle is not None and plan.key.startswith("fc_mfma_")
     # packed weights, widths already multiples of 8 / 32: layer 0 in fp32, the 64 -> 352 layer as three bf16 planes
     assert plan.workspace_bytes == 8 * 64 * 4 + 64 * 352 * 6
-    assert _FusedPlan([5, 100, 50], "tanh", False, 1, 1).workspace_bytes == (8 * 128 + 128 * 64) * 4  # zero padded
+    # zero padded; the last layer (128 -> 64, a wide input onto at most 64 outputs) as three bf16 planes
+    assert _FusedPlan([5, 100, 50], "tanh", False, 1, 1).workspace_bytes == 8 * 128 * 4 + 128 * 64 * 6
     for hs in ([8, 512, 16], [128, 256, 8], [600, 8]):
         bad = _FusedPlan(hs, "silu", False, 1, 1)
         assert bad.handle is None and "e3x_fc_plan_create" in bad.reason
