@@ -215,6 +215,30 @@ def test_fully_connected_net_gradients(case):
         assert float((got * dw).sum()) == pytest.approx(fd, rel=3e-4, abs=1e-3), f"layer {i}"
 
 
+@pytest.mark.parametrize("Z", [1, 15, 16, 17, 33])
+def test_dense_layer_gradients_on_batches_around_one_trip(Z):
+    """The dense weight-gradient kernel walks the batch in trips of 16 rows shared by four waves, the input-gradient
+    kernel in tiles of 32: batches of less than a trip, exactly one, and one row more, against the float64 oracle's
+    analytic gradients (the network is y = act(x W0 s0) W1 s1, so they are three matrix products)."""
+    net = ks.fused_fc_nets()[0].to(DEV)  # 8 -> 64 -> 352, SiLU
+    x = seeded(Z, 8, seed=90 + Z)
+    cot = seeded(Z, 352, seed=190 + Z)
+    xd = x.to(DEV).requires_grad_(True)
+    net(xd).backward(cot.to(DEV))
+    w0, w1 = (getattr(net, f"layer{i}").weight.detach().cpu().double().numpy() for i in range(2))
+    x64, c64 = x.double().numpy(), cot.double().numpy()
+    z = x64 @ w0 / np.sqrt(8.0)
+    cst = onn.normalize2mom_const("silu")
+    sg = 1.0 / (1.0 + np.exp(-z))
+    h = cst * z * sg
+    assert_close(net(x.to(DEV)), onn.fc_forward([w0, w1], x64, "silu"), what=f"fc forward, Z = {Z}")
+    gh = c64 @ w1.T / 8.0
+    gz = gh * cst * sg * (1.0 + z * (1.0 - sg))
+    assert_close(net.layer1.weight.grad, h.T @ c64 / 8.0, what=f"dense weight gradient 64x352, Z = {Z}")
+    assert_close(net.layer0.weight.grad, x64.T @ gz / np.sqrt(8.0), what=f"dense weight gradient 8x64, Z = {Z}")
+    assert_close(xd.grad, gz @ w0.T / np.sqrt(8.0), what=f"dense input gradient, Z = {Z}")
+
+
 def test_fully_connected_net_wide_hidden_layer():
     """Outside the limits of the fused kernel every layer runs on the tensor-product kernels, forward and backward."""
     fc = dict(ks.nn_modules())["fc_wide_hidden"].to(DEV)
