@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt), keyed by the code object the counters were read
 # on: a kernel that has changed since reports no traffic instead of a stale figure.
 NEQUIP_TRAFFIC_BYTES = {
-    "uvu_c81958e38ae94d0c80d6d6a3": (2 * 1611962 + 56250) * 1024,  # FETCH_SIZE 1611962 x 2 KiB + WRITE_SIZE 56250 KiB
+    "uvu_b1d11ac75d8b0830d6b145fd": (2 * 1611878 + 56250) * 1024,  # FETCH_SIZE 1611878 x 2 KiB + WRITE_SIZE 56250 KiB
 }
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
