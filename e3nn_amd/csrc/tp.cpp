@@ -718,6 +718,22 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
   emit_header(s, P);
   if (env_int("E3X_DW_ZC", 0)) s << "#define E3X_DW_ZC " << env_int("E3X_DW_ZC", 0) << "\n";
   if (std::getenv("E3X_DW_SYNTH")) s << "#define E3X_DW_SYNTH " << env_int("E3X_DW_SYNTH", 1) << "\n";
+  {
+    // Split operands (six bf16 products per fp32 one) pay where the 64 x 64 tiles are full: the vector ALU then
+    // prepares operands for 4 x 12 matrix instructions per pass; with 32-wide blocks half of them multiply padding and
+    // the fp32 instruction, which needs no splitting, is faster (measured: 128-wide blocks 73 -> 60 ms, the 32-wide
+    // node-wise layers of the convolution block 0.71 -> 0.78 ms).
+    bool full = true;
+    for (const auto& p : P.paths) {
+      const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2], &c = P.out[p.out];
+      const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1;
+      const bool okU = a.mul % 32 == 0 && a.mul <= k_cap(P.dtype), okV = b.mul % 32 == 0 && b.mul <= k_cap(P.dtype);
+      const bool k_is_x2 = okV && (!okU || d2 < d1);
+      if ((k_is_x2 ? b.mul : a.mul) % 64 || c.mul % 64) full = false;
+    }
+    s << "#define E3X_DW_SPLIT " << env_int("E3X_DW_SPLIT", full ? 1 : 0) << "\n";
+  }
+  if (std::getenv("E3X_DW_OCC")) s << "#define E3X_DW_OCC " << env_int("E3X_DW_OCC", 3) << "\n";
   int n_nz = 0, n_path = 0, dkmax = 1, drmax = 1;
   long long tiles = 0;
   if (!mfma_dw_fits(P))
@@ -1471,7 +1487,7 @@ extern "C" int e3x_tp_backward_w_uvw(e3x_plan* P, const void* x1, const void* x2
     slices = std::min(slices, (long long)((Z + 255) / 256));
     slices = std::max(1LL, std::min(slices, 1024LL));
     long long rows_per_slice = (Z + slices - 1) / slices;
-    rows_per_slice = (rows_per_slice + 23) / 24 * 24;  // whole chunks of the kernel
+    rows_per_slice = (rows_per_slice + 95) / 96 * 96;  // whole chunks of the kernel (24 rows, or 32 on split operands)
     slices = (Z + rows_per_slice - 1) / rows_per_slice;
     int accumulate = slices > 1;
     if (accumulate && (rc = e3x::fill_zero_bytes(grad_w, (size_t)P->weight_numel * 4, st))) return rc;

@@ -90,6 +90,12 @@ def mfma_small():
     return o3.FullyConnectedTensorProduct("64x0e+32x1o", "32x0e+32x1o+32x2e", "64x0e+64x1o+64x1e+64x2e")
 
 
+def mfma_full_tiles():
+    # every multiplicity a multiple of 64: the uvw weight gradient takes its split-operand path (both contraction
+    # orders: paths onto 0e with l > 0 inputs synthesise the A operand, the others the B operand)
+    return o3.FullyConnectedTensorProduct("64x0e+64x1o", "64x0e+64x1o+64x2e", "64x0e+128x1o+64x1e+64x2e")
+
+
 def node_fctp():
     # node-wise step of a convolution: features x a few scalar node attributes (one-hot species), the GEMM K index is
     # the feature multiplicity and the attribute index is a short outer loop (reference
@@ -174,6 +180,7 @@ def all_tensor_products():
         ("cfg4_B", cfg4("B"), (torch.float32, torch.bfloat16)),
         ("cfg5", cfg5(), (torch.float32, torch.bfloat16)),
         ("mfma_small", mfma_small(), (torch.float32,)),
+        ("mfma_full_tiles", mfma_full_tiles(), (torch.float32,)),
         ("node_fctp", node_fctp(), (torch.float32,)),
         ("radial_layer", radial_layer(), (torch.float32,)),
         ("wide_k", wide_k(), (torch.float32,)),
@@ -192,7 +199,7 @@ def all_tensor_products():
 
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
-                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "node_fctp", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
+                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "mfma_full_tiles", "node_fctp", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
                   "unaligned_mfma", "unaligned_offsets", "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
 
 
