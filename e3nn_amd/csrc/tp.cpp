@@ -544,7 +544,16 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   if (P.dtype != E3X_F32) wt = 64;
   std::ostringstream s, nzs, ps, ts;
   emit_header(s, P);
-  if (P.dtype == E3X_F32) s << "#define E3X_UVW_KC " << env_int("E3X_UVW_KC", 32) << "\n";
+  // split-operand matrix steps (see the template) in fp32 storage; weight chunks of 16 K rows then keep the LDS at
+  // 72 KB with 128 output channels (two workgroups per CU)
+  // Default where every block is a multiple of 64 wide (measured on 128-wide blocks, 65536 rows: 55.9 -> 50.0 ms);
+  // narrower blocks leave tiles half empty and keep the fp32 instruction, which needs no splitting.
+  bool full = true;
+  for (const auto& p : P.paths)
+    if (P.in1[p.in1].mul % 64 || P.in2[p.in2].mul % 64 || P.out[p.out].mul % 64) full = false;
+  const int split = P.dtype == E3X_F32 ? env_int("E3X_UVW_SPLIT", full ? 1 : 0) : 0;
+  if (split) s << "#define E3X_UVW_SPLIT 1\n";
+  if (P.dtype == E3X_F32) s << "#define E3X_UVW_KC " << env_int("E3X_UVW_KC", split ? 16 : 32) << "\n";
   if (env_int("E3X_UVW_KS", 0)) s << "#define E3X_UVW_KS " << env_int("E3X_UVW_KS", 0) << "\n";
   if (env_int("E3X_UVW_WPE", wt == 128 ? 2 : 0)) s << "#define E3X_UVW_WPE " << env_int("E3X_UVW_WPE", wt == 128 ? 2 : 0) << "\n";
   int n_nz = 0, n_path = 0, n_target = 0, dka = 1, drmax = 1;

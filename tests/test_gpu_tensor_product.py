@@ -203,7 +203,10 @@ def test_uvw_full_size_dense_configuration():
     assert_close(out[rows], ref, what="cfg5 rows")
     # size-independent properties: bilinearity in (x1, x2), output scale
     out2 = tp(2.0 * x1, -0.5 * x2)
-    assert torch.equal(out2, -out)  # exact: powers of two commute with every rounding
+    # powers of two commute with every rounding, so scaling alone is exact; the sign is not: the matrix passes run on
+    # bf16 matrix instructions (three-way split operands), whose internal sums are not symmetric under negation
+    assert torch.equal(tp(2.0 * x1, 0.5 * x2), out)
+    assert float((out2 + out).abs().max()) <= 2e-6 * float(out.abs().max())
     # weights N(0, 1/fan_in) on top of the path normalisation 1/sqrt(fan_in * paths): variance 1/fan_in
     assert abs(out.var().item() * 16384 - 1.0) < 0.1
     # batch slices give the same rows
