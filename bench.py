@@ -282,9 +282,13 @@ def bench_uvw(args, dev, dtype=torch.float32):
     f_min = 2 * Z * 128**3 * 21  # cheapest contraction order per path: sum of min(2l1+1, 2l2+1, 2l3+1) = 21
     f_gemm = 2 * Z * 128**3 * 35  # outer-product order: sum of (2l3+1) = 35
     peak = BF16_MFMA_PEAK_TFLOPS if dtype == torch.bfloat16 else FP32_MFMA_PEAK_TFLOPS
-    return {"rows": Z, "ms": ms, "tflops_fmin": f_min / (ms * 1e-3) / 1e12, "tflops_fgemm_equiv": f_gemm / (ms * 1e-3) / 1e12,
-            "roofline": {"bound": "mfma", "achieved": f_min / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
-                         "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
+    out = {"rows": Z, "ms": ms, "tflops_fmin": f_min / (ms * 1e-3) / 1e12, "tflops_fgemm_equiv": f_gemm / (ms * 1e-3) / 1e12,
+           "roofline": {"bound": "mfma", "achieved": f_min / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
+                        "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
+    if dtype == torch.float32 and os.environ.get("E3X_UVW_SPLIT", "1") != "0":
+        out["arithmetic"] = ("scaled-accumulator passes: six bf16 MFMA products of three-way split operands, fp32 accumulation "
+                             "(fp32-accurate); tflops / frac count the 2*m*n*k flops of the fp32 product against the fp32 MFMA peak")
+    return out
 
 
 def bench_nequip_cube40(args, dev):
@@ -452,6 +456,7 @@ def bench_uvw_backward(args, dev):
     ms_dw = event_time_ms(lambda: plan.backward_w_uvw(a, b, cot, True), 3, 1)
     f_min = 2 * Z * 128**3 * 21
     return {"rows": Z, "ms_forward_backward": ms, "ms_weight_gradient": ms_dw,
+            "arithmetic": "as uvw_dense_fp32: split-operand bf16 MFMA products, fp32-accurate, priced against the fp32 MFMA peak",
             "roofline_weight_gradient": {"bound": "mfma", "achieved": f_min / (ms_dw * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                                          "unit": "TFLOP/s", "frac": f_min / (ms_dw * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}}  # fmt: skip
 
