@@ -132,6 +132,11 @@ def wide_k():
     return o3.FullyConnectedTensorProduct("256x0e+160x1o", "32x0e+32x1o", "64x0e+64x1o")
 
 
+def wide_k_full_tiles():
+    # as wide_k with every multiplicity a multiple of 64: the split-operand matrix steps on restaged K blocks
+    return o3.FullyConnectedTensorProduct("256x0e+192x1o", "64x0e+64x1o", "64x0e+128x1o")
+
+
 def unaligned_mfma():
     # matrix-core forward, but an irrep no output reaches (3x2e) makes the input row 175 floats long: the matrix-core
     # weight-gradient kernel needs 16-byte aligned operands within a row, so the gradient runs on the vector-ALU kernel
@@ -184,6 +189,7 @@ def all_tensor_products():
         ("node_fctp", node_fctp(), (torch.float32,)),
         ("radial_layer", radial_layer(), (torch.float32,)),
         ("wide_k", wide_k(), (torch.float32,)),
+        ("wide_k_full_tiles", wide_k_full_tiles(), (torch.float32,)),
         ("outer_split", outer_split(), (torch.float32,)),
         ("node_wide_out", node_wide_out(), (torch.float32,)),
         ("node_narrow", node_narrow(), (torch.float32,)),

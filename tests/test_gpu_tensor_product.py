@@ -168,6 +168,8 @@ def _fan_in_weights(tp, seed=0):
 @pytest.mark.parametrize(
     "maker,Z,family",
     [(ks.mfma_small, 150, "uvw_mfma"), (ks.cfg5, 70, "uvw_mfma"), (ks.wide_k, 130, "uvw_mfma"), (ks.outer_split, 200, "uvw_mfma"),
+     # every multiplicity a multiple of 64: the matrix steps on split operands (also on restaged K blocks)
+     (ks.mfma_full_tiles, 150, "uvw_mfma"), (ks.wide_k_full_tiles, 130, "uvw_mfma"),
      # scalar second input: the node-wise kernel; batches that end inside a wave's 64 rows, inside a workgroup's 256
      # rows, and below one wave
      (ks.node_fctp, 333, "uvw_node"), (ks.node_fctp, 17, "uvw_node"), (ks.node_fctp, 1280, "uvw_node"),
