@@ -122,7 +122,12 @@ int e3x_tp_plan_info(const e3x_plan* plan, int64_t* weight_numel, int64_t* in1_d
 /* out[Z, out_dim] = TP(x1[Z, in1_dim], x2[Z, in2_dim], w).  Replaces the generated
  * module called at e3nn/o3/_tensor_product/_tensor_product.py:554
  * (contraction: _codegen.py:148-187, path weights :312, sum/cat :327-343).
- * `out` is fully overwritten (output irreps no instruction reaches become 0). */
+ * `out` is fully overwritten (output irreps no instruction reaches become 0).
+ * fp32 plans of the "uvw_mfma" family whose blocks are all multiples of 64 wide form their products on the
+ * bf16 matrix instruction from operands split into three bf16 pieces each (six cross products, fp32 accumulation):
+ * the results have the accuracy of fp32 products and are reproducible, but negating an input changes last bits
+ * (scaling by a power of two does not).  E3X_UVW_SPLIT=0 in the environment at plan creation keeps the fp32
+ * instruction; the "uvw" weight gradient (E3X_DW_SPLIT) and the dense layers of scalars do the same. */
 int e3x_tp_forward(e3x_plan* plan, const void* x1, const void* x2, const void* w, void* out, int64_t Z,
                    void* stream);
 /* The same with caller-owned device scratch.  Plans of the "uvw_mfma" family in bf16 storage repack the
