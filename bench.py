@@ -286,7 +286,7 @@ def bench_uvw(args, dev, dtype=torch.float32):
            "roofline": {"bound": "mfma", "achieved": f_min / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
                         "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
     if dtype == torch.float32 and os.environ.get("E3X_UVW_SPLIT", "1") != "0":
-        out["arithmetic"] = ("scaled-accumulator passes: six bf16 MFMA products of three-way split operands, fp32 accumulation "
+        out["arithmetic"] = ("matrix passes: six bf16 MFMA products of three-way split operands, fp32 accumulation "
                              "(fp32-accurate); tflops / frac count the 2*m*n*k flops of the fp32 product against the fp32 MFMA peak")
     return out
 
