@@ -367,9 +367,18 @@ def bench_radial_network(args, dev, ctx):
     assert net.fused_plan().handle is not None
     ms1 = event_time_ms(one_kernel, max(5, args.steps // 2), 3)
     msl = event_time_ms(layered, max(5, args.steps // 5), 2)
+    # the backward kernels of the 64 -> 352 layer alone, back to back on random data: weight gradient (SiLU applied to
+    # the saved pre-activations as they are loaded) and input gradient (SiLU derivative in the epilogue)
+    fwd, bwd = net.layer1.act_dense_plans(net.layer0)
+    z = torch.randn(E, 64, generator=torch.Generator().manual_seed(1)).to(dev)
+    g = torch.randn(E, 352, generator=torch.Generator().manual_seed(2)).to(dev)
+    wt = net.layer1.weight.detach().t().contiguous()
+    ms_dw = event_time_ms(lambda: fwd.backward_w(z, g), max(5, args.steps // 5), 2)
+    ms_dx = event_time_ms(lambda: bwd.forward(g, [wt], z), max(5, args.steps // 5), 2)
     flop = 2.0 * E * (8 * 64 + 64 * 352)
     out_bytes = E * (8 + 352) * 4
-    return {"edges": E, "ms_one_kernel": ms1, "ms_layer_by_layer": msl, "tflops_one_kernel": flop / (ms1 * 1e-3) / 1e12,
+    return {"edges": E, "ms_one_kernel": ms1, "ms_layer_by_layer": msl, "ms_weight_gradient_64x352": ms_dw,
+            "ms_input_gradient_352_to_64": ms_dx, "tflops_one_kernel": flop / (ms1 * 1e-3) / 1e12,
             "frac_fp32_mfma_peak": flop / (ms1 * 1e-3) / 1e12 / 157.3, "hbm_gbs_one_kernel": out_bytes / (ms1 * 1e-3) / 1e9,
             "frac_hbm_peak": out_bytes / (ms1 * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "arithmetic": "layer 64->352: six bf16 MFMA products of three-way split operands, fp32 accumulation (fp32-accurate); "
