@@ -192,6 +192,8 @@ extern "C" int e3x_fc_plan_create_fused(const int32_t* hs, int32_t n_hs, int32_t
   P->input_act = input_act;
   P->input_cst = input_cst;
   s << "constexpr int RS = " << rs << ", WAVES = " << waves << ";\n}  // namespace cfg\n";
+  if (const char* v = std::getenv("E3X_FC_STREAM")) s << "#define E3X_FC_STREAM " << std::atoi(v) << "\n";
+  if (const char* v = std::getenv("E3X_FC_STREAM_DIST")) s << "#define E3X_FC_STREAM_DIST " << std::max(1, std::atoi(v)) << "\n";
   const std::string src = s.str() + e3x::kTplCommon + e3x::kTplFcMfma;
   int rc = e3x::get_code_object("fc_mfma", src, &P->key, &P->hsaco);
   if (rc) return rc;
