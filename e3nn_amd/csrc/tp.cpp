@@ -727,6 +727,7 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
   emit_header(s, P);
   if (env_int("E3X_DW_ZC", 0)) s << "#define E3X_DW_ZC " << env_int("E3X_DW_ZC", 0) << "\n";
   if (std::getenv("E3X_DW_SYNTH")) s << "#define E3X_DW_SYNTH " << env_int("E3X_DW_SYNTH", 1) << "\n";
+  if (std::getenv("E3X_DW_PAIR")) s << "#define E3X_DW_PAIR " << env_int("E3X_DW_PAIR", 1) << "\n";
   {
     // Split operands (six bf16 products per fp32 one) pay where the 64 x 64 tiles are full: the vector ALU then
     // prepares operands for 4 x 12 matrix instructions per pass; with 32-wide blocks half of them multiply padding and

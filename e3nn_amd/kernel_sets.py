@@ -103,6 +103,12 @@ def node_fctp():
     return o3.FullyConnectedTensorProduct("128x0e+64x1o+32x2e", "4x0e", "128x0e+64x1o+96x2e")
 
 
+def node_block():
+    # a node-wise layer of an interaction block at NequIP-like width: 32 channels out, 4 species (the weight-gradient
+    # kernel puts two species side by side in the 64 columns of a tile)
+    return o3.FullyConnectedTensorProduct("96x0e+128x1o+32x2e", "4x0e", "32x0e+32x1o+32x2e")
+
+
 def node_wide_out():
     # scalar second input with several 32-channel output tiles per irrep, l = 3 and a pseudoscalar attribute: the
     # shape of an input gradient of a node-wise layer (few channels in, many out)
@@ -191,6 +197,7 @@ def all_tensor_products():
         ("wide_k", wide_k(), (torch.float32,)),
         ("wide_k_full_tiles", wide_k_full_tiles(), (torch.float32,)),
         ("outer_split", outer_split(), (torch.float32,)),
+        ("node_block", node_block(), (torch.float32,)),
         ("node_wide_out", node_wide_out(), (torch.float32,)),
         ("node_narrow", node_narrow(), (torch.float32,)),
         ("node_partial_tile", node_partial_tile(), (torch.float32,)),
@@ -205,7 +212,7 @@ def all_tensor_products():
 
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
-                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "mfma_full_tiles", "node_fctp", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
+                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "mfma_full_tiles", "outer_split", "node_fctp", "node_block", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
                   "unaligned_mfma", "unaligned_offsets", "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
 
 

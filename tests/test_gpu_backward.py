@@ -105,7 +105,7 @@ def test_uvw_input_gradients(maker, Z):
 
 @pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.cfg1, 4099),
                                      (lambda: ks.golden_tp("fctp_per_sample_weights"), 5), (ks.mfma_small, 70),
-                                     (ks.mfma_small, 1500), (ks.mfma_full_tiles, 70), (ks.mfma_full_tiles, 1237), (ks.node_fctp, 700), (ks.radial_layer, 513), (ks.node_wide_out, 300), (ks.node_narrow, 260),
+                                     (ks.mfma_small, 1500), (ks.mfma_full_tiles, 70), (ks.mfma_full_tiles, 1237), (ks.node_fctp, 700), (ks.node_block, 333), (ks.node_block, 20), (ks.outer_split, 410), (ks.radial_layer, 513), (ks.node_wide_out, 300), (ks.node_narrow, 260),
                                      (ks.node_partial_tile, 100), (ks.unaligned_mfma, 300), (ks.unaligned_offsets, 129)])  # fmt: skip
 def test_uvw_weight_gradients(maker, Z):
     tp = maker().to(DEV)

@@ -173,7 +173,7 @@ def _fan_in_weights(tp, seed=0):
      # scalar second input: the node-wise kernel; batches that end inside a wave's 64 rows, inside a workgroup's 256
      # rows, and below one wave
      (ks.node_fctp, 333, "uvw_node"), (ks.node_fctp, 17, "uvw_node"), (ks.node_fctp, 1280, "uvw_node"),
-     (ks.radial_layer, 1000, "uvw_node"), (ks.node_wide_out, 77, "uvw_node"), (ks.node_narrow, 301, "uvw_node"),
+     (ks.radial_layer, 1000, "uvw_node"), (ks.node_block, 200, "uvw_node"), (ks.node_wide_out, 77, "uvw_node"), (ks.node_narrow, 301, "uvw_node"),
      (ks.node_partial_tile, 129, "uvw_node")],
 )  # fmt: skip
 def test_uvw_matrix_core_kernel_against_oracle(maker, Z, family):
