@@ -8,12 +8,34 @@
 ``node_features[edge_src]`` and the per-edge messages are never materialised.
 """
 import torch
+from torch.autograd.function import once_differentiable
 
 from ..o3.irreps import Irrep, Irreps
 from ..o3.tensor_product import FullyConnectedTensorProduct, TensorProduct
 from .edges import DstSortedEdges
 from .fc import FullyConnectedNet
 from .message import message_instructions
+
+
+class _Mix(torch.autograd.Function):
+    """``sc + ((1 - m) + alpha * m * inv) * conv * inv`` (reference points_convolution.py:110-113 with the division by
+    sqrt(num_neighbors) moved behind lin2 and alpha): two elementwise kernels forward and three backward, where autograd
+    through the separate operations launches a dozen over the [N, channels] arrays."""
+
+    @staticmethod
+    def forward(ctx, sc, alpha, conv, m, inv):
+        coeff = torch.addcmul((1 - m) * inv, alpha, m * (inv * inv))  # [N, channels]
+        ctx.save_for_backward(coeff, conv, m)
+        ctx.inv = inv
+        return torch.addcmul(sc, coeff, conv)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        coeff, conv, m = ctx.saved_tensors
+        need_sc, need_alpha, need_conv = ctx.needs_input_grad[:3]
+        g_alpha = ((g * conv) @ (m * (ctx.inv * ctx.inv))).unsqueeze(-1) if need_alpha else None
+        return (g if need_sc else None), g_alpha, (g * coeff if need_conv else None), None, None
 
 
 class Convolution(torch.nn.Module):
@@ -75,6 +97,4 @@ class Convolution(torch.nn.Module):
         inv = 1.0 / self.num_neighbors**0.5
         node_conv_out = self.lin2(node_features, node_attr)
         alpha = self.alpha(node_features, node_attr)
-        m = self.sc.output_mask
-        alpha = (1 - m) + alpha * (m * inv)
-        return torch.addcmul(node_self_connection, alpha, node_conv_out, value=inv)
+        return _Mix.apply(node_self_connection, alpha, node_conv_out, self.sc.output_mask, inv)

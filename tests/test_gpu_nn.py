@@ -346,7 +346,8 @@ def test_convolution_block_forward_and_backward():
     eps = 1e-5
     fd = ((run(x64 + eps * v) - run(x64 - eps * v)) * c64).sum() / (2 * eps)
     assert float((xd.grad.cpu().double().numpy() * v).sum()) == pytest.approx(fd, rel=5e-4)
-    for key, par in (("fc.layer0.weight", conv.fc.layer0.weight), ("lin1.weight", conv.lin1.weight), ("alpha.weight", conv.alpha.weight)):
+    for key, par in (("fc.layer0.weight", conv.fc.layer0.weight), ("lin1.weight", conv.lin1.weight), ("alpha.weight", conv.alpha.weight),
+                     ("lin2.weight", conv.lin2.weight), ("sc.weight", conv.sc.weight)):
         dw = rng.normal(size=params[key].shape)
         hi, lo = dict(params), dict(params)
         hi[key], lo[key] = params[key] + eps * dw, params[key] - eps * dw
