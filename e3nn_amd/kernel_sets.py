@@ -307,8 +307,8 @@ def prebuild(verbose=True, workers=6):
     jobs = []
     for name, mod in nn_modules() + [(f"fused_fc{i}", net) for i, net in enumerate(fused_fc_nets())]:
         for sub in mod.modules():
-            inner = sub.__dict__.get("_tp")  # Linear and the dense layers keep theirs out of the module tree
-            for tp in (sub, inner):
+            # Linear and the dense layers keep theirs out of the module tree, the convolution its alpha on the scalars
+            for tp in (sub, sub.__dict__.get("_tp"), sub.__dict__.get("_alpha_head")):
                 if isinstance(tp, o3.TensorProduct):
                     jobs.append((f"module {name}", tp, (torch.float32,), True))
             if isinstance(sub, nn.FullyConnectedNet):

@@ -11,7 +11,7 @@ import torch
 from torch.autograd.function import once_differentiable
 
 from ..o3.irreps import Irrep, Irreps
-from ..o3.tensor_product import FullyConnectedTensorProduct, TensorProduct
+from ..o3.tensor_product import FullyConnectedTensorProduct, TensorProduct, _permuted_weights
 from .edges import DstSortedEdges
 from .fc import FullyConnectedNet
 from .message import message_instructions
@@ -36,6 +36,39 @@ class _Mix(torch.autograd.Function):
         need_sc, need_alpha, need_conv = ctx.needs_input_grad[:3]
         g_alpha = ((g * conv) @ (m * (ctx.inv * ctx.inv))).unsqueeze(-1) if need_alpha else None
         return (g if need_sc else None), g_alpha, (g * coeff if need_conv else None), None, None
+
+
+class _Lin2Alpha(torch.autograd.Function):
+    """``lin2(features, attr)`` and ``alpha(features, attr)`` as one node of the autograd graph.  ``alpha`` reads only
+    the leading scalars of the features (``head`` is ``alpha`` restricted to them, same weights), so its input gradient
+    is added into the leading columns of lin2's instead of being written as a second zero-padded [N, features] array
+    that autograd then adds to the first: three passes over an array as wide as the messages saved."""
+
+    @staticmethod
+    def forward(ctx, features, attr, w_lin2, w_alpha, lin2, head):
+        ctx.lin2, ctx.head = lin2, head
+        scalars = features[:, : head.irreps_in1.dim].contiguous()
+        ctx.save_for_backward(features, attr, w_lin2, w_alpha, scalars)
+        dt = features.dtype
+        return lin2._plan(dt).forward(features, attr, w_lin2), head._plan(dt).forward(scalars, attr, w_alpha)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g_conv, g_alpha):
+        lin2, head = ctx.lin2, ctx.head
+        features, attr, w_lin2, w_alpha, scalars = ctx.saved_tensors
+        g_conv, g_alpha = g_conv.contiguous(), g_alpha.contiguous()
+        dt = features.dtype
+        g_features = gw_lin2 = gw_alpha = None
+        if ctx.needs_input_grad[2]:
+            gw_lin2 = lin2._plan(dt).backward_w_uvw(features, attr, g_conv, True)
+        if ctx.needs_input_grad[3]:
+            gw_alpha = head._plan(dt).backward_w_uvw(scalars, attr, g_alpha, True)
+        if ctx.needs_input_grad[0]:
+            g_features = lin2._grad_plan("x1", dt).forward(g_conv, attr, _permuted_weights(lin2, w_lin2, (2, 1, 0)))
+            g_scalars = head._grad_plan("x1", dt).forward(g_alpha, attr, _permuted_weights(head, w_alpha, (2, 1, 0)))
+            g_features[:, : scalars.shape[1]] += g_scalars
+        return g_features, None, gw_lin2, gw_alpha, None, None
 
 
 class Convolution(torch.nn.Module):
@@ -74,6 +107,16 @@ class Convolution(torch.nn.Module):
         torch.nn.init.zeros_(self.alpha.weight)  # the block starts as its self-connection
         if self.alpha.output_mask[0] != 1.0:
             raise AssertionError(f"the messages ({irreps_mid}) and the node attributes ({self.irreps_node_attr}) cannot produce a scalar for alpha")
+        # alpha restricted to the leading irreps of the messages when those are all it reads (scalar node attributes and
+        # sorted messages: always): same instructions, weights and normalisation; kept out of the module tree, it has
+        # no parameters and must not add keys to the state_dict
+        self.__dict__["_alpha_head"] = None
+        n_head = 1 + max(ins.i_in1 for ins in self.alpha.instructions)
+        if irreps_mid[:n_head].dim % 4 == 0 and n_head < len(irreps_mid):
+            head = FullyConnectedTensorProduct(irreps_mid[:n_head], self.irreps_node_attr, "0e", internal_weights=False, shared_weights=True)
+            key = lambda tp: [(i.i_in1, i.i_in2, i.i_out, i.path_shape, i.path_weight) for i in tp.instructions]  # noqa: E731
+            if key(head) == key(self.alpha) and head.weight_numel == self.alpha.weight_numel:
+                self.__dict__["_alpha_head"] = head
 
     def forward(self, node_input, node_attr, edge_src, edge_dst, edge_attr, edge_scalars, edges=None) -> torch.Tensor:
         node_self_connection = self.sc(node_input, node_attr)
@@ -95,6 +138,20 @@ class Convolution(torch.nn.Module):
         # to the summed messages (points_convolution.py:108) is applied to their outputs instead, which are four to a
         # thousand times narrower than the messages
         inv = 1.0 / self.num_neighbors**0.5
-        node_conv_out = self.lin2(node_features, node_attr)
-        alpha = self.alpha(node_features, node_attr)
+        if (
+            self._alpha_head is not None
+            and torch.is_grad_enabled()
+            and node_features.requires_grad
+            and not node_attr.requires_grad
+            and node_features.dim() == 2
+            and node_attr.shape[:-1] == node_features.shape[:-1]
+            and node_features.dtype == torch.float32
+        ):
+            node_conv_out, alpha = _Lin2Alpha.apply(
+                node_features.contiguous(), node_attr.to(node_features.dtype).contiguous(), self.lin2.weight, self.alpha.weight,
+                self.lin2, self._alpha_head,
+            )  # fmt: skip
+        else:
+            node_conv_out = self.lin2(node_features, node_attr)
+            alpha = self.alpha(node_features, node_attr)
         return _Mix.apply(node_self_connection, alpha, node_conv_out, self.sc.output_mask, inv)

@@ -354,3 +354,12 @@ def test_convolution_block_forward_and_backward():
         fd = ((run(x64, hi) - run(x64, lo)) * c64).sum() / (2 * eps)
         got = float((par.grad.cpu().double().numpy().reshape(dw.shape) * dw).sum())
         assert got == pytest.approx(fd, rel=5e-4, abs=1e-3), key
+    # lin2 and alpha as one node of the autograd graph (taken above) against the two modules on their own
+    assert conv._alpha_head is not None
+    joint = [xd.grad.clone()] + [p.grad.clone() for p in conv.parameters()]
+    xd.grad = None
+    conv.zero_grad(set_to_none=True)
+    conv.__dict__["_alpha_head"] = None
+    conv(xd, node_attr.to(DEV), src.to(DEV), dst.to(DEV), edge_attr.to(DEV), edge_scalars.to(DEV)).backward(cot.to(DEV))
+    for a_, b_ in zip(joint, [xd.grad] + [p.grad for p in conv.parameters()]):
+        assert_close(a_, b_.cpu().numpy(), atol=1e-5 * max(1.0, float(b_.abs().max())), what="joint lin2 + alpha")
