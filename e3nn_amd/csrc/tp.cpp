@@ -732,14 +732,19 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
     // Split operands (six bf16 products per fp32 one) pay where the 64 x 64 tiles are full: the vector ALU then
     // prepares operands for 4 x 12 matrix instructions per pass; with 32-wide blocks half of them multiply padding and
     // the fp32 instruction, which needs no splitting, is faster (measured: 128-wide blocks 73 -> 60 ms, the 32-wide
-    // node-wise layers of the convolution block 0.71 -> 0.78 ms).
+    // node-wise layers of the convolution block 0.71 -> 0.78 ms).  A 32-channel path whose outer indices go two to a
+    // tile (E3X_DW_PAIR in the template) has no padded columns either: those layers 0.25 -> 0.19 and 0.11 -> 0.09 ms.
     bool full = true;
+    const bool pairing = env_int("E3X_DW_PAIR", 1) != 0;
     for (const auto& p : P.paths) {
       const e3x_irrep &a = P.in1[p.in1], &b = P.in2[p.in2], &c = P.out[p.out];
       const int d1 = 2 * a.l + 1, d2 = 2 * b.l + 1;
       const bool okU = a.mul % 32 == 0 && a.mul <= k_cap(P.dtype), okV = b.mul % 32 == 0 && b.mul <= k_cap(P.dtype);
       const bool k_is_x2 = okV && (!okU || d2 < d1);
-      if ((k_is_x2 ? b.mul : a.mul) % 64 || c.mul % 64) full = false;
+      const int O = k_is_x2 ? a.mul : b.mul, dK = k_is_x2 ? d2 : d1;
+      const bool synth_a = c.l == 0 && dK > 1;
+      const bool paired = pairing && c.mul == 32 && O % 2 == 0 && !synth_a;
+      if (!paired && ((k_is_x2 ? b.mul : a.mul) % 64 || c.mul % 64)) full = false;
     }
     s << "#define E3X_DW_SPLIT " << env_int("E3X_DW_SPLIT", full ? 1 : 0) << "\n";
   }
