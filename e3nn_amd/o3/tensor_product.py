@@ -82,6 +82,7 @@ class _Plan:
         _lib.check(L.e3x_tp_plan_info(handle, ctypes.byref(wn), None, None, None, ctypes.byref(fam), ctypes.byref(key)))
         self.weight_numel, self.family, self.key = wn.value, fam.value.decode(), key.value.decode()
         self.out_dim = irreps_out.dim
+        self._fused_grad_w = None  # whether the plan has the message-step backward kernel; asked on first use
 
     def __del__(self):
         try:
@@ -130,6 +131,32 @@ class _Plan:
                 )  # fmt: skip
             )
         return out
+
+    def gather_scatter_grad_w(self, table, edge_attr, w, row_x, gather_idx, edges):
+        """On the transposed plan of a message step: ``(gather_scatter(table, ...), grad_w[E, weight_numel])`` from one
+        kernel, ``row_x`` being the forward input rows of the nodes that ``edges`` groups by; None when the plan does
+        not fit that kernel."""
+        L = _lib.lib()
+        if self._fused_grad_w is None:
+            rc = L.e3x_tp_plan_prepare_gather_scatter_grad_w(self.handle)
+            if rc != _lib.ERR_INVALID:
+                _lib.check(rc)
+            self._fused_grad_w = rc != _lib.ERR_INVALID
+        if not self._fused_grad_w:
+            return None
+        out = torch.empty(edges.num_nodes, self.out_dim, dtype=table.dtype, device=table.device)
+        grad_w = torch.empty(edges.num_edges, self.weight_numel, dtype=table.dtype, device=table.device)
+        with torch.cuda.device(table.device):
+            _lib.check(
+                L.e3x_tp_gather_scatter_grad_w(
+                    self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(row_x), _lib.ptr(gather_idx),
+                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(edges.row_order),
+                    _lib.ptr(edges.src_rows if gather_idx is edges.edge_src else None),
+                    _lib.ptr(out), _lib.ptr(grad_w), edges.num_edges, table.shape[0], edges.num_nodes,
+                    _lib.stream_ptr(table.device),
+                )  # fmt: skip
+            )
+        return out, grad_w
 
     def gather_scatter_radial(self, table, edge_attr, edge_scalars, w1, w2, act_kind, act_cst, variance_in, variance_out,
                               gather_idx, edges, num_table_rows):
@@ -271,6 +298,11 @@ class _GatherScatterFn(torch.autograd.Function):
         g = g.contiguous()
         need1, need2, needw = ctx.needs_input_grad[:3]
         g1 = g2 = gw = None
+        if need1 and needw and tp.weight_numel and not need2 and node_x.dtype == torch.float32:
+            # d/dnode_x and d/dw from one pass over the weights and one gather of g per edge
+            both = tp._grad_plan("x1", node_x.dtype).gather_scatter_grad_w(g, edge_attr, w, node_x, edges.edge_dst, edges.transposed())
+            if both is not None:
+                return both[0], None, both[1], None, None
         if need1:
             rev = edges.transposed()
             g1 = tp._grad_plan("x1", node_x.dtype).gather_scatter(g, edge_attr, w, edges.edge_dst, rev, g.shape[0])
@@ -574,6 +606,11 @@ class TensorProduct(torch.nn.Module):
         self._grad_plan("x1", dtype)
         if self._live_mode() == "uvu":
             _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(self._plan(dtype).handle))
+            if dtype == torch.float32 and not self.shared_weights and self.weight_numel:
+                # the message-step backward kernel on the transposed plan, where the instruction set fits it
+                rc = _lib.lib().e3x_tp_plan_prepare_gather_scatter_grad_w(self._grad_plan("x1", dtype).handle)
+                if rc != _lib.ERR_INVALID:
+                    _lib.check(rc)
             if dtype != torch.float32 and self.shared_weights and self.weight_numel:  # summed over the batch in fp32
                 _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(self._plan(torch.float32).handle))
         if self._live_mode() == "uvw":

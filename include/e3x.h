@@ -255,6 +255,27 @@ int e3x_tp_backward_w_x2(e3x_plan* plan, const void* x1, const void* x2, const v
                          const void* src, const void* dst, int idx_bits, void* grad_w, void* grad_x2, int64_t E,
                          int64_t num_src_nodes, int64_t num_out_nodes, void* stream);
 
+/* The backward pass of a message step in ONE kernel, called on the TRANSPOSED plan (first input: the messages'
+ * irreps, output: the node features' irreps, same second input and weights) with source and destination exchanged:
+ *   out[n]    = sum over the edges e leaving node n of  plan(table[gather_idx[e]], edge_attr[e], w[e])   (= d/dnode_x)
+ *   grad_w[e] = the gradient of the per-edge weights, which needs the forward input row of the source node:
+ *               row_x[num_out_rows, out_dim] (the node features the forward pass gathered from)
+ * from table = grad_out[num_table_rows, in1_dim] of the forward call.  rowptr / perm (/ row_order) group the edges
+ * by SOURCE node (e3x_csr_build on edge_src); gather_idx = edge_dst, src_rows (may be NULL) = e3x_src_rows_build of
+ * it.  One pass over the weights and one gather of the
+ * output gradient per edge, where e3x_tp_gather_scatter on this plan followed by e3x_tp_backward_w_x2 on the forward
+ * plan makes two of each; out is bit-identical to what e3x_tp_gather_scatter_ordered writes for plans whose lanes
+ * hold fewer than four multiplicity indices.  The gradient of edge_attr is not computed (callers that need it take the
+ * two calls).  The reference obtains all of this by autograd through points_convolution.py:105-106 and the einsums of
+ * e3nn/o3/_tensor_product/_codegen.py:166-187.  fp32, per-edge weights, instruction sets that one kernel covers
+ * (e3x_tp_plan_prepare_gather_scatter_grad_w builds the code object and returns E3X_ERR_INVALID, without a message,
+ * for plans that do not fit); grad_w[E, weight_numel] 16-byte aligned. */
+int e3x_tp_plan_prepare_gather_scatter_grad_w(e3x_plan* plan);
+int e3x_tp_gather_scatter_grad_w(e3x_plan* plan, const void* table, const void* edge_attr, const void* w,
+                                 const void* row_x, const void* gather_idx, int idx_bits, const int32_t* rowptr,
+                                 const int32_t* perm, const int32_t* row_order, const int32_t* src_rows, void* out,
+                                 void* grad_w, int64_t E, int64_t num_table_rows, int64_t num_out_rows, void* stream);
+
 /* Weight gradient of the `uvw` product: grad_w[weight_numel] (shared weights, summed over the batch with
  * fp32 atomics, so the last bits depend on the order) or grad_w[Z, weight_numel] (per-sample weights), from
  * x1[Z, in1_dim], x2[Z, in2_dim], grad_out[Z, out_dim].  The reference obtains it by autograd through

@@ -69,11 +69,20 @@ def test_fused_message_gradients(maker, N, E, idx):
     a2, c2 = node_x.to(DEV).requires_grad_(True), w.to(DEV)
     tp.forward_gather_scatter(a2, attr.to(DEV), c2, edges=edges).backward(cot.to(DEV))
     assert torch.equal(a2.grad, a.grad)
+    # node features and weights but not the edge attributes (training without forces): one kernel on the transposed
+    # plan writes both gradients where the instruction set fits it (a lane group owning a whole row)
+    a4, c4 = node_x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    tp.forward_gather_scatter(a4, attr.to(DEV), c4, edges=edges).backward(cot.to(DEV))
+    assert_close(a4.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dnode_x, one backward kernel")
+    assert_close(c4.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dweight, one backward kernel")
     # negative source indices wrap in the gather; the gradient scatters onto the wrapped rows
     neg = torch.where(torch.arange(E) % 3 == 0, src - N, src)
     a3 = node_x.to(DEV).requires_grad_(True)
     tp.forward_gather_scatter(a3, attr.to(DEV), c2, edges=DstSortedEdges(neg.to(idx).to(DEV), dst.to(idx).to(DEV), N)).backward(cot.to(DEV))
     assert torch.equal(a3.grad, a.grad)
+    a5, c5 = node_x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    tp.forward_gather_scatter(a5, attr.to(DEV), c5, edges=DstSortedEdges(neg.to(idx).to(DEV), dst.to(idx).to(DEV), N)).backward(cot.to(DEV))
+    assert torch.equal(a5.grad, a4.grad) and torch.equal(c5.grad, c4.grad)
 
 
 def test_second_derivatives_raise_instead_of_dropping_terms():
