@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt), keyed by the code object the counters were read
 # on: a kernel that has changed since reports no traffic instead of a stale figure.
 NEQUIP_TRAFFIC_BYTES = {
-    "uvu_b1d11ac75d8b0830d6b145fd": (2 * 1611878 + 56250) * 1024,  # FETCH_SIZE 1611878 x 2 KiB + WRITE_SIZE 56250 KiB
+    "uvu_4b0a501b7a3ff5d049ab11ab": (2 * 1611924 + 56250) * 1024,  # FETCH_SIZE 1611924 x 2 KiB + WRITE_SIZE 56250 KiB
 }
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
@@ -437,8 +437,17 @@ def bench_nequip_backward(args, dev, ctx):
         tp.forward_gather_scatter(a, b, c, edges=edges).backward(cot)
 
     ms = event_time_ms(step, max(5, args.steps // 5), 2)
+    # node features and weights only (an energy-only training step): both gradients come from one kernel
+    a2, c2 = (ctx[k].clone().requires_grad_(True) for k in ("node_x", "w"))
+
+    def step_xw():
+        a2.grad = c2.grad = None
+        tp.forward_gather_scatter(a2, ctx["attr"], c2, edges=edges).backward(cot)
+
+    ms_xw = event_time_ms(step_xw, max(5, args.steps // 5), 2)
     E = ctx["src"].shape[0]
-    return {"edges": E, "ms_forward_backward": ms, "edges_per_s": E / (ms * 1e-3)}
+    return {"edges": E, "ms_forward_backward": ms, "ms_forward_backward_node_features_and_weights": ms_xw,
+            "edges_per_s": E / (ms * 1e-3)}
 
 
 def bench_uvw_backward(args, dev):
