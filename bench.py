@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt), keyed by the code object the counters were read
 # on: a kernel that has changed since reports no traffic instead of a stale figure.
 NEQUIP_TRAFFIC_BYTES = {
-    "uvu_4b0a501b7a3ff5d049ab11ab": (2 * 1611924 + 56250) * 1024,  # FETCH_SIZE 1611924 x 2 KiB + WRITE_SIZE 56250 KiB
+    "uvu_9ad9e6746cebece0b6bb91bb": (2 * 1611871 + 56250) * 1024,  # FETCH_SIZE 1611871 x 2 KiB + WRITE_SIZE 56250 KiB
 }
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
@@ -437,7 +437,7 @@ def bench_nequip_backward(args, dev, ctx):
         tp.forward_gather_scatter(a, b, c, edges=edges).backward(cot)
 
     ms = event_time_ms(step, max(5, args.steps // 5), 2)
-    # node features and weights only (an energy-only training step): both gradients come from one kernel
+    # node features and weights only (an energy-only training step)
     a2, c2 = (ctx[k].clone().requires_grad_(True) for k in ("node_x", "w"))
 
     def step_xw():

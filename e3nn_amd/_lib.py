@@ -71,8 +71,8 @@ _SIGNATURES = {
     "e3x_tp_plan_prepare_backward_w": (c_int, [c_void_p]),
     "e3x_tp_plan_prepare_gather_scatter_grad_w": (c_int, [c_void_p]),
     "e3x_tp_gather_scatter_grad_w": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
-                                             c_void_p]),
+                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                             c_int64, c_void_p]),
     "e3x_tp_backward_w_uvw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "e3x_gate_forward": (c_int, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p]),
     "e3x_gate_backward": (c_int, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p]),

@@ -48,6 +48,7 @@ struct SubKernel {
   // uvu, transposed plan of a message step: the fused kernel that also writes the weight gradient, built on first use
   std::unique_ptr<SubKernel> fused_dw;
   hipFunction_t fn_fused_dw[kMaxDevices] = {nullptr};
+  hipFunction_t fn_fused_dw_x2[kMaxDevices] = {nullptr};  // ... and the gradient of the second input
 };
 
 struct e3x_plan {
@@ -964,7 +965,8 @@ int load_uvu_fused_dw_function(e3x_plan* P, int dev) {
   hipModule_t mod = nullptr;
   hipError_t err = hipModuleLoad(&mod, D->hsaco.c_str());
   if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + D->hsaco + ") failed: " + hipGetErrorString(err));
-  if (hipModuleGetFunction(&D->fn_fused_dw[dev], mod, "e3x_uvu_fused_dw") != hipSuccess)
+  if (hipModuleGetFunction(&D->fn_fused_dw[dev], mod, "e3x_uvu_fused_dw") != hipSuccess ||
+      hipModuleGetFunction(&D->fn_fused_dw_x2[dev], mod, "e3x_uvu_fused_dw_x2") != hipSuccess)
     return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused_dw missing from " + D->hsaco);
   D->module[dev] = mod;
   return E3X_OK;
@@ -1291,8 +1293,8 @@ extern "C" int e3x_tp_plan_prepare_gather_scatter_grad_w(e3x_plan* P) {
 extern "C" int e3x_tp_gather_scatter_grad_w(e3x_plan* P, const void* table, const void* edge_attr, const void* w,
                                             const void* row_x, const void* gather_idx, int idx_bits,
                                             const int32_t* rowptr, const int32_t* perm, const int32_t* row_order,
-                                            const int32_t* src_rows, void* out, void* grad_w, int64_t E,
-                                            int64_t num_table_rows, int64_t num_out_rows, void* stream) {
+                                            const int32_t* src_rows, void* out, void* grad_w, void* grad_x2,
+                                            int64_t E, int64_t num_table_rows, int64_t num_out_rows, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: null plan");
   if (!fused_dw_fits(P))
     return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: needs an all-uvu fp32 plan with per-edge weights that one kernel covers");
@@ -1317,11 +1319,11 @@ extern "C" int e3x_tp_gather_scatter_grad_w(e3x_plan* P, const void* table, cons
   long long n_rows = num_out_rows, n_src = num_table_rows;
   void* args[] = {(void*)&table,  (void*)&edge_attr, (void*)&w,         (void*)&out,    (void*)&gather_idx, (void*)&idx64,
                   (void*)&rowptr, (void*)&perm,      (void*)&row_order, (void*)&n_rows, (void*)&n_src,      (void*)&row_x,
-                  (void*)&grad_w};
+                  (void*)&grad_w, (void*)&grad_x2};
   long long blocks = (n_rows + D->waves_per_block - 1) / D->waves_per_block;
   blocks = (blocks + 7) / 8 * 8;  // the kernel deals contiguous eighths of the rows to the 8 XCDs
   if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: too many rows for one launch");
-  hipError_t err = hipModuleLaunchKernel(D->fn_fused_dw[dev], (unsigned)blocks, 1, 1, 64 * D->waves_per_block, 1, 1, 0, st,
+  hipError_t err = hipModuleLaunchKernel(grad_x2 ? D->fn_fused_dw_x2[dev] : D->fn_fused_dw[dev], (unsigned)blocks, 1, 1, 64 * D->waves_per_block, 1, 1, 0, st,
                                          args, nullptr);
   if (err != hipSuccess)
     return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter_grad_w: launch failed: ") + hipGetErrorString(err));

@@ -132,10 +132,10 @@ class _Plan:
             )
         return out
 
-    def gather_scatter_grad_w(self, table, edge_attr, w, row_x, gather_idx, edges):
-        """On the transposed plan of a message step: ``(gather_scatter(table, ...), grad_w[E, weight_numel])`` from one
-        kernel, ``row_x`` being the forward input rows of the nodes that ``edges`` groups by; None when the plan does
-        not fit that kernel."""
+    def gather_scatter_grad_w(self, table, edge_attr, w, row_x, gather_idx, edges, want_x2=False):
+        """On the transposed plan of a message step: ``(gather_scatter(table, ...), grad_w[E, weight_numel],
+        grad_edge_attr or None)`` from one kernel, ``row_x`` being the forward input rows of the nodes that ``edges``
+        groups by; None when the plan does not fit that kernel."""
         L = _lib.lib()
         if self._fused_grad_w is None:
             rc = L.e3x_tp_plan_prepare_gather_scatter_grad_w(self.handle)
@@ -146,17 +146,18 @@ class _Plan:
             return None
         out = torch.empty(edges.num_nodes, self.out_dim, dtype=table.dtype, device=table.device)
         grad_w = torch.empty(edges.num_edges, self.weight_numel, dtype=table.dtype, device=table.device)
+        grad_x2 = torch.empty_like(edge_attr) if want_x2 else None
         with torch.cuda.device(table.device):
             _lib.check(
                 L.e3x_tp_gather_scatter_grad_w(
                     self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(row_x), _lib.ptr(gather_idx),
                     gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(edges.row_order),
                     _lib.ptr(edges.src_rows if gather_idx is edges.edge_src else None),
-                    _lib.ptr(out), _lib.ptr(grad_w), edges.num_edges, table.shape[0], edges.num_nodes,
+                    _lib.ptr(out), _lib.ptr(grad_w), _lib.ptr(grad_x2), edges.num_edges, table.shape[0], edges.num_nodes,
                     _lib.stream_ptr(table.device),
                 )  # fmt: skip
             )
-        return out, grad_w
+        return out, grad_w, grad_x2
 
     def gather_scatter_radial(self, table, edge_attr, edge_scalars, w1, w2, act_kind, act_cst, variance_in, variance_out,
                               gather_idx, edges, num_table_rows):
@@ -298,11 +299,13 @@ class _GatherScatterFn(torch.autograd.Function):
         g = g.contiguous()
         need1, need2, needw = ctx.needs_input_grad[:3]
         g1 = g2 = gw = None
-        if need1 and needw and tp.weight_numel and not need2 and node_x.dtype == torch.float32:
-            # d/dnode_x and d/dw from one pass over the weights and one gather of g per edge
-            both = tp._grad_plan("x1", node_x.dtype).gather_scatter_grad_w(g, edge_attr, w, node_x, edges.edge_dst, edges.transposed())
-            if both is not None:
-                return both[0], None, both[1], None, None
+        if need1 and needw and tp.weight_numel and node_x.dtype == torch.float32:
+            # every gradient from one pass over the weights and one gather of g per edge
+            res = tp._grad_plan("x1", node_x.dtype).gather_scatter_grad_w(
+                g, edge_attr, w, node_x, edges.edge_dst, edges.transposed(), need2 and edge_attr.shape[1] > 0
+            )
+            if res is not None:
+                return res[0], (res[2] if need2 else None), res[1], None, None
         if need1:
             rev = edges.transposed()
             g1 = tp._grad_plan("x1", node_x.dtype).gather_scatter(g, edge_attr, w, edges.edge_dst, rev, g.shape[0])

@@ -264,9 +264,10 @@ int e3x_tp_backward_w_x2(e3x_plan* plan, const void* x1, const void* x2, const v
  * by SOURCE node (e3x_csr_build on edge_src); gather_idx = edge_dst, src_rows (may be NULL) = e3x_src_rows_build of
  * it.  One pass over the weights and one gather of the
  * output gradient per edge, where e3x_tp_gather_scatter on this plan followed by e3x_tp_backward_w_x2 on the forward
- * plan makes two of each; out is bit-identical to what e3x_tp_gather_scatter_ordered writes for plans whose lanes
- * hold fewer than four multiplicity indices.  The gradient of edge_attr is not computed (callers that need it take the
- * two calls).  The reference obtains all of this by autograd through points_convolution.py:105-106 and the einsums of
+ * plan makes two of each; out agrees with e3x_tp_gather_scatter_ordered to rounding (the same sums per lane group; the groups of a
+ * wavefront are combined by a shuffle butterfly, there sometimes through LDS in another order).  grad_x2[E, in2_dim]
+ * (may be NULL: not computed) is the gradient of edge_attr, summed over the multiplicity indices inside the kernel.
+ * The reference obtains all of this by autograd through points_convolution.py:105-106 and the einsums of
  * e3nn/o3/_tensor_product/_codegen.py:166-187.  fp32, per-edge weights, instruction sets that one kernel covers
  * (e3x_tp_plan_prepare_gather_scatter_grad_w builds the code object and returns E3X_ERR_INVALID, without a message,
  * for plans that do not fit); grad_w[E, weight_numel] 16-byte aligned. */
@@ -274,7 +275,8 @@ int e3x_tp_plan_prepare_gather_scatter_grad_w(e3x_plan* plan);
 int e3x_tp_gather_scatter_grad_w(e3x_plan* plan, const void* table, const void* edge_attr, const void* w,
                                  const void* row_x, const void* gather_idx, int idx_bits, const int32_t* rowptr,
                                  const int32_t* perm, const int32_t* row_order, const int32_t* src_rows, void* out,
-                                 void* grad_w, int64_t E, int64_t num_table_rows, int64_t num_out_rows, void* stream);
+                                 void* grad_w, void* grad_x2, int64_t E, int64_t num_table_rows, int64_t num_out_rows,
+                                 void* stream);
 
 /* Weight gradient of the `uvw` product: grad_w[weight_numel] (shared weights, summed over the batch with
  * fp32 atomics, so the last bits depend on the order) or grad_w[Z, weight_numel] (per-sample weights), from

@@ -68,7 +68,9 @@ def test_fused_message_gradients(maker, N, E, idx):
     # only some inputs require a gradient
     a2, c2 = node_x.to(DEV).requires_grad_(True), w.to(DEV)
     tp.forward_gather_scatter(a2, attr.to(DEV), c2, edges=edges).backward(cot.to(DEV))
-    assert torch.equal(a2.grad, a.grad)
+    # (another kernel than above where one kernel writes every gradient: the lane groups of a wavefront are combined
+    # in another order, so the last bits may differ)
+    assert_close(a2.grad, a.grad.cpu().numpy(), atol=1e-5 * scale(r1), what="d/dnode_x alone")
     # node features and weights but not the edge attributes (training without forces): one kernel on the transposed
     # plan writes both gradients where the instruction set fits it (a lane group owning a whole row)
     a4, c4 = node_x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
@@ -79,7 +81,7 @@ def test_fused_message_gradients(maker, N, E, idx):
     neg = torch.where(torch.arange(E) % 3 == 0, src - N, src)
     a3 = node_x.to(DEV).requires_grad_(True)
     tp.forward_gather_scatter(a3, attr.to(DEV), c2, edges=DstSortedEdges(neg.to(idx).to(DEV), dst.to(idx).to(DEV), N)).backward(cot.to(DEV))
-    assert torch.equal(a3.grad, a.grad)
+    assert torch.equal(a3.grad, a2.grad)
     a5, c5 = node_x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
     tp.forward_gather_scatter(a5, attr.to(DEV), c5, edges=DstSortedEdges(neg.to(idx).to(DEV), dst.to(idx).to(DEV), N)).backward(cot.to(DEV))
     assert torch.equal(a5.grad, a4.grad) and torch.equal(c5.grad, c4.grad)
