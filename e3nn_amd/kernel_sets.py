@@ -213,7 +213,7 @@ def all_tensor_products():
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
                   "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "mfma_full_tiles", "outer_split", "node_fctp", "node_block", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
-                  "unaligned_mfma", "unaligned_offsets", "mixed_modes", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
+                  "unaligned_mfma", "unaligned_offsets", "mixed_modes", "scalar_exact", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
 
 
 def nn_golden():

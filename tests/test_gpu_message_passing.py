@@ -86,6 +86,25 @@ def test_out_of_range_indices_raise_and_empty_graph():
     e = torch.zeros(0, dtype=torch.int64, device=DEV)
     out = tp.forward_gather_scatter(node_x, attr[:0], w[:0], e, e, N)
     assert out.shape == (N, 32) and not out.any()
+    # ... and its backward pass: zero gradients of the right shapes
+    a, b, c = node_x.clone().requires_grad_(True), attr[:0].clone().requires_grad_(True), w[:0].clone().requires_grad_(True)
+    tp.forward_gather_scatter(a, b, c, e, e, N).backward(torch.ones(N, 32, device=DEV))
+    assert a.grad.shape == (N, 32) and not a.grad.any()
+    assert b.grad is None or b.grad.shape == (0, 1)
+    assert c.grad is None or c.grad.shape == (0, 32)
+    # source nodes without edges get a zero gradient row, the others what autograd of the dense form gives
+    src2 = torch.where(src < 3, src + 3, src)  # nodes 0, 1, 2 send nothing
+    a, c = node_x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    tp.forward_gather_scatter(a, attr, c, src2.to(DEV), dst.to(DEV), N).backward(torch.ones(N, 32, device=DEV))
+    assert not a.grad[:3].any() and a.grad[3:].any()
+    ref_x = node_x.clone().requires_grad_(True)
+    ref_w = w.clone().requires_grad_(True)
+    # scalar_exact: 32x0e x 1x0e -> 32x0e, uvu with per-edge weights: message[e, u] = pw * w[e, u] * x[src[e], u] * attr[e, 0]
+    pw = float(tp.instructions[0].path_weight) if hasattr(tp.instructions[0], "path_weight") else 1.0
+    msg = pw * ref_w * ref_x[src2.to(DEV)] * attr
+    torch.zeros(N, 32, device=DEV).index_add(0, dst.to(DEV), msg).sum().backward()
+    assert torch.allclose(a.grad, ref_x.grad, atol=1e-5, rtol=1e-5)
+    assert torch.allclose(c.grad, ref_w.grad, atol=1e-5, rtol=1e-5)
 
 
 def test_run_to_run_bit_reproducible_and_prebuilt_edges():
