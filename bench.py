@@ -338,10 +338,12 @@ def bench_convolution(args, dev, ctx):
         with torch.no_grad():
             return conv(x, node_attr, ctx["src"], ctx["dst"], ctx["attr"], edge_scalars, edges=edges)
 
-    def fwd_bwd():
+    cot = torch.randn(N, conv.irreps_node_output.dim, generator=gen).to(dev)
+
+    def fwd_bwd():  # from a fixed cotangent: no loss function in the timed region
         x.grad = None
         conv.zero_grad(set_to_none=True)
-        conv(x, node_attr, ctx["src"], ctx["dst"], ctx["attr"], edge_scalars, edges=edges).square().sum().backward()
+        conv(x, node_attr, ctx["src"], ctx["dst"], ctx["attr"], edge_scalars, edges=edges).backward(cot)
 
     ms_f = event_time_ms(fwd, max(5, args.steps // 5), 2)
     ms_fb = event_time_ms(fwd_bwd, max(3, args.steps // 10), 1)

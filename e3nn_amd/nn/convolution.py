@@ -18,23 +18,23 @@ from .message import message_instructions
 
 
 class _Mix(torch.autograd.Function):
-    """``sc + ((1 - m) + alpha * m * inv) * conv * inv`` (reference points_convolution.py:110-113 with the division by
-    sqrt(num_neighbors) moved behind lin2 and alpha): two elementwise kernels forward and three backward, where autograd
-    through the separate operations launches a dozen over the [N, channels] arrays."""
+    """``sc + (c0 + alpha * c1) * conv`` with ``c0 = (1 - m) / sqrt(n)``, ``c1 = m / n`` (reference
+    points_convolution.py:110-113 with the division by sqrt(num_neighbors) moved behind lin2 and alpha): two elementwise
+    kernels forward and three backward, where autograd through the separate operations launches a dozen over the
+    [N, channels] arrays."""
 
     @staticmethod
-    def forward(ctx, sc, alpha, conv, m, inv):
-        coeff = torch.addcmul((1 - m) * inv, alpha, m * (inv * inv))  # [N, channels]
-        ctx.save_for_backward(coeff, conv, m)
-        ctx.inv = inv
+    def forward(ctx, sc, alpha, conv, c0, c1):
+        coeff = torch.addcmul(c0, alpha, c1)  # [N, channels]
+        ctx.save_for_backward(coeff, conv, c1)
         return torch.addcmul(sc, coeff, conv)
 
     @staticmethod
     @once_differentiable
     def backward(ctx, g):
-        coeff, conv, m = ctx.saved_tensors
+        coeff, conv, c1 = ctx.saved_tensors
         need_sc, need_alpha, need_conv = ctx.needs_input_grad[:3]
-        g_alpha = ((g * conv) @ (m * (ctx.inv * ctx.inv))).unsqueeze(-1) if need_alpha else None
+        g_alpha = ((g * conv) @ c1).unsqueeze(-1) if need_alpha else None
         return (g if need_sc else None), g_alpha, (g * coeff if need_conv else None), None, None
 
 
@@ -154,4 +154,9 @@ class Convolution(torch.nn.Module):
         else:
             node_conv_out = self.lin2(node_features, node_attr)
             alpha = self.alpha(node_features, node_attr)
-        return _Mix.apply(node_self_connection, alpha, node_conv_out, self.sc.output_mask, inv)
+        m = self.sc.output_mask
+        key = (m.device, m.dtype, m._version, inv)
+        if self.__dict__.get("_mix_key") != key:  # the two constant rows of the mixing, once per device
+            self.__dict__["_mix_key"], self.__dict__["_mix_rows"] = key, ((1 - m) * inv, m * (inv * inv))
+        c0, c1 = self.__dict__["_mix_rows"]
+        return _Mix.apply(node_self_connection, alpha, node_conv_out, c0, c1)
