@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt), keyed by the code object the counters were read
 # on: a kernel that has changed since reports no traffic instead of a stale figure.
 NEQUIP_TRAFFIC_BYTES = {
-    "uvu_9ad9e6746cebece0b6bb91bb": (2 * 1611871 + 56250) * 1024,  # FETCH_SIZE 1611871 x 2 KiB + WRITE_SIZE 56250 KiB
+    "uvu_9a6230a2caf8306da5d9c9f6": (2 * 1611842 + 56250) * 1024,  # FETCH_SIZE 1611842 x 2 KiB + WRITE_SIZE 56250 KiB
 }
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0

@@ -935,40 +935,48 @@ int load_uvu_bwd_functions(e3x_plan* P, int dev) {
 }
 
 // The fused kernel of a transposed message plan that also writes the per-edge weight gradient: fp32, per-edge
-// weights, one kernel and one chunk cover the instruction set (a lane group owns a whole row).
+// weights; every kernel of the plan (instruction sets split over disjoint output irreps have several) gets a
+// companion, and in each a lane group must own a whole row (one chunk).
 bool fused_dw_fits(const e3x_plan* P) {
-  return env_int("E3X_UVU_FUSED_DW", 1) != 0 && P->family == "uvu" && P->dtype == E3X_F32 && !P->shared_weights && P->weight_numel > 0 && P->subs.size() == 1 &&
-         P->subs[0]->chunks == 1 && P->subs[0]->path_ids.size() == P->paths.size() && !P->zero_fill;
+  if (!(env_int("E3X_UVU_FUSED_DW", 1) != 0 && P->family == "uvu" && P->dtype == E3X_F32 && !P->shared_weights &&
+        P->weight_numel > 0 && !P->subs.empty()))
+    return false;
+  for (const auto& K : P->subs)
+    if (K->chunks != 1) return false;
+  return true;
 }
 
 int prepare_uvu_fused_dw(e3x_plan* P) {
   std::lock_guard<std::mutex> lock(P->mu);
-  SubKernel* K = P->subs[0].get();
-  if (K->fused_dw) return E3X_OK;
-  std::unique_ptr<SubKernel> D(new SubKernel);
-  D->path_ids = K->path_ids;
-  std::string src;
-  const std::string extra = "#define E3X_UVU_FUSED_DW 1\n";
-  int rc;
-  // (naming the template switches off the row staging and the row reduction through LDS, which this kernel does not use)
-  if ((rc = build_uvu_source(*P, *D, &src, false, &extra, e3x::kTplUvu))) return rc;
-  if (D->chunks != 1) return fail(E3X_ERR_INVALID, "fused weight gradient: the instruction set needs several chunks");
-  if ((rc = e3x::get_code_object("uvu_fdw", src, &D->key, &D->hsaco))) return rc;
-  K->fused_dw = std::move(D);
+  for (auto& K : P->subs) {
+    if (K->fused_dw) continue;
+    std::unique_ptr<SubKernel> D(new SubKernel);
+    D->path_ids = K->path_ids;
+    std::string src;
+    const std::string extra = "#define E3X_UVU_FUSED_DW 1\n";
+    int rc;
+    // (naming the template switches off the row staging and the row reduction through LDS, which this kernel does not use)
+    if ((rc = build_uvu_source(*P, *D, &src, false, &extra, e3x::kTplUvu))) return rc;
+    if (D->chunks != 1) return fail(E3X_ERR_INVALID, "fused weight gradient: the instruction set needs several chunks");
+    if ((rc = e3x::get_code_object("uvu_fdw", src, &D->key, &D->hsaco))) return rc;
+    K->fused_dw = std::move(D);
+  }
   return E3X_OK;
 }
 
 int load_uvu_fused_dw_function(e3x_plan* P, int dev) {
   std::lock_guard<std::mutex> lock(P->mu);
-  SubKernel* D = P->subs[0]->fused_dw.get();
-  if (D->module[dev]) return E3X_OK;
-  hipModule_t mod = nullptr;
-  hipError_t err = hipModuleLoad(&mod, D->hsaco.c_str());
-  if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + D->hsaco + ") failed: " + hipGetErrorString(err));
-  if (hipModuleGetFunction(&D->fn_fused_dw[dev], mod, "e3x_uvu_fused_dw") != hipSuccess ||
-      hipModuleGetFunction(&D->fn_fused_dw_x2[dev], mod, "e3x_uvu_fused_dw_x2") != hipSuccess)
-    return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused_dw missing from " + D->hsaco);
-  D->module[dev] = mod;
+  for (auto& K : P->subs) {
+    SubKernel* D = K->fused_dw.get();
+    if (D->module[dev]) continue;
+    hipModule_t mod = nullptr;
+    hipError_t err = hipModuleLoad(&mod, D->hsaco.c_str());
+    if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + D->hsaco + ") failed: " + hipGetErrorString(err));
+    if (hipModuleGetFunction(&D->fn_fused_dw[dev], mod, "e3x_uvu_fused_dw") != hipSuccess ||
+        hipModuleGetFunction(&D->fn_fused_dw_x2[dev], mod, "e3x_uvu_fused_dw_x2") != hipSuccess)
+      return fail(E3X_ERR_HIP, "kernel e3x_uvu_fused_dw missing from " + D->hsaco);
+    D->module[dev] = mod;
+  }
   return E3X_OK;
 }
 
@@ -1297,7 +1305,7 @@ extern "C" int e3x_tp_gather_scatter_grad_w(e3x_plan* P, const void* table, cons
                                             int64_t E, int64_t num_table_rows, int64_t num_out_rows, void* stream) {
   if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: null plan");
   if (!fused_dw_fits(P))
-    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: needs an all-uvu fp32 plan with per-edge weights that one kernel covers");
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: needs an all-uvu fp32 plan with per-edge weights whose kernels each cover a row with one chunk");
   if (idx_bits != 32 && idx_bits != 64) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: idx_bits must be 32 or 64");
   if (E < 0 || num_table_rows < 0 || num_out_rows < 0) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: negative size");
   if (num_out_rows == 0) return E3X_OK;
@@ -1309,7 +1317,7 @@ extern "C" int e3x_tp_gather_scatter_grad_w(e3x_plan* P, const void* table, cons
   if ((rc = current_device(&dev))) return rc;
   if ((rc = prepare_uvu_fused_dw(P))) return rc;
   if ((rc = load_uvu_fused_dw_function(P, dev))) return rc;
-  SubKernel* D = P->subs[0]->fused_dw.get();
+  if (P->zero_fill && (rc = zero_output(P, out, num_out_rows, st))) return rc;
   // index mode of the kernel: 0 / 1 = the caller's int32 / int64 list indexed by edge id, 2 = src_rows
   int idx64 = idx_bits == 64;
   if (src_rows) {
@@ -1317,16 +1325,21 @@ extern "C" int e3x_tp_gather_scatter_grad_w(e3x_plan* P, const void* table, cons
     idx64 = 2;
   }
   long long n_rows = num_out_rows, n_src = num_table_rows;
+  int x2_accumulate = 0;  // the first kernel writes the edge-attribute gradient, the others add their paths' share
   void* args[] = {(void*)&table,  (void*)&edge_attr, (void*)&w,         (void*)&out,    (void*)&gather_idx, (void*)&idx64,
                   (void*)&rowptr, (void*)&perm,      (void*)&row_order, (void*)&n_rows, (void*)&n_src,      (void*)&row_x,
-                  (void*)&grad_w, (void*)&grad_x2};
-  long long blocks = (n_rows + D->waves_per_block - 1) / D->waves_per_block;
-  blocks = (blocks + 7) / 8 * 8;  // the kernel deals contiguous eighths of the rows to the 8 XCDs
-  if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: too many rows for one launch");
-  hipError_t err = hipModuleLaunchKernel(grad_x2 ? D->fn_fused_dw_x2[dev] : D->fn_fused_dw[dev], (unsigned)blocks, 1, 1, 64 * D->waves_per_block, 1, 1, 0, st,
-                                         args, nullptr);
-  if (err != hipSuccess)
-    return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter_grad_w: launch failed: ") + hipGetErrorString(err));
+                  (void*)&grad_w, (void*)&grad_x2,   (void*)&x2_accumulate};
+  for (auto& K : P->subs) {
+    SubKernel* D = K->fused_dw.get();
+    long long blocks = (n_rows + D->waves_per_block - 1) / D->waves_per_block;
+    blocks = (blocks + 7) / 8 * 8;  // the kernel deals contiguous eighths of the rows to the 8 XCDs
+    if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_grad_w: too many rows for one launch");
+    hipError_t err = hipModuleLaunchKernel(grad_x2 ? D->fn_fused_dw_x2[dev] : D->fn_fused_dw[dev], (unsigned)blocks, 1, 1,
+                                           64 * D->waves_per_block, 1, 1, 0, st, args, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter_grad_w: launch failed: ") + hipGetErrorString(err));
+    x2_accumulate = 1;
+  }
   return E3X_OK;
 }
 

@@ -268,8 +268,9 @@ int e3x_tp_backward_w_x2(e3x_plan* plan, const void* x1, const void* x2, const v
  * wavefront are combined by a shuffle butterfly, there sometimes through LDS in another order).  grad_x2[E, in2_dim]
  * (may be NULL: not computed) is the gradient of edge_attr, summed over the multiplicity indices inside the kernel.
  * The reference obtains all of this by autograd through points_convolution.py:105-106 and the einsums of
- * e3nn/o3/_tensor_product/_codegen.py:166-187.  fp32, per-edge weights, instruction sets that one kernel covers
- * (e3x_tp_plan_prepare_gather_scatter_grad_w builds the code object and returns E3X_ERR_INVALID, without a message,
+ * e3nn/o3/_tensor_product/_codegen.py:166-187.  fp32, per-edge weights, multiplicities that one lane group of a
+ * wavefront covers (instruction sets that run as several kernels over disjoint output irreps launch as many here)
+ * (e3x_tp_plan_prepare_gather_scatter_grad_w builds the code objects and returns E3X_ERR_INVALID, without a message,
  * for plans that do not fit); grad_w[E, weight_numel] 16-byte aligned. */
 int e3x_tp_plan_prepare_gather_scatter_grad_w(e3x_plan* plan);
 int e3x_tp_gather_scatter_grad_w(e3x_plan* plan, const void* table, const void* edge_attr, const void* w,
