@@ -262,8 +262,19 @@ def bench_mace(args, dev, dtype=torch.float32, variant="A"):
     ms = event_time_ms(lambda: tp.forward_gather_scatter(node_x, attr, w, edges=edges), max(3, args.steps // 4), 2)
     fb = 2 if dtype == torch.bfloat16 else 4
     b = E * (fb * tp.weight_numel + fb * 16 + 2 * 4) + N * fb * (tp.irreps_in1.dim + tp.irreps_out.dim)
-    return {"edges": E, "nodes": N, "ms": ms, "edges_per_s": E / (ms * 1e-3), "achieved_gbs": b / (ms * 1e-3) / 1e9,
-            "roofline_frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "bytes_per_launch": b}  # fmt: skip
+    out = {"edges": E, "nodes": N, "ms": ms, "edges_per_s": E / (ms * 1e-3), "achieved_gbs": b / (ms * 1e-3) / 1e9,
+           "roofline_frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "bytes_per_launch": b}  # fmt: skip
+    if dtype == torch.float32 and variant == "A":
+        # forward + backward with respect to node features, edge attributes and weights, from a fixed cotangent
+        a, bb, c = (t.clone().requires_grad_(True) for t in (node_x, attr, w))
+        cot = torch.randn(N, tp.irreps_out.dim, generator=gen).to(dev)
+
+        def step():
+            a.grad = bb.grad = c.grad = None
+            tp.forward_gather_scatter(a, bb, c, edges=edges).backward(cot)
+
+        out["ms_forward_backward"] = event_time_ms(step, max(3, args.steps // 10), 1)
+    return out
 
 
 def bench_uvw(args, dev, dtype=torch.float32):
