@@ -702,6 +702,12 @@ int build_uvw_node_source(e3x_plan& P, std::string* src) {
   for (const auto& p : P.paths) w_aligned = w_aligned && P.out[p.out].mul % 4 == 0 && p.woff % 4 == 0;
   s << "constexpr bool W_ALIGNED = " << (w_aligned ? "true" : "false") << ";\n";
   s << "constexpr int MAX_BLOCKS = " << max_blocks << ";\n";
+  {
+    // matrix steps on split operands (see the template) where every input multiplicity is a multiple of 16
+    bool split = true;
+    for (const auto& p : P.paths) split = split && P.in1[p.in1].mul % 16 == 0;
+    if (env_int("E3X_NODE_SPLIT", split ? 1 : 0) && split) s << "#define E3X_NODE_SPLIT 1\n";
+  }
   // workgroups per CU the register budget is set for: three when their weights fit (160 KB of LDS per CU)
   s << "constexpr int MIN_WGS = " << env_int("E3X_NODE_WGS", max_blocks <= 48 && max_d <= 5 ? 3 : 2) << ";\n";
   s << "}  // namespace cfg\n";
