@@ -293,13 +293,48 @@ def bench_uvw(args, dev, dtype=torch.float32):
     f_min = 2 * Z * 128**3 * 21  # cheapest contraction order per path: sum of min(2l1+1, 2l2+1, 2l3+1) = 21
     f_gemm = 2 * Z * 128**3 * 35  # outer-product order: sum of (2l3+1) = 35
     peak = BF16_MFMA_PEAK_TFLOPS if dtype == torch.bfloat16 else FP32_MFMA_PEAK_TFLOPS
+    arithmetic = tp._plan(dtype).arithmetic
     out = {"rows": Z, "ms": ms, "tflops_fmin": f_min / (ms * 1e-3) / 1e12, "tflops_fgemm_equiv": f_gemm / (ms * 1e-3) / 1e12,
-           "roofline": {"bound": "mfma", "achieved": f_min / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
-                        "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
-    if dtype == torch.float32 and os.environ.get("E3X_UVW_SPLIT", "1") != "0":
-        out["arithmetic"] = ("matrix passes: six bf16 MFMA products of three-way split operands, fp32 accumulation "
-                             "(fp32-accurate); tflops / frac count the 2*m*n*k flops of the fp32 product against the fp32 MFMA peak")
+           "roofline": {"bound": "mfma", "instruction": arithmetic, "achieved": f_min / (ms * 1e-3) / 1e12, "peak": peak,
+                        "unit": "TFLOP/s", "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
+    if dtype == torch.float32:
+        out["roofline"].update(split_operand_fractions(arithmetic, f_min, ms))
+        if "split" in arithmetic:  # the same product on the fp32 matrix instruction, as a plan of its own
+            out["ms_fp32_instruction"] = with_env("E3X_UVW_SPLIT", "0", lambda: time_fresh_plan(ks.cfg5, tp.weight, x1, x2))
+            out["roofline"]["frac_on_fp32_instruction"] = f_min / (out["ms_fp32_instruction"] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS
     return out
+
+
+def split_operand_fractions(arithmetic, flops, ms):
+    """Both readings of an fp32 product that runs as six bf16 matrix products of three-way split operands:
+    ``frac`` prices the 2mnk flops of the fp32 product against the fp32 matrix peak (what the caller gets);
+    ``frac_of_bf16_peak_executed`` prices the six products the matrix cores execute against the peak of the instruction
+    they execute.  On the fp32 instruction the two coincide and only ``frac`` is reported."""
+    if "split" not in arithmetic:
+        return {}
+    return {"frac_fp32_equivalent": flops / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+            "frac_of_bf16_peak_executed": 6 * flops / (ms * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS}  # fmt: skip
+
+
+def with_env(name, value, fn):
+    """Runs ``fn`` with one environment variable set (the kernel generator reads its switches at plan creation)."""
+    old = os.environ.get(name)
+    os.environ[name] = value
+    try:
+        return fn()
+    finally:
+        if old is None:
+            del os.environ[name]
+        else:
+            os.environ[name] = old
+
+
+def time_fresh_plan(maker, weight, x1, x2):
+    tp = maker().to(x1.device)
+    with torch.no_grad():
+        tp.weight.copy_(weight)
+    assert "split" not in tp._plan(torch.float32).arithmetic
+    return event_time_ms(lambda: tp(x1, x2), 3, 1)
 
 
 def bench_nequip_cube40(args, dev):
@@ -486,10 +521,23 @@ def bench_uvw_backward(args, dev):
     a, b = x1.detach(), x2.detach()
     ms_dw = event_time_ms(lambda: plan.backward_w_uvw(a, b, cot, True), 3, 1)
     f_min = 2 * Z * 128**3 * 21
-    return {"rows": Z, "ms_forward_backward": ms, "ms_weight_gradient": ms_dw,
-            "arithmetic": "as uvw_dense_fp32: split-operand bf16 MFMA products, fp32-accurate, priced against the fp32 MFMA peak",
-            "roofline_weight_gradient": {"bound": "mfma", "achieved": f_min / (ms_dw * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
-                                         "unit": "TFLOP/s", "frac": f_min / (ms_dw * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}}  # fmt: skip
+    arithmetic = plan.arithmetic_weight_gradient
+    roof = {"bound": "mfma", "instruction": arithmetic, "achieved": f_min / (ms_dw * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": f_min / (ms_dw * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}  # fmt: skip
+    roof.update(split_operand_fractions(arithmetic, f_min, ms_dw))
+    out = {"rows": Z, "ms_forward_backward": ms, "ms_weight_gradient": ms_dw, "roofline_weight_gradient": roof}
+    if "split" in arithmetic:
+
+        def fp32_instruction():
+            tp2 = ks.cfg5().to(dev)
+            plan2 = tp2._plan(torch.float32)
+            ms2 = event_time_ms(lambda: plan2.backward_w_uvw(a, b, cot, True), 3, 1)
+            assert "split" not in plan2.arithmetic_weight_gradient
+            return ms2
+
+        out["ms_weight_gradient_fp32_instruction"] = with_env("E3X_DW_SPLIT", "0", fp32_instruction)
+        roof["frac_on_fp32_instruction"] = f_min / (out["ms_weight_gradient_fp32_instruction"] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS
+    return out
 
 
 def main():

@@ -43,6 +43,7 @@ _SIGNATURES = {
     "e3x_tp_plan_destroy": (c_int, [c_void_p]),
     "e3x_tp_plan_info": (c_int, [c_void_p, ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), ctypes.POINTER(c_int64),
                                  ctypes.POINTER(c_int64), ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(ctypes.c_char_p)]),
+    "e3x_tp_plan_arithmetic": (ctypes.c_char_p, [c_void_p, c_int]),
     "e3x_tp_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "e3x_tp_forward_workspace_bytes": (c_size_t, [c_void_p]),
     "e3x_tp_forward_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_size_t, c_void_p]),

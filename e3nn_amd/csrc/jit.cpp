@@ -2,8 +2,10 @@
 //
 // A specialised kernel = generated constexpr tables (one instruction set) + a fixed
 // hand-written device template.  The code object is compiled once with the system HIP
-// compiler and kept under the cache directory, keyed by a hash of the full source text
-// and the compiler flags, so identical instruction sets never compile twice.
+// compiler and kept under the cache directory, keyed by a hash of the full source text,
+// the compiler flags and the compiler's identity (what it prints for --version), so
+// identical instruction sets never compile twice and a compiler upgrade never reuses
+// code objects of the old one.
 #include <atomic>
 #include <dlfcn.h>
 #include <fcntl.h>
@@ -16,6 +18,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
+#include <mutex>
 #include <sstream>
 
 #include "e3x_internal.h"
@@ -59,11 +62,76 @@ static std::string find_compiler() {
   return "hipcc";
 }
 
+// What identifies the compiler in the cache key: $E3X_COMPILER_ID when set (a deployment that ships a prebuilt cache
+// and no compiler names the one that built it), else the first two lines of `<compiler> --version` (HIP version and
+// clang version with its commit).  The compiler is asked once per installation, not per process: the answer is kept
+// in <cache>/compiler_id behind a signature of the installation (resolved paths and sizes of the driver and of the
+// clang++ it runs), and a process whose compiler still has that signature reads it from there without starting a
+// child process.
+static std::string installation_signature(const std::string& cc) {
+  std::string sig;
+  auto add = [&](const std::string& p) {
+    char real[4096];
+    struct stat st;
+    if (::realpath(p.c_str(), real) && ::stat(real, &st) == 0) sig += std::string(real) + ":" + std::to_string((long long)st.st_size) + ";";
+  };
+  add(cc);
+  char real[4096];
+  if (::realpath(cc.c_str(), real)) {
+    std::string dir = real;
+    size_t s = dir.rfind('/');
+    if (s != std::string::npos) add(dir.substr(0, s) + "/../lib/llvm/bin/clang++");
+  }
+  return sig.empty() ? cc : sig;
+}
+
+static const std::string& compiler_identity(const std::string& cc) {
+  static std::once_flag once;
+  static std::string id;
+  std::call_once(once, [&] {
+    if (const char* env = std::getenv("E3X_COMPILER_ID")) {
+      id = env;
+      return;
+    }
+    const std::string sig = installation_signature(cc), note = cache_dir() + "/compiler_id";
+    {
+      std::ifstream f(note);
+      std::string first;
+      if (f && std::getline(f, first) && first == sig) {
+        std::stringstream rest;
+        rest << f.rdbuf();
+        id = rest.str();
+        if (!id.empty()) return;
+      }
+    }
+    std::string cmd;
+    for (char c : cc) cmd += (c == '\'') ? std::string("'\\''") : std::string(1, c);
+    cmd = "'" + cmd + "' --version 2>/dev/null";
+    if (FILE* f = ::popen(cmd.c_str(), "r")) {
+      char line[512];
+      for (int n = 0; n < 2 && std::fgets(line, sizeof(line), f); n++) id += line;
+      ::pclose(f);
+    }
+    if (id.empty()) return;  // no compiler to ask: keys carry no compiler identity and nothing can be compiled anyway
+    ::mkdir(cache_dir().c_str(), 0755);
+    char tag[64];
+    std::snprintf(tag, sizeof(tag), ".tmp%d", (int)getpid());
+    std::ofstream f(note + tag);
+    if (f) {
+      f << sig << "\n" << id;
+      f.close();
+      std::rename((note + tag).c_str(), note.c_str());
+    }
+  });
+  return id;
+}
+
 int get_code_object(const std::string& family, const std::string& source, std::string* key_out,
                     std::string* path_out) {
   std::string flags;
   for (const char* f : kFlags) flags += std::string(f) + " ";
-  const uint64_t h1 = fnv1a(source), h2 = fnv1a(flags + source, 0x9e3779b97f4a7c15ULL);
+  const std::string cc = find_compiler();
+  const uint64_t h1 = fnv1a(source), h2 = fnv1a(compiler_identity(cc) + flags + source, 0x9e3779b97f4a7c15ULL);
   char key[64];
   std::snprintf(key, sizeof(key), "%s_%016llx%08llx", family.c_str(), (unsigned long long)h1,
                 (unsigned long long)(h2 & 0xffffffffULL));
@@ -90,7 +158,6 @@ int get_code_object(const std::string& family, const std::string& source, std::s
     if (!f) return fail(E3X_ERR_COMPILE, "cannot write " + src_path);
     f << source;
   }
-  const std::string cc = find_compiler();
   std::vector<std::string> args = {cc};
   for (const char* f : kFlags) args.push_back(f);
   args.push_back("-o");

@@ -58,6 +58,8 @@ struct e3x_plan {
   int shared_weights = 1, dtype = E3X_F32;
   int64_t in1_dim = 0, in2_dim = 0, out_dim = 0, weight_numel = 0;
   std::string family, key;
+  // which instruction forms the products, forward and in the uvw weight gradient (the latter once that kernel is built)
+  std::string arithmetic = "fp32 vector ALU", arithmetic_dw;
   bool zero_fill = false;  // some output irrep is reached by no instruction
   int n_targets = 0;       // uvw_mfma: grid.y
   std::vector<int> node_tile_rows;  // uvw_node: rows per workgroup of each target, in grid order
@@ -557,6 +559,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
     if (P.in1[p.in1].mul % 64 || P.in2[p.in2].mul % 64 || P.out[p.out].mul % 64) full = false;
   const int split = P.dtype == E3X_F32 ? env_int("E3X_UVW_SPLIT", full ? 1 : 0) : 0;
   if (split) s << "#define E3X_UVW_SPLIT 1\n";
+  P.arithmetic = P.dtype != E3X_F32 ? "bf16 matrix instruction" : split ? "bf16 matrix instruction, six products of three-way split operands" : "fp32 matrix instruction";
   if (P.dtype == E3X_F32) s << "#define E3X_UVW_KC " << env_int("E3X_UVW_KC", split ? 16 : 32) << "\n";
   if (env_int("E3X_UVW_KS", 0)) s << "#define E3X_UVW_KS " << env_int("E3X_UVW_KS", 0) << "\n";
   if (env_int("E3X_UVW_WPE", wt == 128 ? 2 : 0)) s << "#define E3X_UVW_WPE " << env_int("E3X_UVW_WPE", wt == 128 ? 2 : 0) << "\n";
@@ -706,7 +709,9 @@ int build_uvw_node_source(e3x_plan& P, std::string* src) {
     // matrix steps on split operands (see the template) where every input multiplicity is a multiple of 16
     bool split = true;
     for (const auto& p : P.paths) split = split && P.in1[p.in1].mul % 16 == 0;
-    if (env_int("E3X_NODE_SPLIT", split ? 1 : 0) && split) s << "#define E3X_NODE_SPLIT 1\n";
+    split = split && env_int("E3X_NODE_SPLIT", 1) != 0;
+    if (split) s << "#define E3X_NODE_SPLIT 1\n";
+    P.arithmetic = split ? "bf16 matrix instruction, six products of three-way split operands" : "fp32 matrix instruction";
   }
   // workgroups per CU the register budget is set for: three when their weights fit (160 KB of LDS per CU)
   s << "constexpr int MIN_WGS = " << env_int("E3X_NODE_WGS", max_blocks <= 48 && max_d <= 5 ? 3 : 2) << ";\n";
@@ -756,7 +761,9 @@ int build_uvw_mfma_dw_source(e3x_plan& P, std::string* src) {
       const bool paired = pairing && c.mul == 32 && O % 2 == 0 && !synth_a;
       if (!paired && ((k_is_x2 ? b.mul : a.mul) % 64 || c.mul % 64)) full = false;
     }
-    s << "#define E3X_DW_SPLIT " << env_int("E3X_DW_SPLIT", full ? 1 : 0) << "\n";
+    const int split = env_int("E3X_DW_SPLIT", full ? 1 : 0);
+    s << "#define E3X_DW_SPLIT " << split << "\n";
+    P.arithmetic_dw = split ? "bf16 matrix instruction, six products of three-way split operands" : "fp32 matrix instruction";
   }
   if (std::getenv("E3X_DW_OCC")) s << "#define E3X_DW_OCC " << env_int("E3X_DW_OCC", 3) << "\n";
   int n_nz = 0, n_path = 0, dkmax = 1, drmax = 1;
@@ -1126,6 +1133,11 @@ extern "C" int e3x_tp_plan_info(const e3x_plan* plan, int64_t* weight_numel, int
   if (family) *family = plan->family.c_str();
   if (cache_key) *cache_key = plan->key.c_str();
   return E3X_OK;
+}
+
+extern "C" const char* e3x_tp_plan_arithmetic(const e3x_plan* plan, int which) {
+  if (!plan) return "";
+  return which == 0 ? plan->arithmetic.c_str() : plan->arithmetic_dw.c_str();
 }
 
 static int zero_output(e3x_plan* P, void* out, int64_t rows, hipStream_t st) {

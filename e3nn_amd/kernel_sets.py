@@ -167,6 +167,11 @@ def mixed_modes(**extra):
     return o3.TensorProduct("4x0e+4x1o", "4x0e+3x1o+4x1e", "4x0e+4x1o+3x1e+4x0e+1x0o", ins, shared_weights=False, **extra)
 
 
+def right_small():
+    # a small fully connected product with right() compiled: the matrices [irreps_in1.dim, irreps_out.dim] per sample
+    return o3.FullyConnectedTensorProduct("4x0e+4x1o", "0e+1o", "4x0e+4x1o+2x2e", compile_right=True)
+
+
 def scalar_exact():
     # 1x1 Clebsch-Gordan, path weight 1: products and sums of small integers are exact in fp32
     return message_tensor_product("32x0e", "0e", irreps_out="32x0e")
@@ -205,6 +210,7 @@ def all_tensor_products():
         ("unaligned_offsets", unaligned_offsets(), (torch.float32,)),
         ("mixed_modes", mixed_modes(), (torch.float32,)),
         ("scalar_exact", scalar_exact(), (torch.float32,)),
+        ("right_small", right_small(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),
     ]
     return out
@@ -348,3 +354,17 @@ def prebuild(verbose=True, workers=6):
         for name, keys in pool.map(build, jobs):
             if verbose:
                 print(f"{name:40s} {' '.join(keys)}", flush=True)
+    # the benchmark times config 5 on the fp32 matrix instruction beside the split-operand default; the generator reads
+    # its switches from the environment at plan creation, so these two are built here, after the threads are done
+    from . import _lib
+
+    saved = {k: os.environ.get(k) for k in ("E3X_UVW_SPLIT", "E3X_DW_SPLIT")}
+    os.environ.update({k: "0" for k in saved})
+    try:
+        plan = cfg5()._plan(torch.float32)
+        _lib.check(_lib.lib().e3x_tp_plan_prepare_backward_w(plan.handle))
+        if verbose:
+            print(f"{'kernel cfg5 (fp32 matrix instruction)':40s} {plan.key} / {plan.arithmetic} / {plan.arithmetic_weight_gradient}", flush=True)
+    finally:
+        for k, v in saved.items():
+            os.environ.pop(k) if v is None else os.environ.__setitem__(k, v)

@@ -46,20 +46,14 @@ class Linear(torch.nn.Module):
             raise ValueError("Linear: f_in and f_out come together")
         self.f_in, self.f_out = f_in, f_out
         irreps_in, irreps_out = Irreps(irreps_in), Irreps(irreps_out)
-        if instructions is None:
-            instructions = [
-                (i_in, i_out)
-                for i_in, (_, ir_in) in enumerate(irreps_in)
-                for i_out, (_, ir_out) in enumerate(irreps_out)
-                if ir_in == ir_out
-            ]
-        for i_in, i_out in instructions:
-            if not i_in < len(irreps_in):
-                raise IndexError(f"{i_in} is not a valid index for irreps_in")
-            if not i_out < len(irreps_out):
-                raise IndexError(f"{i_out} is not a valid index for irreps_out")
-            if irreps_in[i_in].ir != irreps_out[i_out].ir:
-                raise ValueError(f"{i_in} and {i_out} do not have the same irrep")
+        if instructions is None:  # every pair of blocks that carry the same irrep
+            instructions = [(a, b) for a, x in enumerate(irreps_in) for b, y in enumerate(irreps_out) if x.ir == y.ir]
+        for a, b in instructions:
+            for index, irreps, name in ((a, irreps_in, "irreps_in"), (b, irreps_out, "irreps_out")):
+                if index >= len(irreps):
+                    raise IndexError(f"{index} is not a valid index for {name}")
+            if irreps_in[a].ir != irreps_out[b].ir:
+                raise ValueError(f"{a} and {b} do not have the same irrep")
 
         def alpha(i_in, i_out) -> float:
             x = sum(irreps_in[a if path_normalization == "element" else i_in].mul for a, b in instructions if b == i_out)
@@ -70,23 +64,19 @@ class Linear(torch.nn.Module):
             Instruction(i_in, i_out, (irreps_in[i_in].mul, irreps_out[i_out].mul), alpha(i_in, i_out) ** (-0.5))
             for i_in, i_out in instructions
         ]
-        if biases is None:
-            biases = len(irreps_out) * (False,)
-        if isinstance(biases, bool):
-            biases = [biases and ir.is_scalar() for _, ir in irreps_out]
+        if biases is None or isinstance(biases, bool):  # one flag: a bias on every scalar output block
+            biases = [bool(biases) and ir.is_scalar() for _, ir in irreps_out]
         assert len(biases) == len(irreps_out)
-        assert all(ir.is_scalar() or (not b) for b, (_, ir) in zip(biases, irreps_out))
+        assert all(ir.is_scalar() for flag, (_, ir) in zip(biases, irreps_out) if flag), "only scalars take a bias"
         self._bias_slices = [sl for b, sl in zip(biases, irreps_out.slices()) if b]
         self.instructions += [
             Instruction(-1, i_out, (mul_ir.dim,), 1.0) for i_out, (b, mul_ir) in enumerate(zip(biases, irreps_out)) if b
         ]
 
-        if shared_weights is False and internal_weights is None:
-            internal_weights = False
-        if shared_weights is None:
-            shared_weights = True
-        if internal_weights is None:
-            internal_weights = True
+        # weights are shared over the batch unless the caller says otherwise, and the module owns them exactly when
+        # they are shared (unless the caller says otherwise); per-sample weights cannot be parameters
+        shared_weights = True if shared_weights is None else bool(shared_weights)
+        internal_weights = shared_weights if internal_weights is None else bool(internal_weights)
         assert shared_weights or not internal_weights
         self.internal_weights, self.shared_weights = internal_weights, shared_weights
         self.irreps_in, self.irreps_out = irreps_in, irreps_out

@@ -82,6 +82,7 @@ class _Plan:
         _lib.check(L.e3x_tp_plan_info(handle, ctypes.byref(wn), None, None, None, ctypes.byref(fam), ctypes.byref(key)))
         self.weight_numel, self.family, self.key = wn.value, fam.value.decode(), key.value.decode()
         self.out_dim = irreps_out.dim
+        self.arithmetic = L.e3x_tp_plan_arithmetic(handle, 0).decode()  # which instruction forms the products
         self._fused_grad_w = None  # whether the plan has the message-step backward kernel; asked on first use
 
     def __del__(self):
@@ -175,6 +176,11 @@ class _Plan:
             return None
         _lib.check(rc)
         return out
+
+    @property
+    def arithmetic_weight_gradient(self):
+        """Instruction of the matrix-core ``uvw`` weight gradient; "" before that kernel has been built."""
+        return _lib.lib().e3x_tp_plan_arithmetic(self.handle, 1).decode()
 
     def backward_w_uvw(self, x1, x2, grad_out, shared_weights):
         shape = (self.weight_numel,) if shared_weights else (x1.shape[0], self.weight_numel)

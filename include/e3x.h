@@ -119,6 +119,13 @@ int e3x_tp_plan_destroy(e3x_plan* plan);
 int e3x_tp_plan_info(const e3x_plan* plan, int64_t* weight_numel, int64_t* in1_dim, int64_t* in2_dim,
                      int64_t* out_dim, const char** family, const char** cache_key);
 
+/* Which instruction forms the products of the plan's kernels: "fp32 vector ALU", "fp32 matrix instruction",
+ * "bf16 matrix instruction" (bf16 storage) or "bf16 matrix instruction, six products of three-way split operands"
+ * (fp32 storage, fp32-accurate; see e3x_tp_forward).  which = 0: forward; which = 1: the "uvw" weight gradient on the
+ * matrix cores, "" until that kernel has been built (e3x_tp_plan_prepare_backward_w).  No counterpart in the
+ * reference; benchmarks use it to state the peak a kernel is measured against.  The string lives as long as the plan. */
+const char* e3x_tp_plan_arithmetic(const e3x_plan* plan, int which);
+
 /* out[Z, out_dim] = TP(x1[Z, in1_dim], x2[Z, in2_dim], w).  Replaces the generated
  * module called at e3nn/o3/_tensor_product/_tensor_product.py:554
  * (contraction: _codegen.py:148-187, path weights :312, sum/cat :327-343).

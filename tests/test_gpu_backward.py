@@ -37,11 +37,11 @@ def test_uvu_plain_gradients(maker, Z):
     junk = torch.full((Z, tp.weight_numel), float("nan"), device=DEV)
     del junk
     out.backward(cot.to(DEV))
-    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
-    assert_close(out, ref_out.numpy(), atol=1e-4 * scale(ref_out))
-    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dx1")
-    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
-    assert_close(c.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dw")
+    # per-sample contractions: the benchmark's tolerance for contractions, |err| <= 1e-4 + 1e-5 |ref|
+    assert_close(out, ref_out.numpy())
+    assert_close(a.grad, r1.numpy(), what="d/dx1")
+    assert_close(b.grad, r2.numpy(), what="d/dx2")
+    assert_close(c.grad, rw.numpy(), what="d/dw")
 
 
 @pytest.mark.parametrize("maker,N,E,idx", [(lambda: ks.cfg3(True), 120, 3000, torch.int64), (lambda: ks.cfg3(False), 50, 900, torch.int32),
@@ -63,8 +63,10 @@ def test_fused_message_gradients(maker, N, E, idx):
     scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
     assert_close(out, ref_out.numpy(), atol=1e-4 * scale(ref_out))
     assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dnode_x")
-    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dedge_attr")
-    assert_close(c.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dweight")
+    # sums over the edges of a node are held to a tolerance scaled by their size (the order of summation differs
+    # from scatter_add_), per-edge contractions to the benchmark's 1e-4 + 1e-5 |ref|
+    assert_close(b.grad, r2.numpy(), what="d/dedge_attr")
+    assert_close(c.grad, rw.numpy(), what="d/dweight")
     # only some inputs require a gradient
     a2, c2 = node_x.to(DEV).requires_grad_(True), w.to(DEV)
     tp.forward_gather_scatter(a2, attr.to(DEV), c2, edges=edges).backward(cot.to(DEV))
@@ -76,7 +78,7 @@ def test_fused_message_gradients(maker, N, E, idx):
     a4, c4 = node_x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
     tp.forward_gather_scatter(a4, attr.to(DEV), c4, edges=edges).backward(cot.to(DEV))
     assert_close(a4.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dnode_x, one backward kernel")
-    assert_close(c4.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dweight, one backward kernel")
+    assert_close(c4.grad, rw.numpy(), what="d/dweight, one backward kernel")
     # negative source indices wrap in the gather; the gradient scatters onto the wrapped rows
     neg = torch.where(torch.arange(E) % 3 == 0, src - N, src)
     a3 = node_x.to(DEV).requires_grad_(True)
@@ -108,10 +110,9 @@ def test_uvw_input_gradients(maker, Z):
     a, b = (t.to(DEV).requires_grad_(True) for t in (x1, x2))
     out = tp(a, b, w.to(DEV))
     out.backward(cot.to(DEV))
-    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
-    assert_close(out, ref_out.numpy(), atol=1e-4 * scale(ref_out))
-    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dx1")
-    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
+    assert_close(out, ref_out.numpy())
+    assert_close(a.grad, r1.numpy(), what="d/dx1")
+    assert_close(b.grad, r2.numpy(), what="d/dx2")
 
 
 @pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.cfg1, 4099),
@@ -127,14 +128,16 @@ def test_uvw_weight_gradients(maker, Z):
     _, (r1, r2, rw) = _oracle_grads(lambda a, b, c: tp_forward_torch(spec, a, b, c), (x1, x2, w), cot)
     a, b, c = (t.to(DEV).requires_grad_(True) for t in (x1, x2, w))
     tp(a, b, c).backward(cot.to(DEV))
-    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
-    assert_close(c.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dw")
-    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dx1")
-    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
+    # shared weights: the gradient is a sum over the batch, held to a tolerance scaled by its size; everything else
+    # is a per-sample contraction (1e-4 + 1e-5 |ref|)
+    w_atol = 1e-4 * max(1.0, float(rw.abs().max())) if tp.shared_weights else 1e-4
+    assert_close(c.grad, rw.numpy(), atol=w_atol, what="d/dw")
+    assert_close(a.grad, r1.numpy(), what="d/dx1")
+    assert_close(b.grad, r2.numpy(), what="d/dx2")
     # the weights alone
     c2 = w.to(DEV).requires_grad_(True)
     tp(x1.to(DEV), x2.to(DEV), c2).backward(cot.to(DEV))
-    assert_close(c2.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dw alone")
+    assert_close(c2.grad, rw.numpy(), atol=w_atol, what="d/dw alone")
 
 
 def test_internal_weights_train():
@@ -154,10 +157,9 @@ def test_shared_uvu_weight_gradient():
     _, (r1, r2, rw) = _oracle_grads(lambda a, b, c: tp_forward_torch(spec, a, b, c), (x1, x2, w), cot)
     a, b, c = (t.to(DEV).requires_grad_(True) for t in (x1, x2, w))
     tp(a, b, c).backward(cot.to(DEV))
-    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
-    assert_close(c.grad, rw.numpy(), atol=1e-4 * scale(rw), what="d/dw (shared)")
-    assert_close(a.grad, r1.numpy(), atol=1e-4 * scale(r1), what="d/dx1")
-    assert_close(b.grad, r2.numpy(), atol=1e-4 * scale(r2), what="d/dx2")
+    assert_close(c.grad, rw.numpy(), atol=1e-4 * max(1.0, float(rw.abs().max())), what="d/dw (shared, summed over the batch)")
+    assert_close(a.grad, r1.numpy(), what="d/dx1")
+    assert_close(b.grad, r2.numpy(), what="d/dx2")
 
 
 @pytest.mark.parametrize("maker", [ks.mixed_modes, lambda: ks.golden_tp("modes_uuu_uvuv_uuw_uvv"), lambda: ks.golden_tp("modes_triangular")])

@@ -215,6 +215,79 @@ def test_uvw_full_size_dense_configuration():
     assert torch.equal(tp(x1[1000:1100], x2[1000:1100]), out[1000:1100])
 
 
+@pytest.mark.parametrize("maker", [ks.mfma_full_tiles, ks.cfg5, ks.node_block])
+def test_split_operand_kernels_over_the_exponent_range_and_on_non_finite_rows(maker):
+    # the fp32 plans of these sets form each product from three bf16 pieces per operand.  (i) The pieces keep the
+    # exponent range of fp32: rows scaled by 1e-30 ... 1e30 come out with fp32 accuracy relative to their own scale.
+    # (ii) A row holding inf or NaN comes out non-finite and leaves every other row untouched, bit for bit.  Where the
+    # reference's einsum gives +-inf for such a row (all products of one sign) these kernels give NaN: the piece
+    # h = bf16(inf) is inf and the next piece is inf - inf; finite |x| above 3.39e38, which round to inf in bf16, behave
+    # the same way.  A sum of products of an inf with factors of both signs is NaN in the reference as well.
+    tp = maker().to(DEV)
+    w = _fan_in_weights(tp)
+    with torch.no_grad():
+        tp.weight.copy_(w)
+    Z = 70
+    x1, x2 = seeded(Z, tp.irreps_in1.dim, seed=31), seeded(Z, tp.irreps_in2.dim, seed=32)
+    scales = torch.tensor([1e-30, 1e-15, 1.0, 1e15, 1e30]).repeat(Z // 5)[:, None]
+    out = tp((x1 * scales).to(DEV), x2.to(DEV))
+    ref = otp.tp_forward(oracle_spec(tp), x1.numpy(), x2.numpy(), w.numpy())
+    rel = out.cpu().double() / scales.double()
+    assert_close(rel, ref, what=f"{maker.__name__}: rows scaled by 1e-30 ... 1e30, relative to their scale")
+    clean = tp(x1.to(DEV), x2.to(DEV))
+    bad = x1.clone()
+    bad[3, 0], bad[40, 5] = float("inf"), float("nan")
+    got = tp(bad.to(DEV), x2.to(DEV))
+    keep = torch.ones(Z, dtype=torch.bool)
+    keep[[3, 40]] = False
+    assert torch.equal(got[keep], clean[keep])
+    assert not torch.isfinite(got[3]).all() and not torch.isfinite(got[40]).all()
+
+
+def _uvw_weight_gradient_fp64(tp, x1, x2, cot):
+    """d/dW of sum(cot * tp(x1, x2, W)) for shared uvw weights, written out from the definition
+    out[z, w, k] = pw sum_uv W[u, v, w] sum_ij C[i, j, k] x1[z, u, i] x2[z, v, j]:
+    gW[u, v, w] = pw sum_ij (x1_i (x) x2_j)^T [z, (u, v)] @ (sum_k C[i, j, k] cot[z, w, k]), one GEMM per (i, j)."""
+    from oracle.wigner import wigner_3j
+
+    s1, s2, so = tp.irreps_in1.slices(), tp.irreps_in2.slices(), tp.irreps_out.slices()
+    Z, blocks = x1.shape[0], []
+    for t in tp.instructions:
+        (U, ir1), (V, ir2), (W, iro) = tp.irreps_in1[t.i_in1], tp.irreps_in2[t.i_in2], tp.irreps_out[t.i_out]
+        a, b, g = x1[:, s1[t.i_in1]].reshape(Z, U, -1), x2[:, s2[t.i_in2]].reshape(Z, V, -1), cot[:, so[t.i_out]].reshape(Z, W, -1)
+        C = wigner_3j(ir1.l, ir2.l, iro.l)
+        gw = np.zeros((U * V, W))
+        for i in range(ir1.dim):
+            for j in range(ir2.dim):
+                if np.any(C[i, j]):
+                    gw += (a[:, :, None, i] * b[:, None, :, j]).reshape(Z, U * V).T @ (g @ C[i, j])
+        blocks.append(t.path_weight * gw.reshape(-1))
+    return np.concatenate(blocks)
+
+
+def test_uvw_weight_gradient_on_the_dense_configuration():
+    # the weight gradient of config 5's own instruction set (11 paths of 128 x 128 x 128, 23 M weights) on the
+    # split-operand matrix-core kernel; 300 rows end inside a batch chunk of the kernel.  The float64 reference is the
+    # definition written out (one GEMM per pair of input components), itself checked here against autograd of the
+    # einsum restatement on a small set
+    from oracle.torch_cpu import tp_forward_torch
+
+    small = ks.mfma_small()
+    x1, x2, cot = (seeded(9, d, seed=s).double() for d, s in ((small.irreps_in1.dim, 1), (small.irreps_in2.dim, 2), (small.irreps_out.dim, 3)))
+    wd = seeded(small.weight_numel, seed=4).double().requires_grad_()
+    (auto,) = torch.autograd.grad(tp_forward_torch(oracle_spec(small), x1, x2, wd), wd, cot)
+    assert np.abs(_uvw_weight_gradient_fp64(small, x1.numpy(), x2.numpy(), cot.numpy()) - auto.numpy()).max() < 1e-12
+
+    tp = ks.cfg5().to(DEV)
+    Z = 300
+    x1, x2, cot = seeded(Z, 1152, seed=41), seeded(Z, 1152, seed=42), seeded(Z, 1152, seed=43)
+    wg = _fan_in_weights(tp).to(DEV).requires_grad_()
+    (got,) = torch.autograd.grad(tp(x1.to(DEV), x2.to(DEV), wg), wg, cot.to(DEV))
+    ref = _uvw_weight_gradient_fp64(tp, x1.double().numpy(), x2.double().numpy(), cot.double().numpy())
+    # a sum over the batch: tolerance scaled by its size
+    assert_close(got, ref, atol=1e-4 * max(1.0, float(np.abs(ref).max())), what="cfg5 weight gradient, 300 rows")
+
+
 def _bf16_uvw(seed_w=0):
     tp = ks.cfg5().to(DEV)
     w = _fan_in_weights(tp, seed=seed_w)
@@ -272,8 +345,10 @@ def test_uvw_bf16_storage_full_size():
 
 
 def test_provider_binding_runs_the_same_kernels():
-    # e3x plans built by the provider from (Irreps, Instruction) data give the product's own results, with e3nn's
-    # broadcasting of leading dimensions
+    # modules built by the provider from (Irreps, Instruction) data give the product's own results, with e3nn's
+    # broadcasting of leading dimensions -- also after the pickle round trip e3nn puts its generated modules through
+    import pickle
+
     from e3nn_amd import provider
 
     for tp, shared in ((ks.cfg1().to(DEV), True), (ks.cfg3(True), False)):
@@ -281,6 +356,56 @@ def test_provider_binding_runs_the_same_kernels():
         x1 = seeded(5, 1, tp.irreps_in1.dim, seed=1).to(DEV)
         x2 = seeded(1, 3, tp.irreps_in2.dim, seed=2).to(DEV)
         w = tp.weight.detach() if shared else seeded(5, 3, tp.weight_numel, seed=3).to(DEV)
-        got = gm(x1, x2, w)
         ref = tp(x1, x2) if shared else tp(x1, x2, w)
-        assert got.shape == (5, 3, tp.irreps_out.dim) and torch.equal(got, ref)
+        for mod in (gm, pickle.loads(pickle.dumps(gm))):
+            got = mod(x1, x2, w)
+            assert got.shape == (5, 3, tp.irreps_out.dim) and torch.equal(got, ref)
+        with pytest.raises(RuntimeError, match="share one dtype"):
+            gm(x1, x2.double(), w)
+        with pytest.raises(RuntimeError, match="float32 or bfloat16"):
+            gm(x1.double(), x2.double(), w.double())
+
+
+def test_provider_binding_is_differentiable():
+    # a reference TensorProduct served by the provider must train: gradients of all three arguments through
+    # gm(x1, x2, w) are the package TensorProduct's own (config 1: shared uvw weights; config 3: per-sample uvu
+    # weights), and both agree with float64 autograd of the einsum restatement
+    from e3nn_amd import provider
+    from oracle.torch_cpu import tp_forward_torch
+
+    for tp, shared in ((ks.cfg1().to(DEV), True), (ks.cfg3(True), False)):
+        gm = provider.hip_provider(tp.irreps_in1, tp.irreps_in2, tp.irreps_out, tp.instructions, shared, True, True)
+        x1 = seeded(40, tp.irreps_in1.dim, seed=1)
+        x2 = seeded(40, tp.irreps_in2.dim, seed=2)
+        w = seeded(*((tp.weight_numel,) if shared else (40, tp.weight_numel)), seed=3)
+        cot = seeded(40, tp.irreps_out.dim, seed=4)
+        grads = []
+        for f in (gm, tp):
+            args = [t.to(DEV).requires_grad_() for t in (x1, x2, w)]
+            out = f(*args)
+            assert out.grad_fn is not None
+            grads.append(torch.autograd.grad(out, args, cot.to(DEV)))
+        for got, ref, name in zip(grads[0], grads[1], ("x1", "x2", "w")):
+            if shared and name == "w":  # batch slices meet in fp32 atomics: last-bit differences between two runs
+                assert (got - ref).abs().max().item() <= 1e-5 * ref.abs().max().item(), name
+            else:
+                assert torch.equal(got, ref), name
+        spec = oracle_spec(tp)
+        a, b, c = (t.double().requires_grad_() for t in (x1, x2, w))
+        oracle_grads = torch.autograd.grad(tp_forward_torch(spec, a, b, c), (a, b, c), cot.double())
+        for got, ref, name in zip(grads[0], oracle_grads, ("x1", "x2", "w")):
+            atol = 1e-4 * max(1.0, float(ref.abs().max())) if shared and name == "w" else 1e-4  # batch sum / contraction
+            assert_close(got, ref.numpy(), atol=atol, what=f"provider, d/d{name}")
+
+
+def test_provider_right_binding():
+    from e3nn_amd import provider
+
+    tp = ks.right_small().to(DEV)
+    gm = provider.hip_provider_right(tp.irreps_in1, tp.irreps_in2, tp.irreps_out, tp.instructions, True, True, True)
+    x1 = seeded(6, tp.irreps_in1.dim, seed=1).to(DEV)
+    x2 = seeded(6, tp.irreps_in2.dim, seed=2).to(DEV)
+    mats = gm(x2, tp.weight.detach())
+    assert mats.shape == (6, tp.irreps_in1.dim, tp.irreps_out.dim) and torch.equal(mats, tp.right(x2))
+    ref = otp.tp_forward(oracle_spec(tp), x1.cpu().numpy(), x2.cpu().numpy(), tp.weight.detach().cpu().numpy())
+    assert_close(torch.einsum("zi,zik->zk", x1, mats), ref, what="x @ right(y) through the provider")

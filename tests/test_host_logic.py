@@ -2,7 +2,9 @@
 functions (Wigner 3j, plan creation) and the Python mirror of the reference API."""
 import copy
 import ctypes
+import io
 import os
+import pickle
 import re
 
 import numpy as np
@@ -330,16 +332,84 @@ def test_weight_gradient_entry_point_rejects_other_connection_modes():
 
 
 def test_provider_binding_builds_plans_from_constructor_data():
-    # the code-generation provider a reference maintainer would register: descriptor filled from Irreps + Instruction
+    # the code-generation provider a reference maintainer would register: plans built from Irreps + Instruction data
     from e3nn_amd import provider
 
     for tp in (ks.cfg1(), ks.cfg3(True), ks.mixed_modes()):
         gm = provider.hip_provider(tp.irreps_in1, tp.irreps_in2, tp.irreps_out, tp.instructions, tp.shared_weights, True, True)
         assert isinstance(gm, torch.fx.GraphModule)
         assert (gm.hip.weight_numel, gm.hip.in1_dim, gm.hip.out_dim) == (tp.weight_numel, tp.irreps_in1.dim, tp.irreps_out.dim)
+        # the engine evaluates e3nn's already normalised path weights, not a second normalisation of them
+        engine = gm.hip.engine()
+        assert [t.path_weight for t in engine.instructions] == [t.path_weight for t in tp.instructions if 0 not in t.path_shape]
+        assert engine._plan(torch.float32).key == tp._plan(torch.float32).key  # same specialised kernel
+        assert list(gm.state_dict()) == []  # nothing of the engine leaks into the host module's state_dict
     empty = o3.TensorProduct("0x0e", "0e", "0e", [(0, 0, 0, "uvw", True)])
     assert provider.hip_provider(empty.irreps_in1, empty.irreps_in2, empty.irreps_out, empty.instructions, True, True, True) is None
-    hooks = ["einsum code generator"]
-    provider.register(hooks)
-    provider.register(hooks)
-    assert hooks == [provider.hip_provider, "einsum code generator"]
+    left, right = ["einsum code generator"], ["einsum code generator (right)"]
+    provider.register(left, right)
+    provider.register(left, right)
+    assert left == [provider.hip_provider, "einsum code generator"]
+    assert right == [provider.hip_provider_right, "einsum code generator (right)"]
+
+
+class _Host(torch.nn.Module):
+    """What the reference's ``CodeGenMixin`` does with a generated module (e3nn/util/codegen/_mixin.py:55-133): the
+    submodule leaves the pickled state as ``pickle.dumps(submodule)`` bytes and comes back through ``pickle.loads``."""
+
+    def __init__(self, gm):
+        super().__init__()
+        self.gm = gm
+
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        state["_modules"] = state["_modules"].copy()
+        state["__codegen__"] = pickle.dumps(state["_modules"].pop("gm"))
+        return state
+
+    def __setstate__(self, state):
+        state = state.copy()
+        blob = state.pop("__codegen__")
+        self.__dict__.update(state)
+        self.gm = pickle.loads(blob)
+
+
+def test_provider_module_pickles_and_deepcopies():
+    # reference tests/o3/tensor_product_test.py:429-439 (deepcopy) and the torch.save / pickle life-cycle of a module
+    # that owns a generated submodule; plan creation needs no GPU
+    from e3nn_amd import provider
+
+    for tp, right in ((ks.cfg1(), False), (ks.cfg3(True), False), (ks.mixed_modes(), False), (ks.cfg1(), True)):
+        make = provider.hip_provider_right if right else provider.hip_provider
+        gm = make(tp.irreps_in1, tp.irreps_in2, tp.irreps_out, tp.instructions, tp.shared_weights, True, True)
+        key = gm.hip.engine()._plan(torch.float32).key
+        buf = io.BytesIO()
+        torch.save(gm, buf)
+        buf.seek(0)
+        copies = [pickle.loads(pickle.dumps(gm)), copy.deepcopy(gm), torch.load(buf, weights_only=False),
+                  copy.deepcopy(_Host(gm)).gm, pickle.loads(pickle.dumps(_Host(gm))).gm]  # fmt: skip
+        for c in copies:
+            assert isinstance(c, torch.fx.GraphModule) and c is not gm and c.hip is not gm.hip
+            assert c.hip._engine == []  # no handle travelled; the plan is rebuilt on first use
+            assert (c.hip.irreps, c.hip.instructions, c.hip.shared_weights, c.hip.is_right) == (
+                gm.hip.irreps, gm.hip.instructions, gm.hip.shared_weights, right)  # fmt: skip
+            assert c.hip.engine()._plan(torch.float32).key == key
+            assert c.code == gm.code
+
+
+def test_provider_module_refuses_what_the_kernels_do_not_take():
+    from e3nn_amd import provider
+
+    tp = ks.cfg1()
+    gm = provider.hip_provider(tp.irreps_in1, tp.irreps_in2, tp.irreps_out, tp.instructions, True, True, True)
+    x1, x2, w = torch.zeros(2, tp.irreps_in1.dim), torch.zeros(2, tp.irreps_in2.dim), torch.zeros(tp.weight_numel)
+    with pytest.raises(RuntimeError, match="GPU tensors only"):
+        gm(x1, x2, w)
+    with pytest.raises(RuntimeError, match="GPU tensors only"):
+        gm(x1.requires_grad_(), x2, w)  # never a silent result without a grad_fn
+    meta = lambda t, dt: torch.empty(t.shape, dtype=dt, device="meta")  # noqa: E731  (is_cuda False: refused before any launch)
+    with pytest.raises(RuntimeError):
+        gm(meta(x1, torch.float64), meta(x2, torch.float64), meta(w, torch.float64))
+    # triangular modes have no right() in the reference either (_codegen.py:620-623): the provider defers
+    tri = o3.TensorProduct("4x1o", "4x1o", "6x0e", [(0, 0, 0, "uvu<v", True)])
+    assert provider.hip_provider_right(tri.irreps_in1, tri.irreps_in2, tri.irreps_out, tri.instructions, True, True, True) is None
