@@ -1,11 +1,11 @@
 """Benchmark of the equivariant message-passing hot path on one MI355X.
 
 Headline workload (the benchmark's third configuration, "NequIP-style interaction"): N = 50 000 nodes uniform in a
-cube, radius graph with a 5 A cutoff (cube side 86.8 A -> ~1.87 M directed edges, degree ~37), node
-features 32x0e+32x1o+32x2e fp32, edge attributes = SH(lmax 2) of the edge vectors, uvu tensor product
-(11 paths) with per-edge weights from a 2-layer radial MLP, scatter-summed onto the destination nodes.
-One step = one launch of the fused gather -> tensor product -> scatter kernel over the whole graph, all
-inputs resident in HBM.  The other configurations are reported in "other".
+cube, radius graph with a 5 A cutoff (cube side 86.8 A -> ~1.87 M directed edges, degree ~37; the edge list grouped by
+destination, as a neighbour search emits it), node features 32x0e+32x1o+32x2e fp32, edge attributes = SH(lmax 2) of
+the edge vectors, uvu tensor product (11 paths) with per-edge weights from a 2-layer radial MLP, scatter-summed onto
+the destination nodes.  One step = one launch of the fused gather -> spherical harmonics -> tensor product -> scatter
+kernel over the whole graph, all inputs resident in HBM.  The other configurations are reported in "other".
 
 Prints ONE JSON line.
 """
@@ -28,7 +28,6 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt), keyed by the code object the counters were read
 # on: a kernel that has changed since reports no traffic instead of a stale figure.
 NEQUIP_TRAFFIC_BYTES = {
-    "uvu_9a6230a2caf8306da5d9c9f6": (2 * 1611842 + 56250) * 1024,  # FETCH_SIZE 1611842 x 2 KiB + WRITE_SIZE 56250 KiB
 }
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
@@ -132,7 +131,14 @@ def bench_nequip(args, dev):
     from e3nn_amd import kernel_sets as ks
 
     N, side, cutoff = 50_000, 86.8, 5.0
-    pos, src, dst = radius_graph(N, side, cutoff)
+    pos, src_pairs, dst_pairs = radius_graph(N, side, cutoff)
+    # The edge list as a neighbour search per node emits it: grouped by the node that asks for its neighbours, the
+    # destination.  The reference's models build their graph with torch_cluster's radius_graph and take edge_index[1]
+    # as edge_dst (e3nn/nn/models/gate_points_2101.py:322-324, v2106/gate_points_networks.py:69-71), which is that
+    # order.  The order of the k-d tree's pair list (every pair once, then every pair reversed) is timed beside it
+    # ("pair_order").
+    order = np.argsort(dst_pairs, kind="stable")
+    src, dst = src_pairs[order], dst_pairs[order]
     E = src.shape[0]
     gen = torch.Generator().manual_seed(0)
     tp = ks.cfg3(merged=True)
@@ -148,55 +154,66 @@ def bench_nequip(args, dev):
     for _ in range(5):
         edges = DstSortedEdges(src_t, dst_t, N)
     torch.cuda.synchronize()
-    sort_ms = (time.perf_counter() - t0) * 1e3 / 5  # wall clock incl. allocation and the range-check read-backs
+    prep_ms = (time.perf_counter() - t0) * 1e3 / 5  # wall clock incl. allocation and the range-check read-backs
+    assert edges.walk_perm is None  # grouped by destination already: the kernels walk the list by position
 
     out = [None]
 
     def step():
-        out[0] = tp.forward_gather_scatter(node_x, attr, w, edges=edges)
+        # edge attributes = SH(lmax 2) of the edge vectors, formed inside the kernel from the 12-byte vectors
+        out[0] = tp.forward_gather_scatter_sh(node_x, vec, w, edges, True, "component")
 
     ms, ms_median, ms_min = event_times_ms(step, args.steps, args.warmup)
     # algorithmic bytes: per edge weights + SH + two int64 indices, node table read once, output written once
     bytes_algo = E * (4 * tp.weight_numel + 4 * 9 + 2 * 8) + N * 4 * (tp.irreps_in1.dim + tp.irreps_out.dim)
     gbs = bytes_algo / (ms * 1e-3) / 1e9
+    frac = lambda t: bytes_algo / (t * 1e-3) / 1e9 / HBM_PEAK_GBS  # noqa: E731
     res = {
         "edges": E, "nodes": N, "ms": ms, "ms_median": ms_median, "ms_min": ms_min, "edges_per_s": E / (ms * 1e-3),
-        "bytes_per_launch": bytes_algo, "achieved_gbs": gbs, "edge_sort_ms_per_graph": sort_ms,
-        "kernel_key": tp._plan(torch.float32).key,
-        "edges_per_s_incl_sort": E / ((ms + sort_ms) * 1e-3),
+        "bytes_per_launch": bytes_algo, "achieved_gbs": gbs, "edge_preprocessing_ms_per_graph": prep_ms,
+        "kernel_key": tp._plan(torch.float32).key + "+sh",
+        "edges_per_s_incl_preprocessing": E / ((ms + prep_ms) * 1e-3),
+        # the kernel reads the 12-byte vectors where the algorithmic count has the 36-byte attribute rows
+        "bytes_read_less_than_counted": E * 4 * (9 - 3),
     }  # fmt: skip
-    ctx = dict(tp=tp, node_x=node_x, attr=attr, w=w, src=src_t, dst=dst_t, N=N, out=out[0])
+    ctx = dict(tp=tp, node_x=node_x, attr=attr, w=w, src=src_t, dst=dst_t, N=N, out=out[0], vec=vec)
+    # the same call on stored edge attributes ([E, 9] read from memory)
+    t = event_time_ms(lambda: tp.forward_gather_scatter(node_x, attr, w, edges=edges), args.steps, args.warmup)
+    res["stored_edge_attr"] = {"ms": t, "edges_per_s": E / (t * 1e-3), "roofline_frac": frac(t)}
     # part of the default run; skipped when --only selects sections
     if getattr(args, "locality_variants", False) or getattr(args, "only", None) == "":
-        # same graph, friendlier numbering: (a) edge list sorted by destination, as neighbour-list codes emit it;
-        # (b) nodes renumbered along a Morton curve of their positions as well (a spatially sorted system)
-        def timed(order_nodes):
-            if order_nodes:
-                c = np.floor(pos / 2.5).astype(np.uint64)
+        # same graph: (a) the edge list in the k-d tree's pair order (the kernels then reach the per-edge tensors
+        # through the permutation of the destination sort, built once per graph); (b) nodes renumbered along a Morton
+        # curve of their positions (a spatially sorted system), edge list grouped by destination
+        def timed(s_np, d_np, nx, a2, w2, v2):
+            e2 = DstSortedEdges(torch.from_numpy(s_np).to(dev), torch.from_numpy(d_np).to(dev), N)
+            return e2, {
+                "harmonics_in_kernel": event_time_ms(lambda: tp.forward_gather_scatter_sh(nx, v2, w2, e2, True, "component"), args.steps, args.warmup),
+                "stored_edge_attr": event_time_ms(lambda: tp.forward_gather_scatter(nx, a2, w2, edges=e2), args.steps, args.warmup),
+            }  # fmt: skip
 
-                def spread(v):
-                    v = v & np.uint64(0x3FF)
-                    for sh, m in ((16, 0x30000FF), (8, 0x300F00F), (4, 0x30C30C3), (2, 0x9249249)):
-                        v = (v | (v << np.uint64(sh))) & np.uint64(m)
-                    return v
+        inv = torch.from_numpy(np.argsort(order)).to(dev)  # position of pair-list edge e in the grouped list
+        e_pairs, t_pairs = timed(src_pairs, dst_pairs, node_x, attr[inv].contiguous(), w[inv].contiguous(), vec[inv].contiguous())
+        assert e_pairs.walk_perm is not None
+        c = np.floor(pos / 2.5).astype(np.uint64)
 
-                key = spread(c[:, 0]) | (spread(c[:, 1]) << np.uint64(1)) | (spread(c[:, 2]) << np.uint64(2))
-                rank = np.empty(N, np.int64)
-                rank[np.argsort(key, kind="stable")] = np.arange(N)
-                s2, d2 = rank[src], rank[dst]
-                nx = torch.empty_like(node_x)
-                nx[torch.from_numpy(rank).to(dev)] = node_x
-            else:
-                s2, d2, nx = src, dst, node_x
-            o = np.argsort(d2, kind="stable")
-            ot = torch.from_numpy(o).to(dev)
-            e2 = DstSortedEdges(torch.from_numpy(s2[o]).to(dev), torch.from_numpy(d2[o]).to(dev), N)
-            a2, w2 = attr[ot].contiguous(), w[ot].contiguous()
-            return event_time_ms(lambda: tp.forward_gather_scatter(nx, a2, w2, edges=e2), args.steps, args.warmup)
+        def spread(v):
+            v = v & np.uint64(0x3FF)
+            for sh, m in ((16, 0x30000FF), (8, 0x300F00F), (4, 0x30C30C3), (2, 0x9249249)):
+                v = (v | (v << np.uint64(sh))) & np.uint64(m)
+            return v
 
-        for name, flag in (("sorted_edges", False), ("sorted_edges_morton_nodes", True)):
-            t = timed(flag)
-            res[name] = {"ms": t, "edges_per_s": E / (t * 1e-3), "roofline_frac": bytes_algo / (t * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        key = spread(c[:, 0]) | (spread(c[:, 1]) << np.uint64(1)) | (spread(c[:, 2]) << np.uint64(2))
+        rank = np.empty(N, np.int64)
+        rank[np.argsort(key, kind="stable")] = np.arange(N)
+        s2, d2 = rank[src], rank[dst]
+        nx = torch.empty_like(node_x)
+        nx[torch.from_numpy(rank).to(dev)] = node_x
+        o = np.argsort(d2, kind="stable")
+        ot = torch.from_numpy(o).to(dev)
+        _, t_morton = timed(s2[o], d2[o], nx, attr[ot].contiguous(), w[ot].contiguous(), vec[ot].contiguous())
+        for name, times in (("pair_order", t_pairs), ("morton_nodes", t_morton)):
+            res[name] = {k: {"ms": t, "edges_per_s": E / (t * 1e-3), "roofline_frac": frac(t)} for k, t in times.items()}
     return res, ctx
 
 
@@ -617,12 +634,13 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "NequIP-style uvu interaction: N=50000 nodes, cube side 86.8 A, 5 A cutoff radius graph "
-                        f"(E={neq['edges']}), 32x0e+32x1o+32x2e x SH(lmax 2), 11 paths, 352 weights/edge, int64 indices, "
-                        "fused scatter-sum; edge sort by destination built once per graph, outside the timed region (edge_sort_ms_per_graph)",
+                        f"(E={neq['edges']}, edge list grouped by destination as a neighbour search emits it), 32x0e+32x1o+32x2e x SH(lmax 2) "
+                        "of the edge vectors (formed in the kernel), 11 paths, 352 weights/edge from a radial MLP (an input), int64 indices, "
+                        "fused scatter-sum; row pointers built once per graph, outside the timed region (edge_preprocessing_ms_per_graph)",
         },
         "roofline": {
             "bound": "hbm", "achieved": neq["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": neq["achieved_gbs"] / HBM_PEAK_GBS, "traffic": NEQUIP_TRAFFIC_BYTES.get(neq["kernel_key"].split("+")[0]), "kernel": "e3x_uvu_fused",
+            "frac": neq["achieved_gbs"] / HBM_PEAK_GBS, "traffic": NEQUIP_TRAFFIC_BYTES.get(neq["kernel_key"]), "kernel": "e3x_uvu_sh_fused",
             "algorithmic_bytes": neq["bytes_per_launch"],
             # the same bytes streamed by a kernel that does nothing else (e3x_stream_rows), measured in this run
             "stream_same_bytes_gbs": other.get("stream_rows_headline_bytes", {}).get("read_and_row_stores", {}).get("gbs"),

@@ -62,6 +62,9 @@ _SIGNATURES = {
     "e3x_tp_gather_scatter_workspace_bytes": (c_size_t, [c_void_p, c_int64]),
     "e3x_tp_gather_scatter_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "e3x_tp_plan_prepare_gather_scatter_sh": (c_int, [c_void_p, c_int32, c_int32]),
+    "e3x_tp_gather_scatter_sh": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                         c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p]),
     "e3x_src_rows_build": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "e3x_tp_gather_scatter_radial": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
                                              ctypes.c_double, ctypes.c_double, ctypes.c_double, c_void_p, c_int, c_void_p,

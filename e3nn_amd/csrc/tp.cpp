@@ -7,6 +7,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <sstream>
@@ -69,6 +70,9 @@ struct e3x_plan {
   std::string radial_desc;
   std::mutex mu;
   std::vector<std::unique_ptr<SubKernel>> subs;
+  // uvu with the spherical harmonics 0 .. lmax as second input: variants of the kernels of `subs` that form the
+  // harmonics from the edge vectors themselves, per (normalize, normalization), built on first use
+  std::map<int, std::vector<std::unique_ptr<SubKernel>>> sh_subs;
   // uvu, bf16 storage: the message kernel (gather + product + scatter) with the contraction on the matrix cores,
   // when the instruction set fits it; the plain product keeps the kernels of `subs`
   std::unique_ptr<SubKernel> msg_mfma;
@@ -993,6 +997,59 @@ int load_uvu_fused_dw_function(e3x_plan* P, int dev) {
   return E3X_OK;
 }
 
+// ---- uvu message kernel with the spherical harmonics formed in the kernel -------------------------------------
+// lmax when irreps_in2 is 1x0e + 1x1o + ... + 1x(lmax)(parity (-1)^l) with 1 <= lmax <= 3, else -1
+int sh_lmax_of(const e3x_plan* P) {
+  const int n = (int)P->in2.size();
+  if (P->family != "uvu" || n < 2 || n > 4) return -1;
+  for (int l = 0; l < n; ++l)
+    if (P->in2[l].mul != 1 || P->in2[l].l != l || P->in2[l].p != (l % 2 ? -1 : 1)) return -1;
+  return n - 1;
+}
+
+int prepare_uvu_sh(e3x_plan* P, int normalize, int normalization) {
+  const int lmax = sh_lmax_of(P);
+  if (lmax < 0 || (P->shared_weights && P->weight_numel) || normalization < 0 || normalization > 2) return E3X_ERR_INVALID;
+  const int key = (normalize ? 4 : 0) + normalization;
+  std::lock_guard<std::mutex> lock(P->mu);
+  if (P->sh_subs.count(key)) return E3X_OK;
+  std::ostringstream x;
+  x << "#define E3X_UVU_SH 1\nconstexpr int SH_LMAX = " << lmax << ";\nconstexpr bool SH_NORMALIZE = " << (normalize ? "true" : "false")
+    << ";\nconstexpr float SH_SCALE[4] = {";
+  for (int l = 0; l < 4; ++l) {
+    const double sc = normalization == E3X_NORM_INTEGRAL ? 1.0 / std::sqrt(4.0 * M_PI) : normalization == E3X_NORM_NORM ? 1.0 / std::sqrt(2.0 * l + 1.0) : 1.0;
+    x << fstr(sc) << ", ";
+  }
+  x << "};\n";
+  const std::string extra = x.str();
+  std::vector<std::unique_ptr<SubKernel>> built;
+  for (auto& K : P->subs) {
+    std::unique_ptr<SubKernel> S(new SubKernel);
+    S->path_ids = K->path_ids;
+    std::string src;
+    int rc;
+    if ((rc = build_uvu_source(*P, *S, &src, false, &extra))) return rc;
+    if ((rc = e3x::get_code_object("uvu_sh", src, &S->key, &S->hsaco))) return rc;
+    built.push_back(std::move(S));
+  }
+  P->sh_subs[key] = std::move(built);
+  return E3X_OK;
+}
+
+int load_uvu_sh_functions(e3x_plan* P, int key, int dev) {
+  std::lock_guard<std::mutex> lock(P->mu);
+  for (auto& S : P->sh_subs[key]) {
+    if (S->module[dev]) continue;
+    hipModule_t mod = nullptr;
+    hipError_t err = hipModuleLoad(&mod, S->hsaco.c_str());
+    if (err != hipSuccess) return fail(E3X_ERR_HIP, "hipModuleLoad(" + S->hsaco + ") failed: " + hipGetErrorString(err));
+    if (hipModuleGetFunction(&S->fn_fused[dev], mod, "e3x_uvu_sh_fused") != hipSuccess)
+      return fail(E3X_ERR_HIP, "kernel e3x_uvu_sh_fused missing from " + S->hsaco);
+    S->module[dev] = mod;
+  }
+  return E3X_OK;
+}
+
 int current_device(int* dev) {
   if (hipGetDevice(dev) != hipSuccess || *dev < 0 || *dev >= kMaxDevices) return fail(E3X_ERR_HIP, "hipGetDevice failed");
   return E3X_OK;
@@ -1221,6 +1278,24 @@ extern "C" int e3x_tp_forward_ws(e3x_plan* P, const void* x1, const void* x2, co
   return E3X_OK;
 }
 
+constexpr int kSrcInRowOrderHost = 2;  // index mode of the kernels: the source ids as an int32 list in sorted position order
+
+// one launch of e3x_uvu_fused per kernel of the set (several when the instruction set is split over output irreps)
+static int launch_fused_kernels(const std::vector<std::unique_ptr<SubKernel>>& kernels, int dev, long long n_rows, void** args,
+                                hipStream_t st) {
+  for (auto& K : kernels) {
+    const long long items = n_rows * K->chunks;
+    long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
+    blocks = (blocks + 7) / 8 * 8;  // the kernel deals contiguous eighths of the rows to the 8 XCDs
+    if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
+    hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1,
+                                           0, st, args, nullptr);
+    if (err != hipSuccess)
+      return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
+  }
+  return E3X_OK;
+}
+
 extern "C" int e3x_tp_gather_scatter(e3x_plan* P, const void* node_x, const void* edge_attr, const void* w,
                                      const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
                                      void* out, int64_t E, int64_t num_src_nodes, int64_t num_out_nodes,
@@ -1268,7 +1343,7 @@ extern "C" int e3x_tp_gather_scatter_ws(e3x_plan* P, const void* node_x, const v
   int idx64 = idx_bits == 64;
   if (src_rows) {
     src = src_rows;
-    idx64 = 2;
+    idx64 = kSrcInRowOrderHost;
   }
   long long n_rows = num_out_nodes, n_src = num_src_nodes;
   void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&w,         (void*)&out,    (void*)&src,  (void*)&idx64,
@@ -1297,17 +1372,47 @@ extern "C" int e3x_tp_gather_scatter_ws(e3x_plan* P, const void* node_x, const v
       return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
     return E3X_OK;
   }
-  for (auto& K : P->subs) {
-    const long long items = n_rows * K->chunks;
-    long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
-    blocks = (blocks + 7) / 8 * 8;  // the kernel deals contiguous eighths of the rows to the 8 XCDs
-    if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter: too many rows for one launch");
-    hipError_t err = hipModuleLaunchKernel(K->fn_fused[dev], (unsigned)blocks, 1, 1, 64 * K->waves_per_block, 1, 1,
-                                           0, st, args, nullptr);
-    if (err != hipSuccess)
-      return fail(E3X_ERR_HIP, std::string("e3x_tp_gather_scatter: launch failed: ") + hipGetErrorString(err));
+  return launch_fused_kernels(P->subs, dev, n_rows, args, st);
+}
+
+extern "C" int e3x_tp_plan_prepare_gather_scatter_sh(e3x_plan* P, int32_t normalize, int32_t normalization) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_plan_prepare_gather_scatter_sh: null plan");
+  return prepare_uvu_sh(P, normalize, normalization);  // E3X_ERR_INVALID without a message: callers ask to find out
+}
+
+extern "C" int e3x_tp_gather_scatter_sh(e3x_plan* P, const void* node_x, const float* edge_vec, const void* w,
+                                        const void* src, int idx_bits, const int32_t* rowptr, const int32_t* perm,
+                                        const int32_t* row_order, const int32_t* src_rows, void* out, int64_t E,
+                                        int64_t num_src_nodes, int64_t num_out_nodes, int32_t normalize,
+                                        int32_t normalization, void* stream) {
+  if (!P) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_sh: null plan");
+  int rc = prepare_uvu_sh(P, normalize, normalization);
+  if (rc == E3X_ERR_INVALID)
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_sh: needs an all-uvu plan with per-edge weights whose second input is 0e + 1o + ... up to l <= 3");
+  if (rc) return rc;
+  if (idx_bits != 32 && idx_bits != 64) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_sh: idx_bits must be 32 or 64");
+  if (E < 0 || num_src_nodes < 0 || num_out_nodes < 0) return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_sh: negative size");
+  if (num_out_nodes == 0 || P->out_dim == 0) return E3X_OK;
+  if (!out || !rowptr || (E > 0 && (!src || (P->in1_dim && !node_x) || !edge_vec || (P->weight_numel && !w))))
+    return fail(E3X_ERR_INVALID, "e3x_tp_gather_scatter_sh: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  int dev;
+  if ((rc = current_device(&dev))) return rc;
+  if (P->zero_fill || P->paths.empty()) {
+    if ((rc = zero_output(P, out, num_out_nodes, st))) return rc;
+    if (P->paths.empty()) return E3X_OK;
   }
-  return E3X_OK;
+  const int key = (normalize ? 4 : 0) + normalization;
+  if ((rc = load_uvu_sh_functions(P, key, dev))) return rc;
+  int idx64 = idx_bits == 64;
+  if (src_rows) {
+    src = src_rows;
+    idx64 = kSrcInRowOrderHost;
+  }
+  long long n_rows = num_out_nodes, n_src = num_src_nodes;
+  void* args[] = {(void*)&node_x, (void*)&edge_vec, (void*)&w,         (void*)&out,    (void*)&src,  (void*)&idx64,
+                  (void*)&rowptr, (void*)&perm,     (void*)&row_order, (void*)&n_rows, (void*)&n_src};
+  return launch_fused_kernels(P->sh_subs[key], dev, n_rows, args, st);
 }
 
 extern "C" int e3x_tp_plan_prepare_gather_scatter_grad_w(e3x_plan* P) {

@@ -303,12 +303,19 @@ def conv_wide():
     return nn.Convolution(f, "4x0e", SH2, f, [8, 64], 37.5)
 
 
+# (set, normalize, normalization) of the message kernels that form the spherical harmonics of the edge vectors themselves
+SH_MESSAGE_CASES = [("cfg3_merged", True, "component"), ("cfg3_merged", False, "integral"), ("cfg3_builder", True, "norm"),
+                    ("cfg4_A", True, "component"), ("odd_mul", True, "integral")]  # fmt: skip
+
+
 def prebuild(verbose=True, workers=6):
     """Builds every kernel the tests and the benchmark use.  Plan creation spends its time in the HIP compiler (a child
     process, the calling thread waits with the GIL released), so a few threads build several kernels at once."""
     from concurrent.futures import ThreadPoolExecutor
 
     from e3nn_amd import nn
+
+    from . import _lib
 
     jobs = []
     for name, mod in nn_modules() + [(f"fused_fc{i}", net) for i, net in enumerate(fused_fc_nets())]:
@@ -321,6 +328,9 @@ def prebuild(verbose=True, workers=6):
                 jobs.append((f"module {name} (one kernel)", sub, None, False))
     for name, tp, dtypes in all_tensor_products():
         jobs.append((f"kernel {name}", tp, dtypes, name in BACKWARD_CASES))
+    by_name = {name: tp for name, tp, _ in all_tensor_products()}
+    for name, normalize, normalization in SH_MESSAGE_CASES:
+        jobs.append((f"harmonics {name}", by_name[name], (normalize, normalization), False))
     for name, tp, net in radial_message_cases():
         jobs.append((f"radial {name}", tp, net, False))
     for name, mod in nn_modules():
@@ -329,6 +339,12 @@ def prebuild(verbose=True, workers=6):
 
     def build(job):
         name, tp, dtypes, backward = job
+        if name.startswith("harmonics "):
+            from .o3.spherical_harmonics import _NORMALIZATION
+
+            rc = _lib.lib().e3x_tp_plan_prepare_gather_scatter_sh(tp._plan(torch.float32).handle, int(dtypes[0]), _NORMALIZATION[dtypes[1]])
+            _lib.check(rc)
+            return name, [f"normalize={dtypes[0]} {dtypes[1]}"]
         if name.startswith("radial "):
             plan = dtypes.fused_plan()  # the network on its own, which the tests run beside the fused kernel
             return name, ["built" if tp.prepare_gather_scatter_radial(dtypes) else "(separate kernels)", plan.key or ""]
@@ -356,8 +372,6 @@ def prebuild(verbose=True, workers=6):
                 print(f"{name:40s} {' '.join(keys)}", flush=True)
     # the benchmark times config 5 on the fp32 matrix instruction beside the split-operand default; the generator reads
     # its switches from the environment at plan creation, so these two are built here, after the threads are done
-    from . import _lib
-
     saved = {k: os.environ.get(k) for k in ("E3X_UVW_SPLIT", "E3X_DW_SPLIT")}
     os.environ.update({k: "0" for k in saved})
     try:

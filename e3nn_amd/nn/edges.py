@@ -58,9 +58,38 @@ class DstSortedEdges:
             self._src_rows = rows
         return self._src_rows
 
+    def in_sorted_order(self, *edge_tensors):
+        """Per-edge tensors ``[E, ...]`` rewritten in the order of the destination-sorted list (row ``k`` of a result is
+        row ``perm[k]`` of the argument; differentiable).  Together with :meth:`sorted` this moves the permutation out
+        of the message kernels: done once per graph for the edge attributes and the inputs of the radial network, every
+        layer then produces and consumes its per-edge weights in the order the kernels walk them, a row's weights
+        being one contiguous run instead of scattered rows."""
+        if self.walk_perm is None:
+            return edge_tensors if len(edge_tensors) != 1 else edge_tensors[0]
+        out = tuple(t.index_select(0, self.perm) for t in edge_tensors)
+        return out if len(out) != 1 else out[0]
+
+    def sorted(self) -> "DstSortedEdges":
+        """The same graph with its edge list held in destination order: edge ``k`` is edge ``perm[k]`` of this list, so
+        the kernels read per-edge tensors by position.  Shares the row pointers, the row order and the source rows;
+        nothing is sorted again.  Per-edge tensors go with it through :meth:`in_sorted_order`."""
+        if self.walk_perm is None:
+            return self
+        if self._sorted is None:
+            other = object.__new__(DstSortedEdges)
+            other.__dict__.update(self.__dict__)
+            src = self.src_rows if self.src_rows is not None else torch.where(self.edge_src < 0, self.edge_src + self.num_src_nodes, self.edge_src).index_select(0, self.perm).int()
+            other.edge_src, other.edge_dst = src, self.edge_dst.index_select(0, self.perm)
+            other._src_rows, other.walk_perm = src, None
+            other.perm = torch.arange(self.num_edges, dtype=torch.int32, device=src.device)
+            other._transposed, other._sorted = None, other
+            self._sorted = other
+        return self._sorted
+
     def __init__(self, edge_src: torch.Tensor, edge_dst: torch.Tensor, num_nodes: int, num_src_nodes: int = None,
                  locality_order="auto"):
         self._transposed = None
+        self._sorted = None
         self._src_rows = None
         self._locality_order = locality_order
         if not (edge_src.is_cuda and edge_dst.is_cuda):
@@ -89,6 +118,13 @@ class DstSortedEdges:
                     _lib.ptr(self.perm), _lib.ptr(ws), ws_bytes, st,
                 )  # fmt: skip
             )
+            # A list that is already grouped by destination (what neighbour searches emit: torch_cluster's
+            # radius_graph, which the reference's models call, returns its pairs sorted by the query node) is walked
+            # by position: the stable sort is then the identity and the kernels are handed no permutation, so that
+            # per-edge rows are read as one contiguous run per destination.
+            self.walk_perm = self.perm
+            if E > 1 and bool((self.edge_dst[1:] >= self.edge_dst[:-1]).all()):
+                self.walk_perm = None
             # rows that share their smallest source are processed next to each other (they share most of their
             # sources, which then sit in L2): locality taken from the graph, not from the caller's node numbering
             self.row_order = None

@@ -125,9 +125,30 @@ class _Plan:
             _lib.check(
                 L.e3x_tp_gather_scatter_ws(
                     self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(gather_idx),
-                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(edges.row_order),
+                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.walk_perm), _lib.ptr(edges.row_order),
                     _lib.ptr(edges.src_rows if gather_idx is edges.edge_src else None),
                     _lib.ptr(out), edges.num_edges, num_table_rows, edges.num_nodes, _lib.ptr(ws), ws_bytes,
+                    _lib.stream_ptr(table.device),
+                )  # fmt: skip
+            )
+        return out
+
+    def gather_scatter_sh(self, table, edge_vec, w, gather_idx, edges, num_table_rows, normalize, normalization):
+        """``gather_scatter`` with ``edge_attr`` = the spherical harmonics of ``edge_vec[E, 3]``, formed in the kernel;
+        None when the plan's second input is not ``0e + 1o + ...`` up to ``l <= 3``."""
+        L = _lib.lib()
+        rc = L.e3x_tp_plan_prepare_gather_scatter_sh(self.handle, int(bool(normalize)), normalization)
+        if rc == _lib.ERR_INVALID:
+            return None
+        _lib.check(rc)
+        out = torch.empty(edges.num_nodes, self.out_dim, dtype=table.dtype, device=table.device)
+        with torch.cuda.device(table.device):
+            _lib.check(
+                L.e3x_tp_gather_scatter_sh(
+                    self.handle, _lib.ptr(table), _lib.ptr(edge_vec), _lib.ptr(w), _lib.ptr(gather_idx),
+                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.walk_perm), _lib.ptr(edges.row_order),
+                    _lib.ptr(edges.src_rows if gather_idx is edges.edge_src else None),
+                    _lib.ptr(out), edges.num_edges, num_table_rows, edges.num_nodes, int(bool(normalize)), normalization,
                     _lib.stream_ptr(table.device),
                 )  # fmt: skip
             )
@@ -152,7 +173,7 @@ class _Plan:
             _lib.check(
                 L.e3x_tp_gather_scatter_grad_w(
                     self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(w), _lib.ptr(row_x), _lib.ptr(gather_idx),
-                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(edges.row_order),
+                    gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.walk_perm), _lib.ptr(edges.row_order),
                     _lib.ptr(edges.src_rows if gather_idx is edges.edge_src else None),
                     _lib.ptr(out), _lib.ptr(grad_w), _lib.ptr(grad_x2), edges.num_edges, table.shape[0], edges.num_nodes,
                     _lib.stream_ptr(table.device),
@@ -169,7 +190,7 @@ class _Plan:
             rc = _lib.lib().e3x_tp_gather_scatter_radial(
                 self.handle, _lib.ptr(table), _lib.ptr(edge_attr), _lib.ptr(edge_scalars), _lib.ptr(w1), _lib.ptr(w2),
                 w1.shape[0], w1.shape[1], act_kind, act_cst, float(variance_in), float(variance_out), _lib.ptr(gather_idx),
-                gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.perm), _lib.ptr(out), edges.num_edges,
+                gather_idx.element_size() * 8, _lib.ptr(edges.rowptr), _lib.ptr(edges.walk_perm), _lib.ptr(out), edges.num_edges,
                 num_table_rows, edges.num_nodes, _lib.stream_ptr(table.device),
             )  # fmt: skip
         if rc == _lib.ERR_INVALID:
@@ -300,26 +321,62 @@ class _GatherScatterFn(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, g):
-        tp, edges = ctx.tp, ctx.edges
         node_x, edge_attr, w = ctx.saved_tensors
-        g = g.contiguous()
-        need1, need2, needw = ctx.needs_input_grad[:3]
-        g1 = g2 = gw = None
-        if need1 and needw and tp.weight_numel and node_x.dtype == torch.float32:
-            # every gradient from one pass over the weights and one gather of g per edge
-            res = tp._grad_plan("x1", node_x.dtype).gather_scatter_grad_w(
-                g, edge_attr, w, node_x, edges.edge_dst, edges.transposed(), need2 and edge_attr.shape[1] > 0
-            )
-            if res is not None:
-                return res[0], (res[2] if need2 else None), res[1], None, None
-        if need1:
-            rev = edges.transposed()
-            g1 = tp._grad_plan("x1", node_x.dtype).gather_scatter(g, edge_attr, w, edges.edge_dst, rev, g.shape[0])
-        if need2 or (needw and tp.weight_numel):
-            gw, g2 = tp._plan(node_x.dtype).backward_w_x2(
-                node_x, edge_attr, w, g, edges.edge_src, edges.edge_dst, needw and tp.weight_numel > 0, need2, edges.num_edges
-            )
-        return g1, g2, gw, None, None
+        return _message_gradients(ctx.tp, ctx.edges, node_x, edge_attr, w, g.contiguous(), *ctx.needs_input_grad[:3]) + (None, None)
+
+
+def _message_gradients(tp, edges, node_x, edge_attr, w, g, need1, need2, needw):
+    """``(d/dnode_x, d/dedge_attr, d/dw)`` of ``<g, scatter(tp(node_x[src], edge_attr, w), dst)>``; None where not needed."""
+    g1 = g2 = gw = None
+    if need1 and needw and tp.weight_numel and node_x.dtype == torch.float32:
+        # every gradient from one pass over the weights and one gather of g per edge
+        res = tp._grad_plan("x1", node_x.dtype).gather_scatter_grad_w(
+            g, edge_attr, w, node_x, edges.edge_dst, edges.transposed(), need2 and edge_attr.shape[1] > 0
+        )
+        if res is not None:
+            return res[0], (res[2] if need2 else None), res[1]
+    if need1:
+        rev = edges.transposed()
+        g1 = tp._grad_plan("x1", node_x.dtype).gather_scatter(g, edge_attr, w, edges.edge_dst, rev, g.shape[0])
+    if need2 or (needw and tp.weight_numel):
+        gw, g2 = tp._plan(node_x.dtype).backward_w_x2(
+            node_x, edge_attr, w, g, edges.edge_src, edges.edge_dst, needw and tp.weight_numel > 0, need2, edges.num_edges
+        )
+    return g1, g2, gw
+
+
+class _GatherScatterShFn(torch.autograd.Function):
+    """``_GatherScatterFn`` on ``edge_attr = spherical_harmonics(0 .. lmax, edge_vec)``, the harmonics formed inside the
+    kernel.  The backward pass evaluates them once with the stand-alone kernel (they are 3 % of the per-edge bytes)
+    and runs the message gradients on them; the gradient of the vectors goes through the harmonics' own backward."""
+
+    @staticmethod
+    def forward(ctx, node_x, edge_vec, w, tp, edges, normalize, normalization):
+        from .spherical_harmonics import _NORMALIZATION
+
+        out = tp._plan(node_x.dtype).gather_scatter_sh(
+            node_x, edge_vec, w, edges.edge_src, edges, node_x.shape[0], normalize, _NORMALIZATION[normalization]
+        )
+        if out is None:
+            raise NotImplementedError("forward_gather_scatter_sh needs irreps_in2 = 0e + 1o + ... up to l <= 3 (multiplicity 1)")
+        ctx.tp, ctx.edges, ctx.sh = tp, edges, (normalize, normalization)
+        ctx.save_for_backward(node_x, edge_vec, w)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        from .spherical_harmonics import _SphericalHarmonicsFn
+
+        node_x, edge_vec, w = ctx.saved_tensors
+        need1, need_vec, needw = ctx.needs_input_grad[:3]
+        ls = tuple(range(len(ctx.tp.irreps_in2)))
+        with torch.enable_grad():
+            vec = edge_vec.detach().requires_grad_(need_vec)
+            attr = _SphericalHarmonicsFn.apply(vec, ls, *ctx.sh)
+        g1, g2, gw = _message_gradients(ctx.tp, ctx.edges, node_x, attr.detach().to(node_x.dtype), w, g.contiguous(), need1, need_vec, needw)
+        gvec = torch.autograd.grad(attr, vec, g2.to(attr.dtype))[0] if need_vec else None
+        return g1, gvec, gw, None, None, None, None
 
 
 class _Constants(torch.nn.Module):
@@ -787,6 +844,29 @@ class TensorProduct(torch.nn.Module):
             w = node_x.new_empty(0)
         return _GatherScatterFn.apply(node_x.contiguous(), edge_attr.to(node_x.dtype).contiguous(), w, self, edges)
 
+
+    def forward_gather_scatter_sh(self, node_x, edge_vec, weight, edges, normalize: bool = True, normalization: str = "component"):
+        """``forward_gather_scatter(node_x, spherical_harmonics(range(lmax + 1), edge_vec, normalize, normalization),
+        weight, edges=edges)`` with the harmonics formed inside the kernel: ``edge_vec[E, 3]`` (float32) is read in
+        place of the stored ``[E, (lmax + 1)^2]`` attributes.  Needs ``irreps_in2 = 0e + 1o + ...`` up to ``lmax <= 3``
+        with multiplicity 1 (what the reference's convolutions feed the product, e3nn/nn/models/gate_points_2101.py:329)."""
+        if any(t.connection_mode != "uvu" for t in self.instructions):
+            raise NotImplementedError("forward_gather_scatter_sh needs an all-uvu TensorProduct")
+        assert normalization in ["integral", "component", "norm"]
+        torch._assert(node_x.ndim == 2 and node_x.shape[-1] == self._in1_dim, "Incorrect shape for node_x")
+        torch._assert(edge_vec.shape == (edges.num_edges, 3), "edge_vec must be [num_edges, 3]")
+        self._check_device(node_x, edge_vec)
+        if edge_vec.dtype != torch.float32:
+            raise TypeError(f"edge vectors are read as float32, got {edge_vec.dtype}")
+        torch._assert(edges.num_src_nodes == node_x.shape[0], "edge list was built for another node count")
+        if self.weight_numel:
+            torch._assert(not self.shared_weights, "forward_gather_scatter_sh needs per-edge weights (shared_weights=False)")
+            w = self._get_weights(weight)
+            torch._assert(w.shape == (edges.num_edges, self.weight_numel), "Invalid weight shape")
+            w = w.to(node_x.dtype).contiguous()
+        else:
+            w = node_x.new_empty(0)
+        return _GatherScatterShFn.apply(node_x.contiguous(), edge_vec.contiguous(), w, self, edges, bool(normalize), normalization)
 
     def _radial_description(self, net):
         """Arguments of the library's fused radial-network kernel for ``net``; None when ``net`` is not a two-layer

@@ -66,7 +66,7 @@ class HipTensorProduct(torch.nn.Module):
             ins = [(a, b, c, mode, hw, pw * pw) for a, b, c, mode, hw, pw in self.instructions]
             tp = TensorProduct(
                 in1, in2, out, ins, irrep_normalization="none", path_normalization="none", internal_weights=False,
-                shared_weights=self.shared_weights, compile_left_right=not self.is_right, compile_right=self.is_right,
+                shared_weights=self.shared_weights, compile_right=self.is_right,  # right() runs on the forward kernel
             )  # fmt: skip
             assert all(abs(t.path_weight - row[5]) <= 1e-15 * abs(row[5]) for t, row in zip(tp.instructions, self.instructions))
             tp.compile(torch.float32)  # refusals of the library surface here, as E3xError

@@ -249,6 +249,23 @@ int e3x_tp_gather_scatter_ws(e3x_plan* plan, const void* node_x, const void* edg
 int e3x_src_rows_build(const void* src, int idx_bits, const int32_t* perm, int64_t E, int64_t num_src_nodes,
                        int32_t* src_rows, void* stream);
 
+/* e3x_tp_gather_scatter_ws for plans whose second input is the spherical harmonics of the edge vectors,
+ * irreps_in2 = 0e + 1o + ... up to lmax <= 3 with multiplicity 1 (what the reference's convolutions feed it:
+ * edge_attr = o3.spherical_harmonics(range(lmax + 1), edge_vec, normalize, normalization), e.g.
+ * e3nn/nn/models/gate_points_2101.py:329): the kernel reads edge_vec[E, 3] (always fp32, 12 bytes per edge) and
+ * forms the harmonics itself, with the arithmetic of e3x_sh_forward (e3nn/o3/_spherical_harmonics.py:93-112,
+ * :194-226), instead of reading a stored [E, (lmax + 1)^2] tensor.  Equal to e3x_sh_forward followed by
+ * e3x_tp_gather_scatter_ws up to the rounding of the fused multiply-adds.  `normalize` / `normalization`
+ * (E3X_NORM_*) as in e3x_sh_forward.  A code object of its own per (normalize, normalization), built on first use or
+ * ahead of time (no GPU needed) by e3x_tp_plan_prepare_gather_scatter_sh, which returns E3X_ERR_INVALID for plans
+ * this does not apply to (not all-uvu, shared weights, another second input).  Vector-ALU kernels in either
+ * storage type; no workspace. */
+int e3x_tp_plan_prepare_gather_scatter_sh(e3x_plan* plan, int32_t normalize, int32_t normalization);
+int e3x_tp_gather_scatter_sh(e3x_plan* plan, const void* node_x, const float* edge_vec, const void* w, const void* src,
+                             int idx_bits, const int32_t* rowptr, const int32_t* perm, const int32_t* row_order,
+                             const int32_t* src_rows, void* out, int64_t E, int64_t num_src_nodes,
+                             int64_t num_out_nodes, int32_t normalize, int32_t normalization, void* stream);
+
 /* Gradients of the `uvu` product (plain: src = dst = NULL, row e of every table; fused: the edge lists
  * of e3x_tp_gather_scatter, unsorted) with respect to the per-sample weights and the second input:
  *   grad_w[E, weight_numel] (shared weights: one [weight_numel] vector summed over the edges with fp32 atomics),

@@ -55,6 +55,24 @@ def oracle_rows(tp, rows, node_x, attr, w, src, dst, dtype=torch.float32):
     return ref, n_edges
 
 
+def oracle_rows_fp64_attr(tp, rows, node_x, attr64, w, src, dst):
+    """As oracle_rows, with the edge attributes given in float64 on the CPU (the oracle's own harmonics)."""
+    spec = oracle_spec(tp)
+    dst_l = dst.long()
+    ref = np.zeros((len(rows), tp.irreps_out.dim))
+    n_edges = 0
+    for r, row in enumerate(rows):
+        e = torch.nonzero(dst_l == row).flatten()
+        if e.numel() == 0:
+            continue
+        s = src[e].long()
+        s = torch.where(s < 0, s + node_x.shape[0], s)
+        msg = otp.tp_forward(spec, node_x[s].float().cpu().numpy(), attr64[e.cpu()].numpy(), w[e].float().cpu().numpy())
+        ref[r] = msg.sum(axis=0)
+        n_edges += e.numel()
+    return ref, n_edges
+
+
 def unfused(tp, node_x, attr, w, src, dst, N, chunk=250_000):
     """plain tensor product on gathered rows, then index_add_ (fp32 atomics: the summation order differs)"""
     out = torch.zeros(N, tp.irreps_out.dim, device=DEV, dtype=torch.float32)
@@ -111,6 +129,18 @@ def test_nequip_configuration_at_full_size(side, label):
     if side > 80:
         check_sum_tolerance(out, unfused(tp, node_x, attr, w, src_t, dst_t, N), "NequIP", 2e-6)
     assert torch.isfinite(out).all()
+    # the harmonics formed inside the kernel from the 12-byte edge vectors: against the oracle on the oracle's own
+    # harmonics of the sampled rows (fp64 of the fp32 vectors), and against the stored-attribute kernel on every row
+    del out
+    out_sh = tp.forward_gather_scatter_sh(node_x, vec, w, edges, True, "component")
+    attr64 = torch.zeros(E, 9, dtype=torch.float64)
+    for row in rows:
+        e = torch.nonzero(dst_t == row).flatten().cpu()
+        if e.numel():
+            attr64[e] = torch.from_numpy(osh([0, 1, 2], vec[e.to(DEV)].cpu().numpy().astype(np.float64), True, "component"))
+    ref_sh, _ = oracle_rows_fp64_attr(tp, rows, node_x, attr64, w, src_t, dst_t)
+    assert_close(out_sh[rows], ref_sh, atol=1e-4 * max(1.0, (deg.float().mean().item() / 37) ** 0.5), rtol=1e-5, what=f"NequIP uvu, harmonics in the kernel ({label})")
+    check_sum_tolerance(out_sh, tp.forward_gather_scatter(node_x, attr, w, edges=edges), "harmonics in the kernel vs stored", 2e-6)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -197,6 +197,108 @@ def test_fused_matches_oracle(maker, N, E, idx):
     assert (out - unfused).abs().max().item() < 1e-4 * scale
 
 
+@pytest.mark.parametrize("idx", [torch.int32, torch.int64])
+def test_edge_list_held_in_destination_order(idx):
+    # per-edge tensors rewritten once in the order the kernels walk the edges, and an edge list the caller already holds
+    # grouped by destination (no permutation handed to the kernels): the same bits as the caller's order in the forward
+    # pass and in the per-edge gradients; the gradient of the node features sums the edges leaving a node in the
+    # order of the list it is given, so there the two agree to rounding
+    tp = ks.cfg3(True)
+    N, E = 300, 9_000
+    src, dst = random_graph(N, E, seed=11, dtype=idx)
+    src[3] = -2
+    node_x, attr, w = seeded(N, tp.irreps_in1.dim, seed=1).to(DEV), seeded(E, 9, seed=2).to(DEV), seeded(E, tp.weight_numel, seed=3).to(DEV)
+    cot = seeded(N, tp.irreps_out.dim, seed=4).to(DEV)
+    edges = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    assert edges.walk_perm is not None
+
+    def run(e, a, ww):
+        x, a, ww = (t.clone().requires_grad_() for t in (node_x, a, ww))
+        out = tp.forward_gather_scatter(x, a, ww, edges=e)
+        return (out,) + torch.autograd.grad(out, (x, a, ww), cot)
+
+    ref = run(edges, attr, w)
+    se = edges.sorted()
+    assert se.walk_perm is None and se.sorted() is se and torch.equal(se.rowptr, edges.rowptr)
+    attr_s, w_s = edges.in_sorted_order(attr, w)
+    got = run(se, attr_s, w_s)
+    perm = edges.perm.long()
+    assert torch.equal(got[0], ref[0])
+    assert (got[1] - ref[1]).abs().max().item() <= 1e-5 * ref[1].abs().max().item()
+    assert torch.equal(got[2], ref[2][perm]) and torch.equal(got[3], ref[3][perm])
+    # the caller's own list already grouped by destination: detected, walked by position
+    order = torch.argsort(dst.long(), stable=True)
+    pre = DstSortedEdges(src[order].to(DEV), dst[order].to(DEV), N)
+    assert pre.walk_perm is None and pre.sorted() is pre
+    assert pre.in_sorted_order(attr_s) is attr_s
+    again = run(pre, attr_s, w_s)
+    for a, b in zip(again, got):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("maker,N,E,idx,normalize,normalization", [
+    (lambda: ks.cfg3(True), 700, 26_000, torch.int64, True, "component"),
+    (lambda: ks.cfg3(True), 90, 2_000, torch.int32, False, "integral"),
+    (lambda: ks.cfg3(False), 300, 9_000, torch.int64, True, "norm"),
+    (lambda: ks.cfg4("A"), 60, 1_500, torch.int32, True, "component"),
+    (ks.odd_mul, 90, 2_000, torch.int32, True, "integral"),
+])  # fmt: skip
+def test_fused_with_the_harmonics_formed_in_the_kernel(maker, N, E, idx, normalize, normalization):
+    # edge_attr = spherical_harmonics(0 .. lmax, edge_vec) evaluated inside the message kernel from the 12-byte vectors:
+    # against the oracle on the oracle's own harmonics (float64), a zero vector and negative source indices included
+    from oracle.spherical_harmonics import spherical_harmonics as osh
+
+    tp = maker()
+    src, dst = random_graph(N, E, seed=3, dtype=idx)
+    src[5] = -1  # wraps to the last node, as torch indexing does
+    node_x = seeded(N, tp.irreps_in1.dim, seed=1)
+    vec = seeded(E, 3, seed=2) * (1.0 if normalize else 0.7)
+    vec[7] = 0.0  # normalize: the l = 0 constant and zeros elsewhere, not NaN
+    ls = list(range(tp.irreps_in2.lmax + 1))
+    w = seeded(E, tp.weight_numel, seed=4)
+    edges = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    out = tp.forward_gather_scatter_sh(node_x.to(DEV), vec.to(DEV), w.to(DEV), edges, normalize, normalization)
+    attr64 = osh(ls, vec.numpy().astype(np.float64), normalize, normalization)
+    ref = tp_gather_scatter(oracle_spec(tp), node_x.numpy(), attr64, w.numpy(), src.numpy(), dst.numpy(), N)
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert torch.isfinite(out).all()
+    assert_close(out, ref, atol=1e-4 * scale ** 0.5, rtol=1e-5, what=f"harmonics in the kernel, {normalization}: {tp}")
+    # the two-kernel path (harmonics stored, then the message kernel): same sums up to the harmonics' own rounding
+    attr = o3.spherical_harmonics(ls, vec.to(DEV), normalize, normalization)
+    two = tp.forward_gather_scatter(node_x.to(DEV), attr, w.to(DEV), edges=edges)
+    assert (out - two).abs().max().item() <= 2e-6 * scale
+
+
+def test_fused_with_the_harmonics_formed_in_the_kernel_gradients_and_refusals():
+    from oracle.torch_cpu import spherical_harmonics_torch, tp_gather_scatter_torch
+
+    tp = ks.cfg3(True)
+    spec = oracle_spec(tp)
+    N, E = 120, 3000
+    src, dst = random_graph(N, E, seed=5)
+    node_x, vec, w = seeded(N, tp.irreps_in1.dim, seed=1), seeded(E, 3, seed=2), seeded(E, tp.weight_numel, seed=3)
+    cot = seeded(N, tp.irreps_out.dim, seed=4)
+    a, b, c = (t.double().requires_grad_() for t in (node_x, vec, w))
+    ref = tp_gather_scatter_torch(spec, a, spherical_harmonics_torch(2, b, True), c, src, dst, N)
+    r1, r2, rw = torch.autograd.grad(ref, (a, b, c), cot.double())
+    edges = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    x, v, ww = (t.to(DEV).requires_grad_() for t in (node_x, vec, w))
+    out = tp.forward_gather_scatter_sh(x, v, ww, edges, True, "component")
+    g1, g2, gw = torch.autograd.grad(out, (x, v, ww), cot.to(DEV))
+    scale = lambda r: max(1.0, float(r.abs().max()))  # noqa: E731
+    assert_close(out, ref.detach().numpy(), atol=1e-4 * scale(ref.detach()) ** 0.5)
+    assert_close(g1, r1.numpy(), atol=1e-4 * scale(r1), what="d/dnode_x (harmonics in the kernel)")
+    assert_close(g2, r2.numpy(), atol=1e-4 * scale(r2), what="d/dedge_vec (harmonics in the kernel)")
+    assert_close(gw, rw.numpy(), what="d/dweight (harmonics in the kernel)")
+    # plans whose second input is something else are refused
+    other = ks.scalar_exact()
+    e2 = DstSortedEdges(src.to(DEV), dst.to(DEV), N)
+    with pytest.raises(NotImplementedError):
+        other.forward_gather_scatter_sh(seeded(N, 32).to(DEV), vec.to(DEV), seeded(E, other.weight_numel).to(DEV), e2)
+    with pytest.raises(TypeError):
+        tp.forward_gather_scatter_sh(node_x.to(DEV), vec.double().to(DEV), w.to(DEV), edges)
+
+
 @pytest.mark.parametrize("variant,N,E,idx", [("A", 50, 1000, torch.int32), ("A", 7, 900, torch.int64), ("B", 40, 700, torch.int32),
                                               ("A", 300, 5, torch.int64)])  # fmt: skip
 def test_fused_bf16_storage(variant, N, E, idx):

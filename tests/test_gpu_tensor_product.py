@@ -361,7 +361,7 @@ def test_provider_binding_runs_the_same_kernels():
             got = mod(x1, x2, w)
             assert got.shape == (5, 3, tp.irreps_out.dim) and torch.equal(got, ref)
         with pytest.raises(RuntimeError, match="share one dtype"):
-            gm(x1, x2.double(), w)
+            gm(x1, x2.bfloat16(), w)
         with pytest.raises(RuntimeError, match="float32 or bfloat16"):
             gm(x1.double(), x2.double(), w.double())
 
