@@ -80,10 +80,14 @@ _SIGNATURES = {
     "e3x_tp_backward_w_uvw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "e3x_gate_forward": (c_int, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p]),
     "e3x_gate_backward": (c_int, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p]),
+    "e3x_gate_backward2": (c_int, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                   c_int64, c_int64, c_int32, c_void_p]),
     "e3x_sh_forward": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int64,
                                c_int32, c_void_p]),
     "e3x_sh_backward": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
                                 c_int32, c_void_p]),
+    "e3x_sh_backward2": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_int64, c_int32, c_void_p]),
     "e3x_fc_plan_create": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, ctypes.c_double, c_int32, ctypes.c_double,
                                    ctypes.c_double, c_int32, ctypes.POINTER(c_void_p)]),
     "e3x_fc_plan_create_fused": (c_int, [ctypes.POINTER(c_int32), c_int32, c_int32, ctypes.c_double, c_int32, ctypes.c_double,

@@ -57,6 +57,25 @@ __device__ __forceinline__ void activation(int kind, float x, float& f, float& d
   }
 }
 
+// second derivative of activation `kind` at x (0 for the piecewise linear ones, away from their kink)
+__device__ __forceinline__ float activation_d2(int kind, float x) {
+  switch (kind) {
+    case E3X_ACT_SILU: {
+      const float s = sigmoidf(x);
+      return s * (1.f - s) * (2.f + x * (1.f - 2.f * s));
+    }
+    case E3X_ACT_TANH: {
+      const float f = tanhf(x);
+      return -2.f * f * (1.f - f * f);
+    }
+    case E3X_ACT_SIGMOID: {
+      const float f = sigmoidf(x);
+      return f * (1.f - f) * (1.f - 2.f * f);
+    }
+    default: return 0.f;
+  }
+}
+
 // Thread (tx, ty) of a 64 x 4 block owns column 64 blockIdx.x + tx and walks rows 4 blockIdx.y + ty, + 4 gridDim.y, ...:
 // the block tables are searched once per thread, consecutive lanes touch consecutive columns of a row.
 constexpr int kCols = 64, kRows = 4;
@@ -138,6 +157,92 @@ __global__ __launch_bounds__(kCols* kRows) void gate_bwd_kernel(Tables t, const 
       v += g_cst * df * s;
     }
     gx[z * in_dim + c] = v;
+  }
+}
+
+// The derivative of the backward pass, for a cotangent `cot` on its result gx: with Phi = <cot, gx(x, gout)>,
+//   gg = dPhi/dgout (walk over the output columns) and gx2 = dPhi/dx (walk over the input columns).
+// A scalar block contributes cot * cst * a'(x) to gg and cot * gout * cst * a''(x) to gx2; a gated component with gate
+// s, value y, output gradient g and cotangents (cs, cy): gg = cy cst a(s) + cs cst a'(s) y,
+// dPhi/dy = cs cst a'(s) g, dPhi/ds = cst a'(s) sum(cy g) + cs cst a''(s) sum(g y).
+__global__ __launch_bounds__(kCols* kRows) void gate_bwd2_gg_kernel(Tables t, const float* __restrict__ x,
+                                                                    const float* __restrict__ cot, float* __restrict__ gg,
+                                                                    long long n_rows, int in_dim, int out_dim) {
+  const int c = blockIdx.x * kCols + (threadIdx.x % kCols);
+  if (c >= out_dim) return;
+  int kind = -1, src = 0, gate = -1;
+  float cst = 0.f;
+  for (int b = 0; b < t.n_act; ++b) {
+    const e3x_act_block& a = t.act[b];
+    if (c >= a.offset_out && c < a.offset_out + a.count) kind = a.act, cst = a.cst, src = a.offset_in + (c - a.offset_out);
+  }
+  for (int b = 0; b < t.n_gate; ++b) {
+    const e3x_gate_block& g = t.gate[b];
+    if (c >= g.offset_out && c < g.offset_out + g.mul * g.dim) {
+      const int rel = c - g.offset_out;
+      kind = g.act, cst = g.cst, src = g.gated_offset_in + rel, gate = g.gate_offset_in + rel / g.dim;
+    }
+  }
+  for (long long z = (long long)blockIdx.y * kRows + threadIdx.x / kCols; z < n_rows; z += (long long)gridDim.y * kRows) {
+    const float* row = x + z * in_dim;
+    const float* crow = cot + z * in_dim;
+    float v = 0.f;
+    if (kind >= 0) {
+      float f, df;
+      activation(kind, row[gate >= 0 ? gate : src], f, df);
+      v = gate >= 0 ? cst * (crow[src] * f + crow[gate] * df * row[src]) : cst * df * crow[src];
+    }
+    gg[z * out_dim + c] = v;
+  }
+}
+
+__global__ __launch_bounds__(kCols* kRows) void gate_bwd2_gx_kernel(Tables t, const float* __restrict__ x,
+                                                                    const float* __restrict__ gout,
+                                                                    const float* __restrict__ cot, float* __restrict__ gx2,
+                                                                    long long n_rows, int in_dim, int out_dim) {
+  const int c = blockIdx.x * kCols + (threadIdx.x % kCols);
+  if (c >= in_dim) return;
+  int a_kind = -1, a_out = 0;
+  float a_cst = 0.f;
+  int y_kind = -1, y_out = 0, y_gate = 0;
+  float y_cst = 0.f;
+  int g_kind = -1, g_out = 0, g_src = 0, g_dim = 0;
+  float g_cst = 0.f;
+  for (int b = 0; b < t.n_act; ++b) {
+    const e3x_act_block& a = t.act[b];
+    if (c >= a.offset_in && c < a.offset_in + a.count) a_kind = a.act, a_cst = a.cst, a_out = a.offset_out + (c - a.offset_in);
+  }
+  for (int b = 0; b < t.n_gate; ++b) {
+    const e3x_gate_block& g = t.gate[b];
+    if (c >= g.gated_offset_in && c < g.gated_offset_in + g.mul * g.dim) {
+      const int rel = c - g.gated_offset_in;
+      y_kind = g.act, y_cst = g.cst, y_out = g.offset_out + rel, y_gate = g.gate_offset_in + rel / g.dim;
+    }
+    if (c >= g.gate_offset_in && c < g.gate_offset_in + g.mul) {
+      const int u = c - g.gate_offset_in;
+      g_kind = g.act, g_cst = g.cst, g_out = g.offset_out + u * g.dim, g_src = g.gated_offset_in + u * g.dim, g_dim = g.dim;
+    }
+  }
+  for (long long z = (long long)blockIdx.y * kRows + threadIdx.x / kCols; z < n_rows; z += (long long)gridDim.y * kRows) {
+    const float* row = x + z * in_dim;
+    const float* grow = gout + z * out_dim;
+    const float* crow = cot + z * in_dim;
+    float v = 0.f, f, df;
+    if (a_kind >= 0) v += a_cst * activation_d2(a_kind, row[c]) * grow[a_out] * crow[c];
+    if (y_kind >= 0) {
+      activation(y_kind, row[y_gate], f, df);
+      v += y_cst * df * grow[y_out] * crow[y_gate];
+    }
+    if (g_kind >= 0) {
+      activation(g_kind, row[c], f, df);
+      float s_cg = 0.f, s_gy = 0.f;
+      for (int m = 0; m < g_dim; ++m) {
+        s_cg += crow[g_src + m] * grow[g_out + m];
+        s_gy += grow[g_out + m] * row[g_src + m];
+      }
+      v += g_cst * (df * s_cg + activation_d2(g_kind, row[c]) * crow[c] * s_gy);
+    }
+    gx2[z * in_dim + c] = v;
   }
 }
 
@@ -268,5 +373,29 @@ extern "C" int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, cons
   hipLaunchKernelGGL(gate_bwd_kernel, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
                      (const float*)grad_out, (float*)grad_x, (long long)Z, (int)in_dim, (int)out_dim);
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward: kernel launch failed");
+  return E3X_OK;
+}
+
+extern "C" int e3x_gate_backward2(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_block* gates, int32_t n_gates,
+                                  const void* x, const void* grad_out, const void* cot_x, void* grad_grad_out, void* grad_x,
+                                  int64_t Z, int64_t in_dim, int64_t out_dim, int32_t dtype, void* stream) {
+  if (dtype != E3X_F32) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward2: only fp32 storage is implemented");
+  Tables t;
+  int rc = fill_tables("e3x_gate_backward2", acts, n_acts, gates, n_gates, in_dim, out_dim, &t);
+  if (rc) return rc;
+  if (Z < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward2: negative batch");
+  if (Z == 0) return E3X_OK;
+  if ((in_dim && (!x || !cot_x || !grad_x)) || (out_dim && (!grad_out || !grad_grad_out)))
+    return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward2: null pointer");
+  if (out_dim) {
+    hipLaunchKernelGGL(gate_bwd2_gg_kernel, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
+                       (const float*)cot_x, (float*)grad_grad_out, (long long)Z, (int)in_dim, (int)out_dim);
+    if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward2: kernel launch failed");
+  }
+  if (in_dim) {
+    hipLaunchKernelGGL(gate_bwd2_gx_kernel, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
+                       (const float*)grad_out, (const float*)cot_x, (float*)grad_x, (long long)Z, (int)in_dim, (int)out_dim);
+    if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward2: kernel launch failed");
+  }
   return E3X_OK;
 }

@@ -149,6 +149,7 @@ __global__ __launch_bounds__(kWave* kWavesPerBlock) void sh_tile_kernel(const fl
 // input, so the derivative code is the forward code (no hand-derived formulas to get wrong).
 struct Dual {
   float v, dx, dy, dz;
+  static __device__ __forceinline__ Dual constant(float c) { return {c, 0.f, 0.f, 0.f}; }
 };
 __device__ __forceinline__ Dual operator+(Dual a, Dual b) { return {a.v + b.v, a.dx + b.dx, a.dy + b.dy, a.dz + b.dz}; }
 __device__ __forceinline__ Dual operator-(Dual a, Dual b) { return {a.v - b.v, a.dx - b.dx, a.dy - b.dy, a.dz - b.dz}; }
@@ -157,9 +158,49 @@ __device__ __forceinline__ Dual operator*(Dual a, Dual b) {
 }
 __device__ __forceinline__ Dual operator*(float c, Dual a) { return {c * a.v, c * a.dx, c * a.dy, c * a.dz}; }
 
-template <int LMAX>
-__device__ __forceinline__ void sh_poly_dual(Dual x, Dual y, Dual z, Dual (&o)[(LMAX + 1) * (LMAX + 1)]) {
-  o[0] = {1.f, 0.f, 0.f, 0.f};
+// Second order: a value with its gradient d[i] = d/dx_i, its derivative a = d/dt along one fixed direction, and the
+// gradient of that directional derivative, ad[i] = d^2 / (dt dx_i) -- what the derivative of a backward pass needs
+// (the Hessian applied to one vector), again with the forward code as derivative code.
+struct Dual2 {
+  float v, d[3], a, ad[3];
+  static __device__ __forceinline__ Dual2 constant(float c) { return {c, {0.f, 0.f, 0.f}, 0.f, {0.f, 0.f, 0.f}}; }
+};
+__device__ __forceinline__ Dual2 operator+(Dual2 p, Dual2 q) {
+  return {p.v + q.v, {p.d[0] + q.d[0], p.d[1] + q.d[1], p.d[2] + q.d[2]}, p.a + q.a, {p.ad[0] + q.ad[0], p.ad[1] + q.ad[1], p.ad[2] + q.ad[2]}};
+}
+__device__ __forceinline__ Dual2 operator-(Dual2 p, Dual2 q) {
+  return {p.v - q.v, {p.d[0] - q.d[0], p.d[1] - q.d[1], p.d[2] - q.d[2]}, p.a - q.a, {p.ad[0] - q.ad[0], p.ad[1] - q.ad[1], p.ad[2] - q.ad[2]}};
+}
+__device__ __forceinline__ Dual2 operator*(Dual2 p, Dual2 q) {
+  Dual2 r;
+  r.v = p.v * q.v;
+  r.a = fmaf(p.a, q.v, p.v * q.a);
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    r.d[i] = fmaf(p.d[i], q.v, p.v * q.d[i]);
+    r.ad[i] = fmaf(p.ad[i], q.v, fmaf(p.d[i], q.a, fmaf(p.a, q.d[i], p.v * q.ad[i])));
+  }
+  return r;
+}
+__device__ __forceinline__ Dual2 operator*(float c, Dual2 p) {
+  return {c * p.v, {c * p.d[0], c * p.d[1], c * p.d[2]}, c * p.a, {c * p.ad[0], c * p.ad[1], c * p.ad[2]}};
+}
+// f(p) for a scalar function with f(p.v) = f0, f'(p.v) = f1, f''(p.v) = f2
+__device__ __forceinline__ Dual2 chain(Dual2 p, float f0, float f1, float f2) {
+  Dual2 r;
+  r.v = f0;
+  r.a = f1 * p.a;
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    r.d[i] = f1 * p.d[i];
+    r.ad[i] = fmaf(f2 * p.a, p.d[i], f1 * p.ad[i]);
+  }
+  return r;
+}
+
+template <int LMAX, class D>
+__device__ __forceinline__ void sh_poly_dual(D x, D y, D z, D (&o)[(LMAX + 1) * (LMAX + 1)]) {
+  o[0] = D::constant(1.f);
   if constexpr (LMAX >= 1) {
     const float c = 1.7320508075688772f;
     o[1] = c * x;
@@ -168,9 +209,9 @@ __device__ __forceinline__ void sh_poly_dual(Dual x, Dual y, Dual z, Dual (&o)[(
   }
   if constexpr (LMAX >= 2) {
     const float r15 = 3.872983346207417f, r5 = 2.23606797749979f;
-    const Dual y2 = y * y, s = x * x + z * z;
-    const Dual a20 = r15 * (x * z);
-    const Dual a24 = (0.5f * r15) * (z * z - x * x);
+    const D y2 = y * y, s = x * x + z * z;
+    const D a20 = r15 * (x * z);
+    const D a24 = (0.5f * r15) * (z * z - x * x);
     o[4] = a20;
     o[5] = r15 * (x * y);
     o[6] = r5 * (y2 - 0.5f * s);
@@ -178,7 +219,7 @@ __device__ __forceinline__ void sh_poly_dual(Dual x, Dual y, Dual z, Dual (&o)[(
     o[8] = a24;
     if constexpr (LMAX >= 3) {
       const float r7 = 2.6457513110645907f, c0 = 1.0801234497346435f, c2 = 1.6201851746019651f;
-      const Dual t = 4.0f * y2 - s;
+      const D t = 4.0f * y2 - s;
       o[9] = c0 * (a20 * z + a24 * x);
       o[10] = r7 * (a20 * y);
       o[11] = c2 * (t * x);
@@ -188,6 +229,63 @@ __device__ __forceinline__ void sh_poly_dual(Dual x, Dual y, Dual z, Dual (&o)[(
       o[15] = c0 * (a24 * z - a20 * x);
     }
   }
+}
+
+// The derivative of the backward pass.  With phi(x) = sum_c g_c Y_c(x) the backward pass returns grad phi; for a
+// cotangent t[3] on that result this kernel returns d<t, grad phi>/dg_c = (directional derivative of Y_c along t) and
+// d<t, grad phi>/dx = (Hessian of phi) t, from one evaluation of the polynomials on Dual2 numbers whose fixed
+// direction is t.  The normalisation x / max(|x|, 1e-12) is part of the differentiated function.
+template <int LMAX, bool NORMALIZE>
+__global__ __launch_bounds__(256) void sh_bwd2_kernel(const float* __restrict__ xyz, const float* __restrict__ gout,
+                                                      const float* __restrict__ cot, float* __restrict__ ggout,
+                                                      float* __restrict__ gxyz, long long n, Scale4 sc) {
+  constexpr int NC = (LMAX + 1) * (LMAX + 1);
+  const long long v = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (v >= n) return;
+  Dual2 p[3];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    p[i] = Dual2::constant(xyz[v * 3 + i]);
+    p[i].d[i] = 1.f;
+    p[i].a = cot[v * 3 + i];
+  }
+  if constexpr (NORMALIZE) {
+    const Dual2 s = p[0] * p[0] + p[1] * p[1] + p[2] * p[2];
+    const float nrm = sqrtf(s.v);
+    Dual2 inv;
+    if (nrm < 1e-12f) {
+      inv = Dual2::constant(1e12f);  // below the clamp the map is x / 1e-12
+    } else {
+      const float r = 1.0f / nrm, r2 = r * r;  // s^(-1/2) and its derivatives -1/2 s^(-3/2), 3/4 s^(-5/2)
+      inv = chain(s, r, -0.5f * r * r2, 0.75f * r * r2 * r2);
+    }
+#pragma unroll
+    for (int i = 0; i < 3; ++i) p[i] = p[i] * inv;
+  }
+  Dual2 o[NC];
+  sh_poly_dual<LMAX>(p[0], p[1], p[2], o);
+  float gx[3] = {0.f, 0.f, 0.f};
+  const float* g = gout + v * NC;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int l = c >= 9 ? 3 : (c >= 4 ? 2 : (c >= 1 ? 1 : 0));
+    ggout[v * NC + c] = sc.s[l] * o[c].a;
+    const float gc = g[c] * sc.s[l];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) gx[i] = fmaf(gc, o[c].ad[i], gx[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < 3; ++i) gxyz[v * 3 + i] = gx[i];
+}
+
+template <int LMAX>
+void launch_bwd2(bool normalize, const float* xyz, const float* gout, const float* cot, float* ggout, float* gxyz, long long n,
+                 Scale4 sc, hipStream_t st) {
+  const long long blocks = (n + 255) / 256;
+  if (normalize)
+    hipLaunchKernelGGL((sh_bwd2_kernel<LMAX, true>), dim3((unsigned)blocks), dim3(256), 0, st, xyz, gout, cot, ggout, gxyz, n, sc);
+  else
+    hipLaunchKernelGGL((sh_bwd2_kernel<LMAX, false>), dim3((unsigned)blocks), dim3(256), 0, st, xyz, gout, cot, ggout, gxyz, n, sc);
 }
 
 template <int LMAX, bool NORMALIZE>
@@ -559,5 +657,37 @@ extern "C" int e3x_sh_backward(const int32_t* ls, int32_t n_ls, int32_t normaliz
     default: launch_bwd<3>(normalize, px, pg, po, n, sc, st); break;
   }
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_sh_backward: kernel launch failed");
+  return E3X_OK;
+}
+
+extern "C" int e3x_sh_backward2(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization,
+                                const void* xyz, const void* grad_out, const void* cot_xyz, void* grad_grad_out,
+                                void* grad_xyz, int64_t n, int32_t dtype, void* stream) {
+  if (!ls || n_ls <= 0 || n < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward2: empty l list or negative n");
+  if (dtype != E3X_F32) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward2: only fp32 storage is implemented");
+  if (normalization < 0 || normalization > 2)
+    return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward2: normalization must be integral, component or norm");
+  for (int i = 0; i < n_ls; ++i)
+    if (ls[i] != i || i > 3)
+      return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward2: second derivatives are implemented for the l lists 0 .. lmax <= 3");
+  if (n == 0) return E3X_OK;
+  if (!xyz || !grad_out || !cot_xyz || !grad_grad_out || !grad_xyz) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward2: null pointer");
+  if (n >= (1LL << 31) * 256) return e3x::fail(E3X_ERR_INVALID, "e3x_sh_backward2: too many vectors for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  Scale4 sc;
+  for (int l = 0; l < 4; ++l) {
+    sc.s[l] = 1.0f;
+    if (normalization == E3X_NORM_INTEGRAL) sc.s[l] = (float)(1.0 / std::sqrt(4.0 * M_PI));
+    if (normalization == E3X_NORM_NORM) sc.s[l] = (float)(1.0 / std::sqrt(2.0 * l + 1.0));
+  }
+  const float *px = (const float*)xyz, *pg = (const float*)grad_out, *pc = (const float*)cot_xyz;
+  float *pgg = (float*)grad_grad_out, *po = (float*)grad_xyz;
+  switch (n_ls - 1) {
+    case 0: launch_bwd2<0>(normalize, px, pg, pc, pgg, po, n, sc, st); break;
+    case 1: launch_bwd2<1>(normalize, px, pg, pc, pgg, po, n, sc, st); break;
+    case 2: launch_bwd2<2>(normalize, px, pg, pc, pgg, po, n, sc, st); break;
+    default: launch_bwd2<3>(normalize, px, pg, pc, pgg, po, n, sc, st); break;
+  }
+  if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_sh_backward2: kernel launch failed");
   return E3X_OK;
 }

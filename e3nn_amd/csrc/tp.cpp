@@ -1632,7 +1632,9 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
   if ((src == nullptr) != (dst == nullptr))
     return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: give both index arrays or neither");
   if (E == 0 || (!grad_w && !grad_x2)) return E3X_OK;
-  if (!grad_out || (P->in1_dim && !x1) || (P->in2_dim && !x2) || (P->weight_numel && !w))
+  // x2 is read by the weight gradient only, per-sample weights by the gradient of the second input only
+  if (!grad_out || (P->in1_dim && !x1) || (P->in2_dim && !x2 && grad_w) ||
+      (P->weight_numel && !w && (grad_x2 || P->shared_weights)))
     return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: null pointer");
   hipStream_t st = (hipStream_t)stream;
   int dev, rc;
@@ -1671,7 +1673,7 @@ extern "C" int e3x_tp_backward_w_x2(e3x_plan* P, const void* x1, const void* x2,
     const long long blocks = (items + K->waves_per_block - 1) / K->waves_per_block;
     if (blocks >= (1LL << 31)) return fail(E3X_ERR_INVALID, "e3x_tp_backward_w_x2: too many edges for one launch");
     // rows in 16-byte pieces need aligned rows (their lengths are multiples of four by construction of the variant)
-    const bool staged = K->bwd_lds && grad_w && !(((uintptr_t)x1 | (uintptr_t)w | (uintptr_t)grad_out | (uintptr_t)grad_w) & 15);
+    const bool staged = K->bwd_lds && grad_w && w && x2 && !(((uintptr_t)x1 | (uintptr_t)w | (uintptr_t)grad_out | (uintptr_t)grad_w) & 15);
     hipError_t err = hipModuleLaunchKernel(staged ? K->fn_bwd_edge_lds[dev] : K->fn_bwd_edge[dev], (unsigned)blocks, 1, 1,
                                            64 * K->waves_per_block, 1, 1, 0, st, args, nullptr);
     if (err != hipSuccess)

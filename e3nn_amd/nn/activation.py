@@ -98,10 +98,26 @@ class _GateFn(torch.autograd.Function):
         return mod._launch(x, None)
 
     @staticmethod
-    @once_differentiable
     def backward(ctx, g):
         (x,) = ctx.saved_tensors
-        return ctx.mod._launch(x, g.contiguous()), None
+        return _GateBackwardFn.apply(x, g.contiguous(), ctx.mod), None
+
+
+class _GateBackwardFn(torch.autograd.Function):
+    """``(x, g) -> d<g, gate(x)>/dx``, itself differentiable once more (``e3x_gate_backward2``: second derivatives of the
+    activations), which is what a loss on forces differentiates.  Third derivatives are not provided."""
+
+    @staticmethod
+    def forward(ctx, x, g, mod):
+        ctx.mod = mod
+        ctx.save_for_backward(x, g)
+        return mod._launch(x, g)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, cot):
+        x, g = ctx.saved_tensors
+        return ctx.mod._launch_second(x, g, cot.contiguous()) + (None,)
 
 
 class _BlockModule(torch.nn.Module):
@@ -129,6 +145,17 @@ class _BlockModule(torch.nn.Module):
                                          _lib.ptr(res), Z, in_dim, out_dim, 0, _lib.stream_ptr(x.device))  # fmt: skip
         _lib.check(rc)
         return res
+
+    def _launch_second(self, x, grad_out, cot):
+        """``(d/dx, d/dgrad_out)`` of ``<cot, backward(x, grad_out)>``."""
+        in_dim, out_dim = self._dims
+        Z = x.shape[0]
+        gx, gg = torch.empty_like(x), torch.empty_like(grad_out)
+        with torch.cuda.device(x.device):
+            rc = _lib.lib().e3x_gate_backward2(self._acts, self._n[0], self._gates, self._n[1], _lib.ptr(x), _lib.ptr(grad_out),
+                                               _lib.ptr(cot), _lib.ptr(gg), _lib.ptr(gx), Z, in_dim, out_dim, 0, _lib.stream_ptr(x.device))  # fmt: skip
+        _lib.check(rc)
+        return gx, gg
 
     def forward(self, features):
         in_dim, out_dim = self._dims

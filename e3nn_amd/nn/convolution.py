@@ -8,10 +8,9 @@
 ``node_features[edge_src]`` and the per-edge messages are never materialised.
 """
 import torch
-from torch.autograd.function import once_differentiable
 
 from ..o3.irreps import Irrep, Irreps
-from ..o3.tensor_product import FullyConnectedTensorProduct, TensorProduct, _permuted_weights
+from ..o3.tensor_product import _OUT, FullyConnectedTensorProduct, TensorProduct, _permuted_weights, _slot_backward, _TpSlot
 from .edges import DstSortedEdges
 from .fc import FullyConnectedNet
 from .message import message_instructions
@@ -21,20 +20,22 @@ class _Mix(torch.autograd.Function):
     """``sc + (c0 + alpha * c1) * conv`` with ``c0 = (1 - m) / sqrt(n)``, ``c1 = m / n`` (reference
     points_convolution.py:110-113 with the division by sqrt(num_neighbors) moved behind lin2 and alpha): two elementwise
     kernels forward and three backward, where autograd through the separate operations launches a dozen over the
-    [N, channels] arrays."""
+    [N, channels] arrays.  The backward pass is written in differentiable elementwise operations, so it can itself be
+    differentiated (``create_graph``)."""
 
     @staticmethod
     def forward(ctx, sc, alpha, conv, c0, c1):
         coeff = torch.addcmul(c0, alpha, c1)  # [N, channels]
-        ctx.save_for_backward(coeff, conv, c1)
+        ctx.save_for_backward(coeff, conv, c1, alpha, c0)
         return torch.addcmul(sc, coeff, conv)
 
     @staticmethod
-    @once_differentiable
     def backward(ctx, g):
-        coeff, conv, c1 = ctx.saved_tensors
+        coeff, conv, c1, alpha, c0 = ctx.saved_tensors
+        if torch.is_grad_enabled():
+            coeff = torch.addcmul(c0, alpha, c1)  # as a function of alpha
         need_sc, need_alpha, need_conv = ctx.needs_input_grad[:3]
-        g_alpha = ((g * conv) @ c1).unsqueeze(-1) if need_alpha else None
+        g_alpha = (g * conv * c1).sum(-1, keepdim=True) if need_alpha else None
         return (g if need_sc else None), g_alpha, (g * coeff if need_conv else None), None, None
 
 
@@ -53,11 +54,19 @@ class _Lin2Alpha(torch.autograd.Function):
         return lin2._plan(dt).forward(features, attr, w_lin2), head._plan(dt).forward(scalars, attr, w_alpha)
 
     @staticmethod
-    @once_differentiable
     def backward(ctx, g_conv, g_alpha):
         lin2, head = ctx.lin2, ctx.head
         features, attr, w_lin2, w_alpha, scalars = ctx.saved_tensors
         g_conv, g_alpha = g_conv.contiguous(), g_alpha.contiguous()
+        if torch.is_grad_enabled():
+            # under create_graph: the two products' own differentiable gradients
+            need = ctx.needs_input_grad
+            k = head.irreps_in1.dim
+            gf, _, gw_lin2 = _slot_backward(_TpSlot, _OUT, (features, attr, w_lin2), g_conv, (need[0], False, need[2]), lin2)
+            gs, _, gw_alpha = _slot_backward(_TpSlot, _OUT, (features[:, :k].contiguous(), attr, w_alpha), g_alpha, (need[0], False, need[3]), head)
+            if need[0]:
+                gf = gf + torch.nn.functional.pad(gs, (0, features.shape[1] - k))
+            return gf, None, gw_lin2, gw_alpha, None, None
         dt = features.dtype
         g_features = gw_lin2 = gw_alpha = None
         if ctx.needs_input_grad[2]:

@@ -13,65 +13,95 @@ Two device paths, both HIP kernels of this package:
 import ctypes
 
 import torch
-from torch.autograd.function import once_differentiable
 
 from .. import _lib
 from ..o3.tensor_product import TensorProduct
 from .activation import _KINDS, Activation, activation_name, second_moment_constant
 
 
-class _DenseFn(torch.autograd.Function):
-    """``x @ W * s`` of one layer on the one-layer specialisations of the fused kernel (s is folded in by the plans)."""
+_X, _WT, _G = 0, 1, 2
+
+
+def _dense_member(layer, slot, a, b):
+    """One of the three maps of the bilinear form ``F(x, W, g) = <g, x @ W * s>`` of a layer (``s`` is folded in by the
+    plans): ``_G``: ``x @ W * s``; ``_X``: ``g @ W^T * s``; ``_WT``: ``x^T @ g * s``; ``a, b`` are the other two slots in
+    the order (x, W, g)."""
+    if slot == _G:
+        return layer._fwd.forward(a, [b.contiguous()])
+    if slot == _X:  # g @ W^T * s through the plan [h_out -> h_in], whose own factor is 1 / sqrt(h_out)
+        w, g = a, b.contiguous()
+        g = g.clone() if g.data_ptr() % 16 else g
+        return layer._bwd.forward(g, [(w.t() * (layer._scale * layer.h_out**0.5)).contiguous()])
+    x, g = a.contiguous(), b.contiguous()
+    x, g = (t.clone() if t.data_ptr() % 16 else t for t in (x, g))
+    if layer._fwd.has_backward_w:
+        return layer._fwd.backward_w(x, g)
+    # wider than the dense weight-gradient kernel takes: the uvw weight gradient of the same layer
+    ones = x.new_ones(x.shape[0], 1)
+    gw = layer._tp._plan(torch.float32).backward_w_uvw(x, ones, g, True).reshape(layer.h_in, layer.h_out)
+    return gw * (layer._scale * layer.h_in**0.5)  # the tensor product's path weight is 1 / sqrt(h_in)
+
+
+class _DenseSlot(torch.autograd.Function):
+    """Member ``slot`` of the closed family of one dense layer (see ``_dense_member``): the derivative of a member with
+    respect to one of its arguments is another member, so derivatives of every order run on the same three kernels."""
 
     @staticmethod
-    def forward(ctx, x, w, layer):
-        ctx.layer = layer
-        ctx.save_for_backward(x, w)
-        return layer._fwd.forward(x, [w.contiguous()])
+    def forward(ctx, slot, layer, a, b):
+        ctx.slot, ctx.layer = slot, layer
+        ctx.save_for_backward(a, b)
+        return _dense_member(layer, slot, a, b)
 
     @staticmethod
-    @once_differentiable
-    def backward(ctx, g):
-        x, w = ctx.saved_tensors
-        layer = ctx.layer
-        g = g.contiguous()
-        if g.data_ptr() % 16:
-            g = g.clone()
-        gx = gw = None
-        if ctx.needs_input_grad[0]:
-            # g @ W^T * s through the plan [h_out -> h_in], whose own factor is 1 / sqrt(h_out)
-            wt = (w.t() * (layer._scale * layer.h_out**0.5)).contiguous()
-            gx = layer._bwd.forward(g, [wt])
-        if ctx.needs_input_grad[1]:
-            if layer._fwd.has_backward_w:
-                gw = layer._fwd.backward_w(x, g)
-            else:  # wider than the dense weight-gradient kernel takes: the uvw weight gradient of the same layer
-                ones = x.new_ones(x.shape[0], 1)
-                gw = layer._tp._plan(torch.float32).backward_w_uvw(x, ones, g, True).reshape(layer.h_in, layer.h_out)
-                gw = gw * (layer._scale * layer.h_in**0.5)  # the tensor product's path weight is 1 / sqrt(h_in)
-        return gx, gw, None
+    def backward(ctx, cot):
+        others = [t for t in range(3) if t != ctx.slot]
+        full = {ctx.slot: cot.contiguous(), **dict(zip(others, ctx.saved_tensors))}
+        grads = []
+        for t, need in zip(others, ctx.needs_input_grad[2:4]):
+            grads.append(_DenseSlot.apply(t, ctx.layer, *[full[u] for u in range(3) if u != t]) if need else None)
+        return (None, None, *grads)
+
+
+class _DenseFn:
+    """``x @ W * s`` of one layer on the one-layer specialisations of the fused kernel, under autograd."""
+
+    @staticmethod
+    def apply(x, w, layer):
+        return _DenseSlot.apply(_G, layer, x, w)
 
 
 class _ActDenseFn(torch.autograd.Function):
     """``dense(act(z))`` of two consecutive layers without the activated tensor: the dense kernel applies the
     activation to its input rows as it loads them (forward and weight gradient), and the backward pass takes the input
-    gradient through the activation in the epilogue of the input-gradient kernel, ``(g @ W^T * s) * cst * act'(z)``."""
+    gradient through the activation in the epilogue of the input-gradient kernel, ``(g @ W^T * s) * cst * act'(z)``.
+    Under ``create_graph`` the backward pass is the differentiable composition of the activation's and the dense
+    layer's own gradients instead (the activated tensor is then formed)."""
 
     @staticmethod
     def forward(ctx, z, w, layer, prev):
         ctx.plans = layer.act_dense_plans(prev)
         ctx.scale = layer._scale * layer.h_out**0.5
+        ctx.layer, ctx.prev = layer, prev
         ctx.save_for_backward(z, w)
         return ctx.plans[0].forward(z, [w.contiguous()])
 
     @staticmethod
-    @once_differentiable
     def backward(ctx, g):
         z, w = ctx.saved_tensors
         fwd, bwd = ctx.plans
         g = g.contiguous()
         if g.data_ptr() % 16:
             g = g.clone()
+        if torch.is_grad_enabled():
+            from .activation import _GateBackwardFn
+
+            h = ctx.prev.act(z)  # differentiable in z
+            gz = gw = None
+            if ctx.needs_input_grad[0]:
+                gz = _GateBackwardFn.apply(z, _DenseSlot.apply(_X, ctx.layer, w, g), ctx.prev.act)
+            if ctx.needs_input_grad[1]:
+                gw = _DenseSlot.apply(_WT, ctx.layer, h, g)
+            return gz, gw, None, None
         gz = gw = None
         if ctx.needs_input_grad[0]:
             gz = bwd.forward(g, [(w.t() * ctx.scale).contiguous()], z)

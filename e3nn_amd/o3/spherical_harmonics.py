@@ -15,6 +15,17 @@ from .irreps import Irreps
 _NORMALIZATION = {"integral": _lib.NORM_INTEGRAL, "component": _lib.NORM_COMPONENT, "norm": _lib.NORM_NORM}
 
 
+def _launch(entry, ls, normalize, normalization, n, device, *tensors):
+    arr = (ctypes.c_int32 * len(ls))(*ls)
+    with torch.cuda.device(device):
+        _lib.check(
+            getattr(_lib.lib(), entry)(
+                arr, len(ls), int(bool(normalize)), _NORMALIZATION[normalization], *[_lib.ptr(t) for t in tensors], n,
+                _lib.F32, _lib.stream_ptr(device),
+            )  # fmt: skip
+        )
+
+
 class _SphericalHarmonicsFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, ls, normalize, normalization):
@@ -27,35 +38,53 @@ class _SphericalHarmonicsFn(torch.autograd.Function):
         n = xyz.shape[0]
         n_out = sum(2 * l + 1 for l in ls)
         out = torch.empty(n, n_out, dtype=x.dtype, device=x.device)
-        arr = (ctypes.c_int32 * len(ls))(*ls)
-        with torch.cuda.device(x.device):
-            _lib.check(
-                _lib.lib().e3x_sh_forward(
-                    arr, len(ls), int(bool(normalize)), _NORMALIZATION[normalization], _lib.ptr(xyz), _lib.ptr(out), n,
-                    _lib.F32, _lib.stream_ptr(x.device),
-                )  # fmt: skip
-            )
-        ctx.save_for_backward(xyz)
-        ctx.cfg = (ls, normalize, normalization, batch)
+        _launch("e3x_sh_forward", ls, normalize, normalization, n, x.device, xyz, out)
+        ctx.save_for_backward(x)
+        ctx.cfg = (ls, normalize, normalization)
         return out.reshape(batch + (n_out,))
 
     @staticmethod
-    @once_differentiable
     def backward(ctx, g):
-        (xyz,) = ctx.saved_tensors
-        ls, normalize, normalization, batch = ctx.cfg
+        (x,) = ctx.saved_tensors
+        return _ShBackwardFn.apply(x, g, *ctx.cfg), None, None, None
+
+
+class _ShBackwardFn(torch.autograd.Function):
+    """``(x, g) -> grad_x <g, Y(x)>``, itself differentiable once more (``e3x_sh_backward2``): what a loss on forces
+    differentiates.  Third derivatives are not provided."""
+
+    @staticmethod
+    def forward(ctx, x, g, ls, normalize, normalization):
+        batch = x.shape[:-1]
+        xyz = x.reshape(-1, 3).contiguous()
         n = xyz.shape[0]
-        g = g.reshape(n, -1).contiguous()
+        g2 = g.reshape(n, -1).contiguous()
         gx = torch.empty_like(xyz)
-        arr = (ctypes.c_int32 * len(ls))(*ls)
-        with torch.cuda.device(xyz.device):
-            _lib.check(
-                _lib.lib().e3x_sh_backward(
-                    arr, len(ls), int(bool(normalize)), _NORMALIZATION[normalization], _lib.ptr(xyz), _lib.ptr(g),
-                    _lib.ptr(gx), n, _lib.F32, _lib.stream_ptr(xyz.device),
-                )  # fmt: skip
-            )
-        return gx.reshape(batch + (3,)), None, None, None
+        _launch("e3x_sh_backward", ls, normalize, normalization, n, x.device, xyz, g2, gx)
+        ctx.save_for_backward(xyz, g2)
+        ctx.cfg = (ls, normalize, normalization, batch, g.shape)
+        return gx.reshape(batch + (3,))
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, cot):
+        xyz, g = ctx.saved_tensors
+        ls, normalize, normalization, batch, g_shape = ctx.cfg
+        if tuple(ls) != tuple(range(len(ls))) or len(ls) > 4:
+            raise NotImplementedError("second derivatives of the spherical harmonics are implemented for l = 0 .. lmax <= 3")
+        n = xyz.shape[0]
+        cot = cot.reshape(n, 3).contiguous()
+        gg, gx = torch.empty_like(g), torch.empty_like(xyz)
+        _launch("e3x_sh_backward2", ls, normalize, normalization, n, xyz.device, xyz, g, cot, gg, gx)
+        return gx.reshape(batch + (3,)), gg.reshape(g_shape), None, None, None
+
+
+def _sh_forward(x, ls, normalize, normalization):
+    return _SphericalHarmonicsFn.apply(x, tuple(ls), normalize, normalization)
+
+
+def _sh_backward(x, g, ls, normalize, normalization):
+    return _ShBackwardFn.apply(x, g, tuple(ls), normalize, normalization)
 
 
 class SphericalHarmonics(torch.nn.Module):

@@ -19,7 +19,6 @@ from math import prod, sqrt
 from typing import List, Optional, Union
 
 import torch
-from torch.autograd.function import once_differentiable
 
 from .. import _lib, get_optimization_defaults
 from .irreps import Irreps
@@ -81,7 +80,7 @@ class _Plan:
         wn, fam, key = ctypes.c_int64(), ctypes.c_char_p(), ctypes.c_char_p()
         _lib.check(L.e3x_tp_plan_info(handle, ctypes.byref(wn), None, None, None, ctypes.byref(fam), ctypes.byref(key)))
         self.weight_numel, self.family, self.key = wn.value, fam.value.decode(), key.value.decode()
-        self.out_dim = irreps_out.dim
+        self.out_dim, self.in2_dim = irreps_out.dim, irreps_in2.dim
         self.arithmetic = L.e3x_tp_plan_arithmetic(handle, 0).decode()  # which instruction forms the products
         self._fused_grad_w = None  # whether the plan has the message-step backward kernel; asked on first use
 
@@ -218,9 +217,13 @@ class _Plan:
         return gw
 
     def backward_w_x2(self, x1, x2, w, grad_out, src, dst, want_w, want_x2, num_edges):
+        """``x2`` may be None when only ``want_x2`` is set (the weight gradient alone reads it), per-sample ``w`` when
+        only ``want_w`` is."""
         gw_shape = (self.weight_numel,) if self.shared_weights else (num_edges, self.weight_numel)
         gw = torch.empty(gw_shape, dtype=x1.dtype, device=x1.device) if want_w else None
-        gx2 = torch.empty(num_edges, x2.shape[1], dtype=x1.dtype, device=x1.device) if want_x2 else None
+        gx2 = torch.empty(num_edges, self.in2_dim, dtype=x1.dtype, device=x1.device) if want_x2 else None
+        if w is None and self.shared_weights and self.weight_numel:
+            w = x1.new_zeros(self.weight_numel)
         bits = src.element_size() * 8 if src is not None else 64
         with torch.cuda.device(x1.device):
             _lib.check(
@@ -256,99 +259,169 @@ def _permuted_weights(tp, w, perm):
     return w.index_select(-1, index)
 
 
-class _TensorProductFn(torch.autograd.Function):
-    """Plain tensor product.  The map is trilinear, so every gradient is again a tensor product:
-    d/dx1 and (for ``uvw``) d/dx2 run the forward kernels on transposed plans; d/dw and d/dx2 of
-    ``uvu`` have their own edge-parallel kernel."""
+# ---------------------------------------------------------------------------------------------------- autograd
+# The product is trilinear, so F(x1, x2, w, g) = <g, tp(x1, x2, w)> is linear in each of its four slots.  The product
+# itself is dF/dg and its three gradients are dF/dx1, dF/dx2, dF/dw, each a function of the other three slots; and the
+# derivative of any of these four maps with respect to one of ITS arguments, contracted with a cotangent c, is again
+# one of the four maps, evaluated with c in the slot that the differentiated map stands for.  The family is closed, so
+# one autograd Function per family, whose backward applies the same Function, gives derivatives of every order (the
+# reference gets them by differentiating its einsums, e3nn/o3/_tensor_product/_codegen.py:148-187; a loss on forces
+# needs the second).  Every member runs on a kernel that exists for the first-order pass: the forward kernel, the
+# forward kernel on a transposed plan, or one of the weight / second-input gradient kernels.
+_X1, _X2, _W, _OUT = 0, 1, 2, 3
+
+
+def _tp_gradients(tp, x1, x2, w, g, need1, need2, needw):
+    """``(d/dx1, d/dx2, d/dw)`` of ``<g, tp(x1, x2, w)>``, None where not needed: d/dx1 and (for ``uvw``) d/dx2 run the
+    forward kernels on transposed plans; d/dw and d/dx2 of ``uvu`` have their own edge-parallel kernel, which writes
+    both in one pass when both are wanted.  An argument that no wanted gradient depends on (``x1`` for d/dx1, ``x2``
+    for d/dx2, ``w`` for d/dw) may be None."""
+    g = g.contiguous()
+    dt, Z = g.dtype, g.shape[0]
+    g1 = g2 = gw = None
+    mode = tp._live_mode()
+    needw = needw and tp.weight_numel > 0
+    if mode == "uvu":
+        if need1:
+            g1 = tp._grad_plan("x1", dt).forward(g, x2, w)
+        if need2 or needw:
+            if tp.shared_weights and needw and dt != torch.float32:
+                # the sum over the batch is taken by fp32 atomics: the fp32 kernel on widened copies
+                gw, g2 = tp._plan(torch.float32).backward_w_x2(
+                    x1.float(), x2.float(), None if w is None else w.float(), g.float(), None, None, True, need2, Z
+                )
+                gw = gw.to(dt)
+                g2 = None if g2 is None else g2.to(dt)
+            else:
+                gw, g2 = tp._plan(dt).backward_w_x2(x1, x2, w, g, None, None, needw, need2, Z)
+    elif mode == "uvw":
+        if needw:
+            if dt != torch.float32:
+                # the weight-gradient kernels read fp32 rows: widened copies of the operands, result in storage type
+                gw = tp._plan(torch.float32).backward_w_uvw(x1.float(), x2.float(), g.float(), tp.shared_weights).to(dt)
+            else:
+                gw = tp._plan(dt).backward_w_uvw(x1, x2, g, tp.shared_weights)
+        if need1:
+            g1 = tp._grad_plan("x1", dt).forward(g, x2, _permuted_weights(tp, w, (2, 1, 0)))
+        if need2:
+            g2 = tp._grad_plan("x2", dt).forward(x1, g, _permuted_weights(tp, w, (0, 2, 1)))
+    elif mode == "general":
+        raise AssertionError("general connection modes are differentiated through TensorProduct._dense_equivalent")
+    else:
+        g1 = g.new_zeros(Z, tp._in1_dim) if need1 else None
+        g2 = g.new_zeros(Z, tp._in2_dim) if need2 else None
+    return g1, g2, gw
+
+
+def _slot_backward(fn, slot, saved, cot, needs, *context):
+    """Backward of one member of a closed family (see above): the gradient with respect to the argument that fills
+    slot ``t`` is the member ``t`` evaluated with the cotangent in slot ``slot``.  Differentiable itself."""
+    others = [t for t in range(4) if t != slot]
+    full = {slot: cot, **dict(zip(others, saved))}
+    grads = []
+    for t, need in zip(others, needs):
+        grads.append(fn.apply(t, *context, *[full[u] for u in range(4) if u != t]) if need else None)
+    return grads
+
+
+class _TpSlot(torch.autograd.Function):
+    """Member ``slot`` of the family of the plain product: ``_OUT`` is ``tp(x1, x2, w)``, ``_X1`` / ``_X2`` / ``_W`` its
+    gradients; the three tensor arguments are the other slots in the order (x1, x2, w, g)."""
 
     @staticmethod
-    def forward(ctx, x1, x2, w, tp):
-        ctx.tp = tp
-        ctx.save_for_backward(x1, x2, w)
-        return tp._plan(x1.dtype).forward(x1, x2, w)
+    def forward(ctx, slot, tp, a, b, c):
+        ctx.slot, ctx.tp = slot, tp
+        ctx.save_for_backward(a, b, c)
+        if slot == _OUT:
+            return tp._plan(a.dtype).forward(a, b, c)
+        x1, x2, w, g = [a, b, c][:slot] + [None] + [a, b, c][slot:]
+        out = _tp_gradients(tp, x1, x2, w, g, slot == _X1, slot == _X2, slot == _W)[slot]
+        if out is None:  # the gradient of weights that do not exist
+            shape = (0,) if tp.shared_weights else (g.shape[0], 0)
+            out = g.new_zeros(shape)
+        return out
 
     @staticmethod
-    @once_differentiable
-    def backward(ctx, g):
-        tp = ctx.tp
-        x1, x2, w = ctx.saved_tensors
-        g = g.contiguous()
-        need1, need2, needw = ctx.needs_input_grad[:3]
-        g1 = g2 = gw = None
-        mode = tp._live_mode()
-        if mode == "uvu":
-            if need1:
-                g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, w)
-            if need2 or (needw and tp.weight_numel):
-                if tp.shared_weights and needw and tp.weight_numel and x1.dtype != torch.float32:
-                    # the sum over the batch is taken by fp32 atomics: the fp32 kernel on widened copies
-                    gw, g2 = tp._plan(torch.float32).backward_w_x2(
-                        x1.float(), x2.float(), w.float(), g.float(), None, None, True, need2, x1.shape[0]
-                    )
-                    gw = gw.to(x1.dtype)
-                    g2 = None if g2 is None else g2.to(x1.dtype)
-                else:
-                    gw, g2 = tp._plan(x1.dtype).backward_w_x2(x1, x2, w, g, None, None, needw and tp.weight_numel > 0, need2, x1.shape[0])
-        elif mode == "uvw":
-            if needw and tp.weight_numel:
-                if x1.dtype != torch.float32:
-                    # the weight-gradient kernels read fp32 rows: widened copies of the operands, result in storage type
-                    gw = tp._plan(torch.float32).backward_w_uvw(x1.float(), x2.float(), g.float(), tp.shared_weights).to(x1.dtype)
-                else:
-                    gw = tp._plan(x1.dtype).backward_w_uvw(x1, x2, g, tp.shared_weights)
-            if need1:
-                g1 = tp._grad_plan("x1", x1.dtype).forward(g, x2, _permuted_weights(tp, w, (2, 1, 0)))
-            if need2:
-                g2 = tp._grad_plan("x2", x1.dtype).forward(x1, g, _permuted_weights(tp, w, (0, 2, 1)))
-        elif mode == "general":
-            raise AssertionError("general connection modes are differentiated through TensorProduct._dense_equivalent")
-        else:
-            g1, g2 = torch.zeros_like(x1), torch.zeros_like(x2)
-            gw = torch.zeros_like(w) if needw else None
-        return g1, g2, gw, None
+    def backward(ctx, cot):
+        saved, needs = ctx.saved_tensors, ctx.needs_input_grad[2:5]
+        if ctx.slot == _OUT and not torch.is_grad_enabled():
+            # the first-order pass: kernels that write several gradients at once
+            g1, g2, gw = _tp_gradients(ctx.tp, *saved, cot, *needs)
+            if needs[2] and gw is None:
+                gw = torch.zeros_like(saved[2])
+            return None, None, g1, g2, gw
+        return (None, None, *_slot_backward(_TpSlot, ctx.slot, saved, cot.contiguous(), needs, ctx.tp))
 
 
-class _GatherScatterFn(torch.autograd.Function):
-    """``scatter(tp(node_x[src], edge_attr, w), dst)``; d/dnode_x is the same fused kernel on the transposed
-    plan with the roles of source and destination exchanged."""
+class _TensorProductFn:
+    """``tp(x1, x2, w)`` under autograd (every order of differentiation)."""
 
     @staticmethod
-    def forward(ctx, node_x, edge_attr, w, tp, edges):
-        ctx.tp, ctx.edges = tp, edges
-        ctx.save_for_backward(node_x, edge_attr, w)
-        return tp._plan(node_x.dtype).gather_scatter(node_x, edge_attr, w, edges.edge_src, edges, node_x.shape[0])
-
-    @staticmethod
-    @once_differentiable
-    def backward(ctx, g):
-        node_x, edge_attr, w = ctx.saved_tensors
-        return _message_gradients(ctx.tp, ctx.edges, node_x, edge_attr, w, g.contiguous(), *ctx.needs_input_grad[:3]) + (None, None)
+    def apply(x1, x2, w, tp):
+        return _TpSlot.apply(_OUT, tp, x1, x2, w)
 
 
 def _message_gradients(tp, edges, node_x, edge_attr, w, g, need1, need2, needw):
-    """``(d/dnode_x, d/dedge_attr, d/dw)`` of ``<g, scatter(tp(node_x[src], edge_attr, w), dst)>``; None where not needed."""
+    """``(d/dnode_x, d/dedge_attr, d/dw)`` of ``<g, scatter(tp(node_x[src], edge_attr, w), dst)>``; None where not needed.
+    d/dnode_x is the fused kernel on the transposed plan with the roles of source and destination exchanged.  An
+    argument that no wanted gradient depends on may be None."""
+    g = g.contiguous()
+    dt = g.dtype
     g1 = g2 = gw = None
-    if need1 and needw and tp.weight_numel and node_x.dtype == torch.float32:
+    needw = needw and tp.weight_numel > 0
+    if need1 and needw and dt == torch.float32:
         # every gradient from one pass over the weights and one gather of g per edge
-        res = tp._grad_plan("x1", node_x.dtype).gather_scatter_grad_w(
+        res = tp._grad_plan("x1", dt).gather_scatter_grad_w(
             g, edge_attr, w, node_x, edges.edge_dst, edges.transposed(), need2 and edge_attr.shape[1] > 0
         )
         if res is not None:
             return res[0], (res[2] if need2 else None), res[1]
     if need1:
         rev = edges.transposed()
-        g1 = tp._grad_plan("x1", node_x.dtype).gather_scatter(g, edge_attr, w, edges.edge_dst, rev, g.shape[0])
-    if need2 or (needw and tp.weight_numel):
-        gw, g2 = tp._plan(node_x.dtype).backward_w_x2(
-            node_x, edge_attr, w, g, edges.edge_src, edges.edge_dst, needw and tp.weight_numel > 0, need2, edges.num_edges
-        )
+        g1 = tp._grad_plan("x1", dt).gather_scatter(g, edge_attr, w, edges.edge_dst, rev, g.shape[0])
+    if need2 or needw:
+        gw, g2 = tp._plan(dt).backward_w_x2(node_x, edge_attr, w, g, edges.edge_src, edges.edge_dst, needw, need2, edges.num_edges)
     return g1, g2, gw
+
+
+class _MessageSlot(torch.autograd.Function):
+    """Member ``slot`` of the family of the message step ``scatter(tp(node_x[src], edge_attr, w), dst)``: slots
+    (node_x [N_src, dim1], edge_attr [E, dim2], w [E, weight_numel], g [N, dim_out])."""
+
+    @staticmethod
+    def forward(ctx, slot, tp, edges, a, b, c):
+        ctx.slot, ctx.tp, ctx.edges = slot, tp, edges
+        ctx.save_for_backward(a, b, c)
+        if slot == _OUT:
+            return tp._plan(a.dtype).gather_scatter(a, b, c, edges.edge_src, edges, a.shape[0])
+        x, attr, w, g = [a, b, c][:slot] + [None] + [a, b, c][slot:]
+        out = _message_gradients(tp, edges, x, attr, w, g, slot == _X1, slot == _X2, slot == _W)[slot]
+        return g.new_zeros(edges.num_edges, 0) if out is None else out  # (the gradient of weights that do not exist)
+
+    @staticmethod
+    def backward(ctx, cot):
+        saved, needs = ctx.saved_tensors, ctx.needs_input_grad[3:6]
+        if ctx.slot == _OUT and not torch.is_grad_enabled():
+            g1, g2, gw = _message_gradients(ctx.tp, ctx.edges, *saved, cot, *needs)
+            if needs[2] and gw is None:
+                gw = torch.zeros_like(saved[2])
+            return None, None, None, g1, g2, gw
+        return (None, None, None, *_slot_backward(_MessageSlot, ctx.slot, saved, cot.contiguous(), needs, ctx.tp, ctx.edges))
+
+
+class _GatherScatterFn:
+    """``scatter(tp(node_x[src], edge_attr, w), dst)`` under autograd (every order of differentiation)."""
+
+    @staticmethod
+    def apply(node_x, edge_attr, w, tp, edges):
+        return _MessageSlot.apply(_OUT, tp, edges, node_x, edge_attr, w)
 
 
 class _GatherScatterShFn(torch.autograd.Function):
     """``_GatherScatterFn`` on ``edge_attr = spherical_harmonics(0 .. lmax, edge_vec)``, the harmonics formed inside the
     kernel.  The backward pass evaluates them once with the stand-alone kernel (they are 3 % of the per-edge bytes)
-    and runs the message gradients on them; the gradient of the vectors goes through the harmonics' own backward."""
+    and runs the message gradients on them; the gradient of the vectors goes through the harmonics' own backward.
+    Under ``create_graph`` the backward pass is the differentiable composition of the two families."""
 
     @staticmethod
     def forward(ctx, node_x, edge_vec, w, tp, edges, normalize, normalization):
@@ -364,18 +437,21 @@ class _GatherScatterShFn(torch.autograd.Function):
         return out
 
     @staticmethod
-    @once_differentiable
     def backward(ctx, g):
-        from .spherical_harmonics import _SphericalHarmonicsFn
+        from .spherical_harmonics import _sh_backward, _sh_forward
 
         node_x, edge_vec, w = ctx.saved_tensors
         need1, need_vec, needw = ctx.needs_input_grad[:3]
-        ls = tuple(range(len(ctx.tp.irreps_in2)))
-        with torch.enable_grad():
-            vec = edge_vec.detach().requires_grad_(need_vec)
-            attr = _SphericalHarmonicsFn.apply(vec, ls, *ctx.sh)
-        g1, g2, gw = _message_gradients(ctx.tp, ctx.edges, node_x, attr.detach().to(node_x.dtype), w, g.contiguous(), need1, need_vec, needw)
-        gvec = torch.autograd.grad(attr, vec, g2.to(attr.dtype))[0] if need_vec else None
+        tp, edges = ctx.tp, ctx.edges
+        ls = tuple(range(len(tp.irreps_in2)))
+        if torch.is_grad_enabled():
+            attr = _sh_forward(edge_vec, ls, *ctx.sh).to(node_x.dtype)  # differentiable in edge_vec
+            g1, g2, gw = _slot_backward(_MessageSlot, _OUT, (node_x, attr, w), g.contiguous(), (need1, need_vec, needw), tp, edges)
+            gvec = _sh_backward(edge_vec, g2.to(edge_vec.dtype), ls, *ctx.sh) if need_vec else None
+            return g1, gvec, gw, None, None, None, None
+        attr = _sh_forward(edge_vec, ls, *ctx.sh).to(node_x.dtype)
+        g1, g2, gw = _message_gradients(tp, edges, node_x, attr, w, g, need1, need_vec, needw)
+        gvec = _sh_backward(edge_vec, g2.to(edge_vec.dtype), ls, *ctx.sh) if need_vec else None
         return g1, gvec, gw, None, None, None, None
 
 

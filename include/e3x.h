@@ -274,7 +274,8 @@ int e3x_tp_gather_scatter_sh(e3x_plan* plan, const void* node_x, const float* ed
  * e3nn/o3/_tensor_product/_codegen.py:166-187.  The gradient with respect to the first input is the
  * forward entry point applied to a transposed plan (inputs grad_out and x2, output irreps_in1, same
  * weights) with source and destination exchanged; no separate entry point is needed for it.
- * Only for all-`uvu` plans; bf16 storage only for per-sample weights and plans of a single kernel. */
+ * Only for all-`uvu` plans; bf16 storage only for per-sample weights and plans of a single kernel.
+ * x2 may be NULL when grad_w is (only the weight gradient reads it), per-sample w when grad_x2 is. */
 int e3x_tp_backward_w_x2(e3x_plan* plan, const void* x1, const void* x2, const void* w, const void* grad_out,
                          const void* src, const void* dst, int idx_bits, void* grad_w, void* grad_x2, int64_t E,
                          int64_t num_src_nodes, int64_t num_out_nodes, void* stream);
@@ -328,6 +329,17 @@ int e3x_sh_forward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t n
 int e3x_sh_backward(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization, const void* xyz,
                     const void* grad_out, void* grad_xyz, int64_t n, int32_t dtype, void* stream);
 
+/* The derivative of e3x_sh_backward, for training on quantities that are themselves gradients (forces): with
+ * phi(x) = <grad_out, Y(x)>, whose gradient e3x_sh_backward returns, and a cotangent cot_xyz[n, 3] on that gradient,
+ *   grad_grad_out[n, n_out] = d<cot, grad phi>/d grad_out = the directional derivative of Y along cot,
+ *   grad_xyz[n, 3]          = d<cot, grad phi>/d xyz      = the Hessian of phi applied to cot
+ * (the normalisation of the vectors is part of the differentiated function).  The reference obtains both by
+ * differentiating its polynomial chain twice (e3nn/o3/_spherical_harmonics.py:193-249).  Implemented for the l lists
+ * 0 .. lmax <= 3 (the closed forms); E3X_ERR_INVALID for any other list. */
+int e3x_sh_backward2(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t normalization, const void* xyz,
+                     const void* grad_out, const void* cot_xyz, void* grad_grad_out, void* grad_xyz, int64_t n,
+                     int32_t dtype, void* stream);
+
 /* Gated non-linearity on rows x[Z, in_dim] -> out[Z, out_dim] (fp32), at most 16 blocks of each kind; columns of `out`
  * that no block covers become 0.  Replaces nn.Gate.forward (e3nn/nn/_gate.py:121-144: Extract, Activation,
  * ElementwiseTensorProduct, cat) and, with n_gates = 0, nn.Activation.forward (e3nn/nn/_activation.py:78-104);
@@ -338,6 +350,13 @@ int e3x_gate_forward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_b
 int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_block* gates, int32_t n_gates, const void* x,
                       const void* grad_out, void* grad_x, int64_t Z, int64_t in_dim, int64_t out_dim, int32_t dtype,
                       void* stream);
+/* The derivative of e3x_gate_backward: for a cotangent cot_x[Z, in_dim] on its result,
+ * grad_grad_out[Z, out_dim] = d<cot_x, grad_x>/d grad_out and grad_x[Z, in_dim] = d<cot_x, grad_x>/dx (second
+ * derivatives of the activations; 0 for abs and relu away from 0).  The reference differentiates
+ * e3nn/nn/_gate.py:121-144 and e3nn/nn/_activation.py:78-104 twice by autograd. */
+int e3x_gate_backward2(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_block* gates, int32_t n_gates,
+                       const void* x, const void* grad_out, const void* cot_x, void* grad_grad_out, void* grad_x,
+                       int64_t Z, int64_t in_dim, int64_t out_dim, int32_t dtype, void* stream);
 
 /* Fully-connected network of scalars hs[0] -> hs[1] -> ... -> hs[n_hs-1] in ONE kernel (fp32, matrix cores):
  *   layer l:  x <- act(x @ W_l / sqrt(hs[l] var_in)) * act_cst * sqrt(var_out)      (with activation)

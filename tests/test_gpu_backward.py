@@ -89,15 +89,6 @@ def test_fused_message_gradients(maker, N, E, idx):
     assert torch.equal(a5.grad, a4.grad) and torch.equal(c5.grad, c4.grad)
 
 
-def test_second_derivatives_raise_instead_of_dropping_terms():
-    # the backward passes are kernels on fresh buffers (no graph): double backward must fail loudly
-    tp = ks.cfg1().to(DEV)
-    x1, x2 = seeded(8, 64).to(DEV).requires_grad_(True), seeded(8, 9).to(DEV)
-    (g,) = torch.autograd.grad(tp(x1, x2).square().sum(), x1, create_graph=True)
-    with pytest.raises(RuntimeError, match="once_differentiable"):
-        g.sum().backward()
-
-
 @pytest.mark.parametrize("maker,Z", [(lambda: ks.golden_tp("fctp_small_cfg5_like"), 6), (ks.cfg1, 50), (ks.mfma_small, 70),
                                      (lambda: ks.golden_tp("fctp_per_sample_weights"), 5), (ks.node_fctp, 90), (ks.radial_layer, 77), (ks.node_wide_out, 45), (ks.node_narrow, 40)])  # fmt: skip
 def test_uvw_input_gradients(maker, Z):
