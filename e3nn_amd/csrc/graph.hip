@@ -30,6 +30,9 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices];
 std::mutex g_scratch_mutex;
+// one call at a time per device: the callers of a device share its array, and a call ends with the stream synchronised
+// (the range-check read-back), so holding the lock from the first launch to that point makes host threads take turns
+std::mutex g_scratch_busy[kMaxDevices];
 
 // device address of `scratch` on the current device, looked up once per device
 int static_scratch(void** out) {
@@ -246,11 +249,14 @@ extern "C" int e3x_csr_build_static(const void* dst, int idx_bits, int64_t E, in
              "(use e3x_csr_build with a workspace)", (long long)E, need, kStaticScratchBytes);
     return e3x::fail(E3X_ERR_INVALID, msg);
   }
+  if (E == 0) return e3x_csr_build(dst, idx_bits, E, num_nodes, rowptr, perm, nullptr, kStaticScratchBytes, stream);  // touches no scratch
   void* ws = nullptr;
-  if (E > 0) {  // E == 0 touches no scratch
-    const int rc = static_scratch(&ws);
-    if (rc != E3X_OK) return rc;
-  }
+  const int rc = static_scratch(&ws);
+  if (rc != E3X_OK) return rc;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return e3x::fail(E3X_ERR_HIP, "e3x_csr_build_static: no current HIP device");
+  std::lock_guard<std::mutex> busy(g_scratch_busy[dev]);
   return e3x_csr_build(dst, idx_bits, E, num_nodes, rowptr, perm, ws, kStaticScratchBytes, stream);
 }
 

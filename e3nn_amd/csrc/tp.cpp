@@ -1348,10 +1348,11 @@ extern "C" int e3x_tp_gather_scatter_ws(e3x_plan* P, const void* node_x, const v
   long long n_rows = num_out_nodes, n_src = num_src_nodes;
   void* args[] = {(void*)&node_x, (void*)&edge_attr, (void*)&w,         (void*)&out,    (void*)&src,  (void*)&idx64,
                   (void*)&rowptr, (void*)&perm,      (void*)&row_order, (void*)&n_rows, (void*)&n_src};
-  // the matrix-core message kernel: needs the workspace for the node table in operand order, 8-byte aligned weight
-  // rows and a 16-byte aligned workspace; without them the vector-ALU kernels below run
+  // the matrix-core message kernel: needs the workspace for the node table in operand order, and 16-byte aligned
+  // node table, weights, edge attributes, output and workspace (their rows are whole 16-byte pieces by construction of
+  // the kernel, and it reads and writes them as such); without them the vector-ALU kernels below run
   if (P->msg_mfma && E > 0 && workspace && workspace_bytes >= e3x_tp_gather_scatter_workspace_bytes(P, num_src_nodes) &&
-      !(((uintptr_t)w | (uintptr_t)edge_attr) & 15) && !((uintptr_t)workspace & 15)) {
+      !(((uintptr_t)w | (uintptr_t)edge_attr | (uintptr_t)node_x | (uintptr_t)out | (uintptr_t)workspace) & 15)) {
     SubKernel* K = P->msg_mfma.get();
     {
       const long long pblocks = n_src;  // a workgroup per node

@@ -153,14 +153,17 @@ int e3x_tp_forward_ws(e3x_plan* plan, const void* x1, const void* x2, const void
 size_t e3x_csr_workspace_bytes(int64_t E, int64_t num_nodes);
 int e3x_csr_build(const void* dst, int idx_bits, int64_t E, int64_t num_nodes, int32_t* rowptr, int32_t* perm,
                   void* workspace, size_t workspace_bytes, void* stream);
-/* e3x_csr_build for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
- * capture set-up, tight serving loops that rebuild the neighbour list every few steps, harnesses that forbid
- * hipMalloc).  No counterpart in the reference.  The sort buffers live in a file-scope device array of
+/* e3x_csr_build for callers that cannot allocate device memory or hand over a workspace (tight serving loops that
+ * rebuild the neighbour list every few steps, harnesses that forbid hipMalloc, set-up code that runs before a HIP
+ * graph is captured).  Like e3x_csr_build it copies the range-check flag back and synchronises the stream before it
+ * returns, so it must not be issued while the stream is capturing.  No counterpart in the reference.  The sort buffers live in a file-scope device array of
  * e3x_csr_static_scratch_bytes() = 64 MiB that every GPU the library runs on holds until the process ends; its
  * address is looked up once per device, on the first call there.  The call allocates and frees nothing.  Limit: the
  * buffers of e3x_csr_workspace_bytes(E, num_nodes) must fit the array (2 097 152 edges always do); larger edge lists
- * return E3X_ERR_INVALID.  All calls on one GPU share the array: calls that overlap there (two host threads or two
- * streams) race, consecutive calls on one stream do not.  Results are bit-identical to e3x_csr_build. */
+ * return E3X_ERR_INVALID.  All calls on one GPU share the array; the library makes the host threads of a process take
+ * turns (a per-device lock held from the first launch to the final synchronisation), so only callers outside its
+ * reach -- another process's library has an array of its own; the same array used through a stale pointer -- could
+ * overlap.  Results are bit-identical to e3x_csr_build. */
 size_t e3x_csr_static_scratch_bytes(void);
 int e3x_csr_build_static(const void* dst, int idx_bits, int64_t E, int64_t num_nodes, int32_t* rowptr, int32_t* perm,
                          void* stream);

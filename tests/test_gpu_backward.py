@@ -45,7 +45,10 @@ def test_uvu_plain_gradients(maker, Z):
 
 
 @pytest.mark.parametrize("maker,N,E,idx", [(lambda: ks.cfg3(True), 120, 3000, torch.int64), (lambda: ks.cfg3(False), 50, 900, torch.int32),
-                                           (lambda: ks.cfg4("A"), 25, 300, torch.int32)])  # fmt: skip
+                                           (lambda: ks.cfg4("A"), 25, 300, torch.int32),
+                                           # multiplicities that leave lane groups partly filled (80, 24, 5): every
+                                           # weight-gradient column must still be written (the buffer is not zero-filled)
+                                           (ks.odd_mul, 40, 600, torch.int32)])  # fmt: skip
 def test_fused_message_gradients(maker, N, E, idx):
     tp = maker()
     spec = oracle_spec(tp)

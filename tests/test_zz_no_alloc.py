@@ -71,3 +71,40 @@ def test_static_scratch_rejects_edge_lists_beyond_its_buffers():
     rc = L.e3x_csr_build_static(_lib.ptr(one), 32, too_many, 8, _lib.ptr(one), _lib.ptr(one), _lib.stream_ptr(DEV))
     assert rc == _lib.ERR_INVALID
     assert b"static buffer" in L.e3x_last_error()
+
+
+def test_static_scratch_host_threads_take_turns():
+    # two host threads on streams of their own share the device's one array; the library serialises them (a per-device
+    # lock from the first launch to the final synchronisation), so both get the right answer
+    import threading
+
+    g = torch.Generator().manual_seed(9)
+    jobs = [(150_000, 20_000), (90_000, 7_000)]
+    dsts = [torch.randint(0, N, (E,), generator=g).to(DEV) for E, N in jobs]
+    results = [None, None]
+
+    def work(i):
+        L = _lib.lib()
+        E, N = jobs[i]
+        with torch.cuda.device(DEV):
+            stream = torch.cuda.Stream(device=DEV)
+            rowptr = torch.empty(N + 1, dtype=torch.int32, device=DEV)
+            perm = torch.empty(E, dtype=torch.int32, device=DEV)
+            torch.cuda.synchronize()
+            for _ in range(5):
+                rc = L.e3x_csr_build_static(_lib.ptr(dsts[i]), 64, E, N, _lib.ptr(rowptr), _lib.ptr(perm), _lib.c_void_p(stream.cuda_stream))
+                if rc != 0:
+                    results[i] = rc
+                    return
+            stream.synchronize()
+            results[i] = (rowptr.cpu().numpy(), perm.cpu().numpy())
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for i, (E, N) in enumerate(jobs):
+        assert isinstance(results[i], tuple), results[i]
+        rp, pm = _reference(dsts[i], N)
+        assert np.array_equal(results[i][0], rp) and np.array_equal(results[i][1], pm)
