@@ -316,7 +316,7 @@ def bench_uvw(args, dev, dtype=torch.float32):
                         "unit": "TFLOP/s", "frac": f_min / (ms * 1e-3) / 1e12 / peak}, "flops_per_launch": f_min}  # fmt: skip
     if dtype == torch.float32:
         out["roofline"].update(split_operand_fractions(arithmetic, f_min, ms))
-        if "split" in arithmetic:  # the same product on the fp32 matrix instruction, as a plan of its own
+        if "split" in arithmetic and not args.no_instruction_variants:  # the same product on the fp32 matrix instruction, as a plan of its own
             out["ms_fp32_instruction"] = with_env("E3X_UVW_SPLIT", "0", lambda: time_fresh_plan(ks.cfg5, tp.weight, x1, x2))
             out["roofline"]["frac_on_fp32_instruction"] = f_min / (out["ms_fp32_instruction"] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS
     return out
@@ -543,7 +543,7 @@ def bench_uvw_backward(args, dev):
             "unit": "TFLOP/s", "frac": f_min / (ms_dw * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}  # fmt: skip
     roof.update(split_operand_fractions(arithmetic, f_min, ms_dw))
     out = {"rows": Z, "ms_forward_backward": ms, "ms_weight_gradient": ms_dw, "roofline_weight_gradient": roof}
-    if "split" in arithmetic:
+    if "split" in arithmetic and not args.no_instruction_variants:
 
         def fp32_instruction():
             tp2 = ks.cfg5().to(dev)
@@ -565,6 +565,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--locality-variants", action="store_true", help="time the headline graph with sorted edges / Morton node ids also when --only is given")
     ap.add_argument("--no-headline", action="store_true", help="profiling aid: run only the sections of --only (those that do not build on the headline graph) and print their results, so that a profile holds the launches of one configuration only")
+    ap.add_argument("--no-instruction-variants", action="store_true", help="profiling aid: do not time config 5 on the fp32 matrix instruction beside the default kernels, so that a profile holds one code object per kernel name")
     ap.add_argument("--only", default="", help="comma list of extra sections to run: copy,sh,mace,mace_b,mace_bf16,nequip40,uvw,uvw_bf16,conv,radial,nequip_bwd,uvw_bwd (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:

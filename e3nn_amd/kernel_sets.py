@@ -2,11 +2,9 @@
 
 ``cfg1`` ... ``cfg5`` are the five benchmark configurations; the other makers are the shapes each kernel family is
 exercised on (tile edges, ragged channel counts, every connection mode).  ``prebuild`` compiles all of their kernels
-into the in-tree cache, so that nothing has to be compiled on a GPU box.  Instruction sets described by data files
-(JSON written from the reference: instruction tables plus constructor arguments) join the list after
-``use_golden(directory)``.
+into the in-tree cache, so that nothing has to be compiled on a GPU box; callers may hand it further products and
+modules to build beside these (the test suite adds the instruction sets of its fixtures).
 """
-import json
 import os
 
 import torch
@@ -14,55 +12,11 @@ import torch
 from . import o3
 from .nn.message import message_tensor_product
 
-GOLDEN = None  # directory with tp_cases.json / nn_cases.json (+ .npz); see use_golden
-
-
-def use_golden(directory):
-    """Adds the instruction sets of ``directory``/tp_cases.json and the modules of nn_cases.json to the build list."""
-    global GOLDEN
-    GOLDEN = directory if directory and os.path.isdir(directory) else None
-    return GOLDEN
-
-
 SH2 = str(o3.Irreps.spherical_harmonics(2))
 SH3 = str(o3.Irreps.spherical_harmonics(3))
 
-GOLDEN_GPU_CASES = [
-    "fctp_cfg1", "fctp_small_cfg5_like", "fctp_per_sample_weights", "fctp_norm_path",
-    "uvu_merged_cfg3_like_mul4", "uvu_builder_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2",
-    "uvu_builderB_cfg4_like_mul2", "uvu_shared_v2", "uvu_mixed_weightless", "empty_path_and_missing_output",
-    "modes_uuu_uvuv_uuw_uvv", "modes_triangular", "conv_small",
-]  # fmt: skip
-
-
-def golden_meta():
-    if GOLDEN is None:
-        raise RuntimeError("no golden directory: call use_golden(path) first")
-    with open(os.path.join(GOLDEN, "tp_cases.json")) as f:
-        return json.load(f)
-
-
-# backward pass in bf16 storage: a matrix-core uvw set, shared uvu weights, per-edge uvu weights
-BACKWARD_BF16_CASES = ["mfma_small", "uvu_shared_v2", "cfg3_merged"]
-
-
-def tp_from_meta(m, **extra):
-    upw = m.get("user_path_weights", [1.0] * len(m["instructions"]))
-    ins = [tuple(t[:5]) + (pw,) for t, pw in zip(m["instructions"], upw)]
-    kw = {}
-    if m.get("irrep_normalization"):
-        kw = dict(irrep_normalization=m["irrep_normalization"], path_normalization=m["path_normalization"])
-    return o3.TensorProduct(
-        m["irreps_in1"], m["irreps_in2"], m["irreps_out"], ins,
-        internal_weights=m["internal_weights"], shared_weights=m["shared_weights"], **kw, **extra,
-    )  # fmt: skip
-
-
-def golden_tp(name, meta=None, **extra):
-    m = dict((meta or golden_meta())[name])
-    if name == "fctp_norm_path":
-        m.update(irrep_normalization="norm", path_normalization="path")
-    return tp_from_meta(m, **extra)
+# backward pass in bf16 storage as well (callers of prebuild may add names): a matrix-core uvw set, per-edge uvu weights
+BACKWARD_BF16_CASES = ["mfma_small", "cfg3_merged"]
 
 
 def cfg1():
@@ -184,11 +138,7 @@ def odd_mul():
 
 def all_tensor_products():
     """(name, TensorProduct, dtypes) for everything that must be in the kernel cache."""
-    out = []
-    if GOLDEN is not None:
-        meta = golden_meta()
-        out = [(n, golden_tp(n, meta), (torch.float32,)) for n in GOLDEN_GPU_CASES]
-    out += [
+    out = [
         ("cfg1", cfg1(), (torch.float32,)),
         ("cfg3_merged", cfg3(True), (torch.float32, torch.bfloat16)),
         ("cfg3_builder", cfg3(False), (torch.float32,)),
@@ -217,17 +167,9 @@ def all_tensor_products():
 
 
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
-BACKWARD_CASES = ["uvu_merged_cfg3_like_mul4", "uvu_builderA_cfg4_like_mul2", "uvu_shared_v2", "fctp_small_cfg5_like",
-                  "fctp_per_sample_weights", "cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "mfma_full_tiles", "outer_split", "node_fctp", "node_block", "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul",
-                  "unaligned_mfma", "unaligned_offsets", "mixed_modes", "scalar_exact", "modes_uuu_uvuv_uuw_uvv", "modes_triangular"]  # fmt: skip
-
-
-def nn_golden():
-    import numpy as np
-
-    with open(os.path.join(GOLDEN, "nn_cases.json")) as f:
-        meta = json.load(f)
-    return np.load(os.path.join(GOLDEN, "nn_cases.npz")), meta
+BACKWARD_CASES = ["cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "mfma_full_tiles", "outer_split", "node_fctp", "node_block",
+                  "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul", "unaligned_mfma", "unaligned_offsets",
+                  "mixed_modes", "scalar_exact"]  # fmt: skip
 
 
 def linear_channels(norm="element"):
@@ -238,24 +180,12 @@ def nn_modules():
     """(name, module) for the node-wise blocks the GPU tests run; every TensorProduct inside needs its kernels."""
     from e3nn_amd import nn
 
-    out = []
-    meta = None
-    if GOLDEN is not None:
-        _, meta = nn_golden()
-        for name in ("linear_mixed", "linear_path_norm", "linear_bias"):
-            m = meta[name]
-            out.append((name, o3.Linear(m["irreps_in"], m["irreps_out"], **m["kwargs"])))
-    out.append(("linear_wide", o3.Linear("128x0e+128x1o+64x2e", "128x0e+64x1o+32x1o")))
+    out = [("linear_wide", o3.Linear("128x0e+128x1o+64x2e", "128x0e+64x1o+32x1o"))]
     for norm in ("element", "path"):  # input and output channels: the product on f_in / f_out copies of every irrep
         out.append((f"linear_channels_{norm}", linear_channels(norm)))
-    if meta is not None:
-        out.append(("fc_golden", nn.FullyConnectedNet(meta["fc"]["hs"], torch.nn.functional.silu)))
     out.append(("fc_radial", nn.FullyConnectedNet([8, 64, 352], torch.nn.functional.silu)))
     # a hidden layer too wide for the one-kernel path and its one-layer specialisations: tensor-product kernels throughout
     out.append(("fc_wide_hidden", nn.FullyConnectedNet([8, 512, 16], torch.nn.functional.silu)))
-    if meta is not None:
-        a = meta["conv"]["args"]
-        out.append(("conv_golden", nn.Convolution(a[0], a[1], a[2], a[3], a[4], a[5])))
     out.append(("conv_wide", conv_wide()))
     return out
 
@@ -308,8 +238,9 @@ SH_MESSAGE_CASES = [("cfg3_merged", True, "component"), ("cfg3_merged", False, "
                     ("cfg4_A", True, "component"), ("odd_mul", True, "integral")]  # fmt: skip
 
 
-def prebuild(verbose=True, workers=6):
-    """Builds every kernel the tests and the benchmark use.  Plan creation spends its time in the HIP compiler (a child
+def prebuild(verbose=True, workers=6, extra_tensor_products=(), extra_modules=(), backward_cases=(), backward_bf16_cases=()):
+    """Builds every kernel of this module's lists, plus ``extra_tensor_products`` (``(name, TensorProduct, dtypes)``;
+    those named in ``backward_cases`` with their backward kernels) and ``extra_modules`` (``(name, module)``).  Plan creation spends its time in the HIP compiler (a child
     process, the calling thread waits with the GIL released), so a few threads build several kernels at once."""
     from concurrent.futures import ThreadPoolExecutor
 
@@ -318,7 +249,10 @@ def prebuild(verbose=True, workers=6):
     from . import _lib
 
     jobs = []
-    for name, mod in nn_modules() + [(f"fused_fc{i}", net) for i, net in enumerate(fused_fc_nets())]:
+    modules = nn_modules() + list(extra_modules)
+    products = all_tensor_products() + list(extra_tensor_products)
+    backward = set(BACKWARD_CASES) | set(backward_cases)
+    for name, mod in modules + [(f"fused_fc{i}", net) for i, net in enumerate(fused_fc_nets())]:
         for sub in mod.modules():
             # Linear and the dense layers keep theirs out of the module tree, the convolution its alpha on the scalars
             for tp in (sub, sub.__dict__.get("_tp"), sub.__dict__.get("_alpha_head")):
@@ -326,14 +260,14 @@ def prebuild(verbose=True, workers=6):
                     jobs.append((f"module {name}", tp, (torch.float32,), True))
             if isinstance(sub, nn.FullyConnectedNet):
                 jobs.append((f"module {name} (one kernel)", sub, None, False))
-    for name, tp, dtypes in all_tensor_products():
-        jobs.append((f"kernel {name}", tp, dtypes, name in BACKWARD_CASES))
-    by_name = {name: tp for name, tp, _ in all_tensor_products()}
+    for name, tp, dtypes in products:
+        jobs.append((f"kernel {name}", tp, dtypes, name in backward))
+    by_name = {name: tp for name, tp, _ in products}
     for name, normalize, normalization in SH_MESSAGE_CASES:
         jobs.append((f"harmonics {name}", by_name[name], (normalize, normalization), False))
     for name, tp, net in radial_message_cases():
         jobs.append((f"radial {name}", tp, net, False))
-    for name, mod in nn_modules():
+    for name, mod in modules:
         if isinstance(mod, nn.Convolution):  # the block runs its radial network inside the message kernel when it can
             jobs.append((f"radial {name}", mod.tp, mod.fc, False))
 
@@ -362,7 +296,7 @@ def prebuild(verbose=True, workers=6):
         keys = [tp._plan(dt).key for dt in dtypes]
         if backward:
             tp.compile_backward(torch.float32)
-        if name.replace("kernel ", "") in BACKWARD_BF16_CASES:
+        if name.replace("kernel ", "") in set(BACKWARD_BF16_CASES) | set(backward_bf16_cases):
             tp.compile_backward(torch.bfloat16)
         return name, keys
 
