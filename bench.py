@@ -24,10 +24,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-# L2-miss traffic of one e3x_uvu_fused launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by the 1 GiB copy kernel (profiles/uvu_fused_nequip.txt), keyed by the code object the counters were read
+# L2-miss traffic of one e3x_uvu_sh_fused launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by the 1 GiB copy kernel (profiles/uvu_sh_fused_nequip.txt), keyed by the code object the counters were read
 # on: a kernel that has changed since reports no traffic instead of a stale figure.
 NEQUIP_TRAFFIC_BYTES = {
+    "uvu_3da245a80ccf1772fda9e383+sh": (2 * 1523940 + 56250) * 1024,  # FETCH_SIZE 1523940 x 2 KiB + WRITE_SIZE 56250 KiB
 }
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0

@@ -234,6 +234,16 @@ def test_edge_list_held_in_destination_order(idx):
     again = run(pre, attr_s, w_s)
     for a, b in zip(again, got):
         assert torch.equal(a, b)
+    # the kernel with the radial network inside and the one that forms the harmonics itself walk such a list by position too
+    _, tp_r, net = ks.radial_message_cases()[0]
+    net = net.to(DEV)
+    scal, vec = seeded(E, net.hs[0], seed=5).to(DEV), seeded(E, 3, seed=6).to(DEV)
+    with torch.no_grad():
+        ref_r = tp_r.forward_gather_scatter_radial(node_x, attr, scal, net, edges)
+        got_r = tp_r.forward_gather_scatter_radial(node_x, attr_s, edges.in_sorted_order(scal), net, se)
+        assert ref_r is not None and got_r is not None
+        assert (ref_r - got_r).abs().max().item() <= 1e-5 * ref_r.abs().max().item()  # (edge ranges of the workers move with the order)
+        assert torch.equal(tp.forward_gather_scatter_sh(node_x, vec, w, edges), tp.forward_gather_scatter_sh(node_x, edges.in_sorted_order(vec), w_s, se))
 
 
 @pytest.mark.parametrize("maker,N,E,idx,normalize,normalization", [
