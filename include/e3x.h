@@ -133,7 +133,8 @@ const char* e3x_tp_plan_arithmetic(const e3x_plan* plan, int which);
  * fp32 plans of the "uvw_mfma" family whose blocks are all multiples of 64 wide form their products on the
  * bf16 matrix instruction from operands split into three bf16 pieces each (six cross products, fp32 accumulation):
  * the results have the accuracy of fp32 products and are reproducible, but negating an input changes last bits
- * (scaling by a power of two does not).  E3X_UVW_SPLIT=0 in the environment at plan creation keeps the fp32
+ * (scaling by a power of two does not), and a row holding +-inf, or a finite value above 3.39e38 in magnitude (inf in
+ * bf16), comes out NaN where the fp32 instruction gives +-inf: the split forms x - bf16(x).  Rows are independent.  E3X_UVW_SPLIT=0 in the environment at plan creation keeps the fp32
  * instruction; the "uvw" weight gradient (E3X_DW_SPLIT) and the dense layers of scalars do the same. */
 int e3x_tp_forward(e3x_plan* plan, const void* x1, const void* x2, const void* w, void* out, int64_t Z,
                    void* stream);
