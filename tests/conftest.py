@@ -37,7 +37,7 @@ def golden_tp():
 def pytest_terminal_summary(terminalreporter):
     """Raw error figures of every comparison against the oracle made in this session (max abs, max relative),
     beside the pass / fail of the tolerance checks; also written as parity_errors.json into the directory named by
-    E3X_PARITY_ERRORS_DIR (default: the run's output directory at the repository root) when it exists."""
+    E3X_PARITY_ERRORS_DIR, when that is set and exists."""
     from tests.helpers import ERROR_LOG
 
     if not ERROR_LOG:
@@ -48,7 +48,7 @@ def pytest_terminal_summary(terminalreporter):
     for r in ERROR_LOG:
         tr.write_line(f"{r['what'][:60]:60s} {r['n']:9d} {r['max_abs_err']:10.3e} {r['max_abs_ref']:10.3e} "
                       f"{r['max_rel_err']:10.3e} {r['worst_err_over_tol']:8.3f}")  # fmt: skip
-    out_dir = os.environ.get("E3X_PARITY_ERRORS_DIR", os.path.join(ROOT, "gpurun_out"))
-    if os.path.isdir(out_dir):
+    out_dir = os.environ.get("E3X_PARITY_ERRORS_DIR")
+    if out_dir and os.path.isdir(out_dir):
         with open(os.path.join(out_dir, "parity_errors.json"), "w") as f:
             json.dump(ERROR_LOG, f, indent=1)
