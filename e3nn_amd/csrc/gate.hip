@@ -2,7 +2,7 @@
 // copy of a non-scalar irrep is multiplied by its own activated gate scalar.  Replaces nn.Gate.forward
 // (e3nn/nn/_gate.py:121-144: Extract -> Activation -> ElementwiseTensorProduct -> cat, about a dozen ATen kernels and
 // three intermediates) and, with no gated part, nn.Activation.forward (e3nn/nn/_activation.py:78-104).  One pass over
-// the row: HBM-bound, (in_dim + out_dim) * 4 bytes per row.
+// the row: HBM-bound, (in_dim + out_dim) * 4 bytes per row (2 bytes per element in bf16 storage; fp32 arithmetic).
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -18,6 +18,12 @@ struct Tables {
   e3x_gate_block gate[kMaxBlocks];
   int n_act, n_gate;
 };
+
+// rows are stored as fp32 or bf16; the arithmetic is fp32 either way
+__device__ __forceinline__ float ld(const float* p, long long i) { return p[i]; }
+__device__ __forceinline__ float ld(const __bf16* p, long long i) { return (float)p[i]; }
+__device__ __forceinline__ void st(float* p, long long i, float v) { p[i] = v; }
+__device__ __forceinline__ void st(__bf16* p, long long i, float v) { p[i] = (__bf16)v; }
 
 __device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(-x)); }
 
@@ -80,8 +86,9 @@ __device__ __forceinline__ float activation_d2(int kind, float x) {
 // the block tables are searched once per thread, consecutive lanes touch consecutive columns of a row.
 constexpr int kCols = 64, kRows = 4;
 
-__global__ __launch_bounds__(kCols* kRows) void gate_fwd_kernel(Tables t, const float* __restrict__ x,
-                                                                float* __restrict__ out, long long n_rows, int in_dim,
+template <class T>
+__global__ __launch_bounds__(kCols* kRows) void gate_fwd_kernel(Tables t, const T* __restrict__ x,
+                                                                T* __restrict__ out, long long n_rows, int in_dim,
                                                                 int out_dim) {
   const int c = blockIdx.x * kCols + (threadIdx.x % kCols);
   if (c >= out_dim) return;
@@ -99,20 +106,21 @@ __global__ __launch_bounds__(kCols* kRows) void gate_fwd_kernel(Tables t, const 
     }
   }
   for (long long z = (long long)blockIdx.y * kRows + threadIdx.x / kCols; z < n_rows; z += (long long)gridDim.y * kRows) {
-    const float* row = x + z * in_dim;
+    const T* row = x + z * in_dim;
     float v = 0.f;
     if (kind >= 0) {
       float f, df;
-      activation(kind, row[gate >= 0 ? gate : src], f, df);
-      v = gate >= 0 ? cst * f * row[src] : cst * f;
+      activation(kind, ld(row, gate >= 0 ? gate : src), f, df);
+      v = gate >= 0 ? cst * f * ld(row, src) : cst * f;
     }
-    out[z * out_dim + c] = v;
+    st(out, z * out_dim + c, v);
   }
 }
 
 // the same walk over the input columns: a scalar or gated component takes one term, a gate sums over its irrep
-__global__ __launch_bounds__(kCols* kRows) void gate_bwd_kernel(Tables t, const float* __restrict__ x,
-                                                                const float* __restrict__ gout, float* __restrict__ gx,
+template <class T>
+__global__ __launch_bounds__(kCols* kRows) void gate_bwd_kernel(Tables t, const T* __restrict__ x,
+                                                                const T* __restrict__ gout, T* __restrict__ gx,
                                                                 long long n_rows, int in_dim, int out_dim) {
   const int c = blockIdx.x * kCols + (threadIdx.x % kCols);
   if (c >= in_dim) return;
@@ -139,24 +147,24 @@ __global__ __launch_bounds__(kCols* kRows) void gate_bwd_kernel(Tables t, const 
     }
   }
   for (long long z = (long long)blockIdx.y * kRows + threadIdx.x / kCols; z < n_rows; z += (long long)gridDim.y * kRows) {
-    const float* row = x + z * in_dim;
-    const float* grow = gout + z * out_dim;
+    const T* row = x + z * in_dim;
+    const T* grow = gout + z * out_dim;
     float v = 0.f, f, df;
     if (a_kind >= 0) {
-      activation(a_kind, row[c], f, df);
-      v += a_cst * df * grow[a_out];
+      activation(a_kind, ld(row, c), f, df);
+      v += a_cst * df * ld(grow, a_out);
     }
     if (y_kind >= 0) {
-      activation(y_kind, row[y_gate], f, df);
-      v += y_cst * f * grow[y_out];
+      activation(y_kind, ld(row, y_gate), f, df);
+      v += y_cst * f * ld(grow, y_out);
     }
     if (g_kind >= 0) {
-      activation(g_kind, row[c], f, df);
+      activation(g_kind, ld(row, c), f, df);
       float s = 0.f;
-      for (int m = 0; m < g_dim; ++m) s += grow[g_out + m] * row[g_src + m];
+      for (int m = 0; m < g_dim; ++m) s += ld(grow, g_out + m) * ld(row, g_src + m);
       v += g_cst * df * s;
     }
-    gx[z * in_dim + c] = v;
+    st(gx, z * in_dim + c, v);
   }
 }
 
@@ -165,8 +173,9 @@ __global__ __launch_bounds__(kCols* kRows) void gate_bwd_kernel(Tables t, const 
 // A scalar block contributes cot * cst * a'(x) to gg and cot * gout * cst * a''(x) to gx2; a gated component with gate
 // s, value y, output gradient g and cotangents (cs, cy): gg = cy cst a(s) + cs cst a'(s) y,
 // dPhi/dy = cs cst a'(s) g, dPhi/ds = cst a'(s) sum(cy g) + cs cst a''(s) sum(g y).
-__global__ __launch_bounds__(kCols* kRows) void gate_bwd2_gg_kernel(Tables t, const float* __restrict__ x,
-                                                                    const float* __restrict__ cot, float* __restrict__ gg,
+template <class T>
+__global__ __launch_bounds__(kCols* kRows) void gate_bwd2_gg_kernel(Tables t, const T* __restrict__ x,
+                                                                    const T* __restrict__ cot, T* __restrict__ gg,
                                                                     long long n_rows, int in_dim, int out_dim) {
   const int c = blockIdx.x * kCols + (threadIdx.x % kCols);
   if (c >= out_dim) return;
@@ -184,21 +193,22 @@ __global__ __launch_bounds__(kCols* kRows) void gate_bwd2_gg_kernel(Tables t, co
     }
   }
   for (long long z = (long long)blockIdx.y * kRows + threadIdx.x / kCols; z < n_rows; z += (long long)gridDim.y * kRows) {
-    const float* row = x + z * in_dim;
-    const float* crow = cot + z * in_dim;
+    const T* row = x + z * in_dim;
+    const T* crow = cot + z * in_dim;
     float v = 0.f;
     if (kind >= 0) {
       float f, df;
-      activation(kind, row[gate >= 0 ? gate : src], f, df);
-      v = gate >= 0 ? cst * (crow[src] * f + crow[gate] * df * row[src]) : cst * df * crow[src];
+      activation(kind, ld(row, gate >= 0 ? gate : src), f, df);
+      v = gate >= 0 ? cst * (ld(crow, src) * f + ld(crow, gate) * df * ld(row, src)) : cst * df * ld(crow, src);
     }
-    gg[z * out_dim + c] = v;
+    st(gg, z * out_dim + c, v);
   }
 }
 
-__global__ __launch_bounds__(kCols* kRows) void gate_bwd2_gx_kernel(Tables t, const float* __restrict__ x,
-                                                                    const float* __restrict__ gout,
-                                                                    const float* __restrict__ cot, float* __restrict__ gx2,
+template <class T>
+__global__ __launch_bounds__(kCols* kRows) void gate_bwd2_gx_kernel(Tables t, const T* __restrict__ x,
+                                                                    const T* __restrict__ gout,
+                                                                    const T* __restrict__ cot, T* __restrict__ gx2,
                                                                     long long n_rows, int in_dim, int out_dim) {
   const int c = blockIdx.x * kCols + (threadIdx.x % kCols);
   if (c >= in_dim) return;
@@ -224,25 +234,25 @@ __global__ __launch_bounds__(kCols* kRows) void gate_bwd2_gx_kernel(Tables t, co
     }
   }
   for (long long z = (long long)blockIdx.y * kRows + threadIdx.x / kCols; z < n_rows; z += (long long)gridDim.y * kRows) {
-    const float* row = x + z * in_dim;
-    const float* grow = gout + z * out_dim;
-    const float* crow = cot + z * in_dim;
+    const T* row = x + z * in_dim;
+    const T* grow = gout + z * out_dim;
+    const T* crow = cot + z * in_dim;
     float v = 0.f, f, df;
-    if (a_kind >= 0) v += a_cst * activation_d2(a_kind, row[c]) * grow[a_out] * crow[c];
+    if (a_kind >= 0) v += a_cst * activation_d2(a_kind, ld(row, c)) * ld(grow, a_out) * ld(crow, c);
     if (y_kind >= 0) {
-      activation(y_kind, row[y_gate], f, df);
-      v += y_cst * df * grow[y_out] * crow[y_gate];
+      activation(y_kind, ld(row, y_gate), f, df);
+      v += y_cst * df * ld(grow, y_out) * ld(crow, y_gate);
     }
     if (g_kind >= 0) {
-      activation(g_kind, row[c], f, df);
+      activation(g_kind, ld(row, c), f, df);
       float s_cg = 0.f, s_gy = 0.f;
       for (int m = 0; m < g_dim; ++m) {
-        s_cg += crow[g_src + m] * grow[g_out + m];
-        s_gy += grow[g_out + m] * row[g_src + m];
+        s_cg += ld(crow, g_src + m) * ld(grow, g_out + m);
+        s_gy += ld(grow, g_out + m) * ld(row, g_src + m);
       }
-      v += g_cst * (df * s_cg + activation_d2(g_kind, row[c]) * crow[c] * s_gy);
+      v += g_cst * (df * s_cg + activation_d2(g_kind, ld(row, c)) * ld(crow, c) * s_gy);
     }
-    gx2[z * in_dim + c] = v;
+    st(gx2, z * in_dim + c, v);
   }
 }
 
@@ -333,22 +343,26 @@ int fill_tables(const char* who, const e3x_act_block* acts, int n_acts, const e3
 extern "C" int e3x_gate_forward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_block* gates, int32_t n_gates,
                                 const void* x, void* out, int64_t Z, int64_t in_dim, int64_t out_dim, int32_t dtype,
                                 void* stream) {
-  if (dtype != E3X_F32) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: only fp32 storage is implemented");
+  if (dtype != E3X_F32 && dtype != E3X_BF16) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: storage is fp32 or bf16");
   Tables t;
   int rc = fill_tables("e3x_gate_forward", acts, n_acts, gates, n_gates, in_dim, out_dim, &t);
   if (rc) return rc;
   if (Z < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: negative batch");
   if (Z == 0 || out_dim == 0) return E3X_OK;
   if (!x || !out) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_forward: null pointer");
-  if (is_flat(t, Z, in_dim, out_dim, x, out, nullptr)) {
+  if (dtype == E3X_F32 && is_flat(t, Z, in_dim, out_dim, x, out, nullptr)) {
     const long long n4 = Z * in_dim / 4;
     hipLaunchKernelGGL(act_flat_fwd_kernel, dim3(flat_grid(n4)), dim3(256), 0, (hipStream_t)stream, t.act[0].act, t.act[0].cst,
                        (const float4*)x, (float4*)out, n4);
     if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_forward: kernel launch failed");
     return E3X_OK;
   }
-  hipLaunchKernelGGL(gate_fwd_kernel, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
-                     (float*)out, (long long)Z, (int)in_dim, (int)out_dim);
+  if (dtype == E3X_BF16)
+    hipLaunchKernelGGL(gate_fwd_kernel<__bf16>, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t,
+                       (const __bf16*)x, (__bf16*)out, (long long)Z, (int)in_dim, (int)out_dim);
+  else
+    hipLaunchKernelGGL(gate_fwd_kernel<float>, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t,
+                       (const float*)x, (float*)out, (long long)Z, (int)in_dim, (int)out_dim);
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_forward: kernel launch failed");
   return E3X_OK;
 }
@@ -356,22 +370,26 @@ extern "C" int e3x_gate_forward(const e3x_act_block* acts, int32_t n_acts, const
 extern "C" int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_block* gates, int32_t n_gates,
                                  const void* x, const void* grad_out, void* grad_x, int64_t Z, int64_t in_dim,
                                  int64_t out_dim, int32_t dtype, void* stream) {
-  if (dtype != E3X_F32) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: only fp32 storage is implemented");
+  if (dtype != E3X_F32 && dtype != E3X_BF16) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: storage is fp32 or bf16");
   Tables t;
   int rc = fill_tables("e3x_gate_backward", acts, n_acts, gates, n_gates, in_dim, out_dim, &t);
   if (rc) return rc;
   if (Z < 0) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: negative batch");
   if (Z == 0 || in_dim == 0) return E3X_OK;
   if (!x || !grad_out || !grad_x) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward: null pointer");
-  if (is_flat(t, Z, in_dim, out_dim, x, grad_out, grad_x)) {
+  if (dtype == E3X_F32 && is_flat(t, Z, in_dim, out_dim, x, grad_out, grad_x)) {
     const long long n4 = Z * in_dim / 4;
     hipLaunchKernelGGL(act_flat_bwd_kernel, dim3(flat_grid(n4)), dim3(256), 0, (hipStream_t)stream, t.act[0].act, t.act[0].cst,
                        (const float4*)x, (const float4*)grad_out, (float4*)grad_x, n4);
     if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward: kernel launch failed");
     return E3X_OK;
   }
-  hipLaunchKernelGGL(gate_bwd_kernel, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
-                     (const float*)grad_out, (float*)grad_x, (long long)Z, (int)in_dim, (int)out_dim);
+  if (dtype == E3X_BF16)
+    hipLaunchKernelGGL(gate_bwd_kernel<__bf16>, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t,
+                       (const __bf16*)x, (const __bf16*)grad_out, (__bf16*)grad_x, (long long)Z, (int)in_dim, (int)out_dim);
+  else
+    hipLaunchKernelGGL(gate_bwd_kernel<float>, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t,
+                       (const float*)x, (const float*)grad_out, (float*)grad_x, (long long)Z, (int)in_dim, (int)out_dim);
   if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward: kernel launch failed");
   return E3X_OK;
 }
@@ -379,7 +397,7 @@ extern "C" int e3x_gate_backward(const e3x_act_block* acts, int32_t n_acts, cons
 extern "C" int e3x_gate_backward2(const e3x_act_block* acts, int32_t n_acts, const e3x_gate_block* gates, int32_t n_gates,
                                   const void* x, const void* grad_out, const void* cot_x, void* grad_grad_out, void* grad_x,
                                   int64_t Z, int64_t in_dim, int64_t out_dim, int32_t dtype, void* stream) {
-  if (dtype != E3X_F32) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward2: only fp32 storage is implemented");
+  if (dtype != E3X_F32 && dtype != E3X_BF16) return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward2: storage is fp32 or bf16");
   Tables t;
   int rc = fill_tables("e3x_gate_backward2", acts, n_acts, gates, n_gates, in_dim, out_dim, &t);
   if (rc) return rc;
@@ -388,13 +406,23 @@ extern "C" int e3x_gate_backward2(const e3x_act_block* acts, int32_t n_acts, con
   if ((in_dim && (!x || !cot_x || !grad_x)) || (out_dim && (!grad_out || !grad_grad_out)))
     return e3x::fail(E3X_ERR_INVALID, "e3x_gate_backward2: null pointer");
   if (out_dim) {
-    hipLaunchKernelGGL(gate_bwd2_gg_kernel, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
-                       (const float*)cot_x, (float*)grad_grad_out, (long long)Z, (int)in_dim, (int)out_dim);
+    if (dtype == E3X_BF16)
+      hipLaunchKernelGGL(gate_bwd2_gg_kernel<__bf16>, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t,
+                         (const __bf16*)x, (const __bf16*)cot_x, (__bf16*)grad_grad_out, (long long)Z, (int)in_dim, (int)out_dim);
+    else
+      hipLaunchKernelGGL(gate_bwd2_gg_kernel<float>, walk_grid(Z, out_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t,
+                         (const float*)x, (const float*)cot_x, (float*)grad_grad_out, (long long)Z, (int)in_dim, (int)out_dim);
     if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward2: kernel launch failed");
   }
   if (in_dim) {
-    hipLaunchKernelGGL(gate_bwd2_gx_kernel, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t, (const float*)x,
-                       (const float*)grad_out, (const float*)cot_x, (float*)grad_x, (long long)Z, (int)in_dim, (int)out_dim);
+    if (dtype == E3X_BF16)
+      hipLaunchKernelGGL(gate_bwd2_gx_kernel<__bf16>, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t,
+                         (const __bf16*)x, (const __bf16*)grad_out, (const __bf16*)cot_x, (__bf16*)grad_x, (long long)Z, (int)in_dim,
+                         (int)out_dim);
+    else
+      hipLaunchKernelGGL(gate_bwd2_gx_kernel<float>, walk_grid(Z, in_dim), dim3(kCols * kRows), 0, (hipStream_t)stream, t,
+                         (const float*)x, (const float*)grad_out, (const float*)cot_x, (float*)grad_x, (long long)Z, (int)in_dim,
+                         (int)out_dim);
     if (hipGetLastError() != hipSuccess) return e3x::fail(E3X_ERR_HIP, "e3x_gate_backward2: kernel launch failed");
   }
   return E3X_OK;

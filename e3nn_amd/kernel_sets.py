@@ -238,6 +238,10 @@ SH_MESSAGE_CASES = [("cfg3_merged", True, "component"), ("cfg3_merged", False, "
                     ("cfg4_A", True, "component"), ("odd_mul", True, "integral")]  # fmt: skip
 
 
+# node-wise blocks that the GPU tests also run in bf16 storage (forward and backward)
+BF16_MODULES = ("fc_radial", "conv_wide", "linear_wide")
+
+
 def prebuild(verbose=True, workers=6, extra_tensor_products=(), extra_modules=(), backward_cases=(), backward_bf16_cases=()):
     """Builds every kernel of this module's lists, plus ``extra_tensor_products`` (``(name, TensorProduct, dtypes)``;
     those named in ``backward_cases`` with their backward kernels) and ``extra_modules`` (``(name, module)``).  Plan creation spends its time in the HIP compiler (a child
@@ -257,7 +261,8 @@ def prebuild(verbose=True, workers=6, extra_tensor_products=(), extra_modules=()
             # Linear and the dense layers keep theirs out of the module tree, the convolution its alpha on the scalars
             for tp in (sub, sub.__dict__.get("_tp"), sub.__dict__.get("_alpha_head")):
                 if isinstance(tp, o3.TensorProduct):
-                    jobs.append((f"module {name}", tp, (torch.float32,), True))
+                    dtypes = (torch.float32, torch.bfloat16) if name in BF16_MODULES else (torch.float32,)
+                    jobs.append((f"module {name}", tp, dtypes, True))
             if isinstance(sub, nn.FullyConnectedNet):
                 jobs.append((f"module {name} (one kernel)", sub, None, False))
     for name, tp, dtypes in products:
@@ -296,7 +301,7 @@ def prebuild(verbose=True, workers=6, extra_tensor_products=(), extra_modules=()
         keys = [tp._plan(dt).key for dt in dtypes]
         if backward:
             tp.compile_backward(torch.float32)
-        if name.replace("kernel ", "") in set(BACKWARD_BF16_CASES) | set(backward_bf16_cases):
+        if name.replace("kernel ", "") in set(BACKWARD_BF16_CASES) | set(backward_bf16_cases) or (backward and torch.bfloat16 in dtypes):
             tp.compile_backward(torch.bfloat16)
         return name, keys
 

@@ -120,6 +120,10 @@ class _GateBackwardFn(torch.autograd.Function):
         return ctx.mod._launch_second(x, g, cot.contiguous()) + (None,)
 
 
+def _storage(x):
+    return _lib.BF16 if x.dtype == torch.bfloat16 else _lib.F32
+
+
 class _BlockModule(torch.nn.Module):
     """Rows ``[..., in_dim] -> [..., out_dim]`` through tables of scalar and gated blocks."""
 
@@ -139,10 +143,10 @@ class _BlockModule(torch.nn.Module):
         with torch.cuda.device(x.device):
             if grad_out is None:
                 rc = L.e3x_gate_forward(self._acts, self._n[0], self._gates, self._n[1], _lib.ptr(x), _lib.ptr(res), Z, in_dim,
-                                        out_dim, 0, _lib.stream_ptr(x.device))  # fmt: skip
+                                        out_dim, _storage(x), _lib.stream_ptr(x.device))  # fmt: skip
             else:
                 rc = L.e3x_gate_backward(self._acts, self._n[0], self._gates, self._n[1], _lib.ptr(x), _lib.ptr(grad_out),
-                                         _lib.ptr(res), Z, in_dim, out_dim, 0, _lib.stream_ptr(x.device))  # fmt: skip
+                                         _lib.ptr(res), Z, in_dim, out_dim, _storage(x), _lib.stream_ptr(x.device))  # fmt: skip
         _lib.check(rc)
         return res
 
@@ -153,7 +157,7 @@ class _BlockModule(torch.nn.Module):
         gx, gg = torch.empty_like(x), torch.empty_like(grad_out)
         with torch.cuda.device(x.device):
             rc = _lib.lib().e3x_gate_backward2(self._acts, self._n[0], self._gates, self._n[1], _lib.ptr(x), _lib.ptr(grad_out),
-                                               _lib.ptr(cot), _lib.ptr(gg), _lib.ptr(gx), Z, in_dim, out_dim, 0, _lib.stream_ptr(x.device))  # fmt: skip
+                                               _lib.ptr(cot), _lib.ptr(gg), _lib.ptr(gx), Z, in_dim, out_dim, _storage(x), _lib.stream_ptr(x.device))  # fmt: skip
         _lib.check(rc)
         return gx, gg
 
@@ -162,8 +166,8 @@ class _BlockModule(torch.nn.Module):
         torch._assert(features.shape[-1] == in_dim, "Incorrect last dimension for features")
         if not features.is_cuda:
             raise RuntimeError("e3nn_amd runs on the GPU only: move the features to a HIP device")
-        if features.dtype != torch.float32:
-            raise NotImplementedError("the gate kernel is fp32 only")
+        if features.dtype not in (torch.float32, torch.bfloat16):
+            raise NotImplementedError("the gate kernel stores rows as fp32 or bf16")
         x = features.reshape(-1, in_dim).contiguous()
         return _GateFn.apply(x, self).reshape(features.shape[:-1] + (out_dim,))
 

@@ -344,7 +344,8 @@ int e3x_sh_backward2(const int32_t* ls, int32_t n_ls, int32_t normalize, int32_t
                      const void* grad_out, const void* cot_xyz, void* grad_grad_out, void* grad_xyz, int64_t n,
                      int32_t dtype, void* stream);
 
-/* Gated non-linearity on rows x[Z, in_dim] -> out[Z, out_dim] (fp32), at most 16 blocks of each kind; columns of `out`
+/* Gated non-linearity on rows x[Z, in_dim] -> out[Z, out_dim] (stored as fp32 or bf16, `dtype`; fp32 arithmetic), at
+ * most 16 blocks of each kind; columns of `out`
  * that no block covers become 0.  Replaces nn.Gate.forward (e3nn/nn/_gate.py:121-144: Extract, Activation,
  * ElementwiseTensorProduct, cat) and, with n_gates = 0, nn.Activation.forward (e3nn/nn/_activation.py:78-104);
  * `cst` is the second-moment normalisation of e3nn/math/_normalize_activation.py:22-57.  e3x_gate_backward writes

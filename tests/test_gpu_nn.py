@@ -363,3 +363,100 @@ def test_convolution_block_forward_and_backward():
     conv(xd, node_attr.to(DEV), src.to(DEV), dst.to(DEV), edge_attr.to(DEV), edge_scalars.to(DEV)).backward(cot.to(DEV))
     for a_, b_ in zip(joint, [xd.grad] + [p.grad for p in conv.parameters()]):
         assert_close(a_, b_.cpu().numpy(), atol=1e-5 * max(1.0, float(b_.abs().max())), what="joint lin2 + alpha")
+
+
+# bf16 storage of the node-wise blocks: rows and parameters are stored as bf16, the kernels compute in fp32.  The
+# reference is the same module on the same (bf16-representable) numbers held as fp32.  Every stage that stores its
+# result as bf16 rounds it by at most 2^-8 of its size (eight significant bits, round to nearest), and the next stage
+# sums such values: the tolerance is 2^-8 of the largest reference value per stored stage, plus rel 1e-2 as for the
+# bf16 message kernels.
+def _bf16_tol(ref, stages=1):
+    return dict(atol=stages * 2.0**-8 * float(ref.detach().abs().max()), rtol=1e-2)
+
+
+def test_gate_and_activation_in_bf16_storage():
+    gate = nn.Gate("16x0e+4x0o", ["silu", "tanh"], "8x0e+4x0o", ["sigmoid", "tanh"], "8x1o+4x2e")
+    x = seeded(257, gate.irreps_in.dim, seed=3).bfloat16()
+    cot = seeded(257, gate.irreps_out.dim, seed=4).bfloat16()
+    xb, xf = x.to(DEV).requires_grad_(True), x.float().to(DEV).requires_grad_(True)
+    ob, of = gate(xb), gate(xf)
+    assert ob.dtype == torch.bfloat16
+    # one rounding of the fp32 result to bf16: at most 2^-8 of the value
+    assert_close(ob, of.detach().cpu().numpy(), atol=1e-30, rtol=2.0**-8, what="gate, bf16 storage")
+    ob.backward(cot.to(DEV))
+    of.backward(cot.float().to(DEV))
+    assert xb.grad.dtype == torch.bfloat16
+    assert_close(xb.grad, xf.grad.cpu().numpy(), atol=2.0**-8 * float(xf.grad.abs().max()), rtol=2.0**-8, what="gate gradient, bf16 storage")
+    act = nn.Activation("64x0e+8x1o", [torch.nn.functional.silu, None])
+    y = seeded(100, act.irreps_in.dim, seed=5).bfloat16().to(DEV)
+    assert_close(act(y), act(y.float()).cpu().numpy(), atol=1e-30, rtol=2.0**-8, what="activation, bf16 storage")
+    # second derivative (a loss on a gradient), against the fp32 kernels on the same numbers
+    res = []
+    for t in (x.to(DEV), x.float().to(DEV)):
+        t = t.requires_grad_(True)
+        (g1,) = torch.autograd.grad(gate(t).square().sum(), t, create_graph=True)
+        (g2,) = torch.autograd.grad(g1.square().sum(), t)
+        res.append(g2)
+    assert_close(res[0], res[1].cpu().numpy(), **_bf16_tol(res[1], 3), what="gate second derivative, bf16 storage")
+    with pytest.raises(NotImplementedError):
+        gate(x.half().to(DEV))
+
+
+def test_node_wise_blocks_in_bf16_storage():
+    import copy
+
+    lin = dict(ks.nn_modules())["linear_wide"].to(DEV)
+    x = seeded(300, lin.irreps_in.dim, seed=6).bfloat16().to(DEV)
+    with torch.no_grad():
+        lin.weight.copy_(lin.weight.bfloat16().float())
+    ref_in = x.float().requires_grad_(True)
+    ref = lin(ref_in)
+    ref.backward(torch.ones_like(ref))
+    lb = copy.deepcopy(lin).to(torch.bfloat16)
+    xb = x.clone().requires_grad_(True)
+    out = lb(xb)
+    assert out.dtype == torch.bfloat16
+    assert_close(out, ref.detach().cpu().numpy(), **_bf16_tol(ref), what="linear, bf16 storage")
+    out.backward(torch.ones_like(out))
+    assert_close(xb.grad, ref_in.grad.cpu().numpy(), **_bf16_tol(ref_in.grad), what="linear d/dx, bf16 storage")
+    assert_close(lb.weight.grad, lin.weight.grad.cpu().numpy(), **_bf16_tol(lin.weight.grad), what="linear d/dw, bf16 storage")
+
+    net = dict(ks.nn_modules())["fc_radial"].to(DEV)
+    with torch.no_grad():
+        for p in net.parameters():
+            p.copy_(p.bfloat16().float())
+    s = seeded(1000, 8, seed=7).bfloat16().to(DEV)
+    ref = net(s.float())
+    nb = copy.deepcopy(net).to(torch.bfloat16)
+    assert_close(nb(s), ref.detach().cpu().numpy(), **_bf16_tol(ref, 2), what="radial network, bf16 storage")
+    with torch.no_grad():
+        assert_close(nb(s), ref.detach().cpu().numpy(), **_bf16_tol(ref, 2), what="radial network without gradients, bf16 storage")
+
+    conv = ks.conv_wide().to(DEV)
+    with torch.no_grad():
+        conv.alpha.weight.normal_()
+        for p in conv.parameters():
+            p.copy_(p.bfloat16().float())
+    N, E = 150, 2500
+    g = torch.Generator().manual_seed(11)
+    src, dst = torch.randint(0, N, (E,), generator=g).to(DEV), torch.randint(0, N, (E,), generator=g).to(DEV)
+    node_input, node_attr = seeded(N, 288, seed=1).bfloat16().to(DEV), seeded(N, 4, seed=2).bfloat16().to(DEV)
+    edge_attr = o3.spherical_harmonics([0, 1, 2], seeded(E, 3, seed=3).to(DEV), True, "component").bfloat16()
+    edge_scalars = seeded(E, 8, seed=4).bfloat16().to(DEV)
+    xf = node_input.float().requires_grad_(True)
+    ref = conv(xf, node_attr.float(), src, dst, edge_attr.float(), edge_scalars.float())
+    cot = seeded(N, 288, seed=5).bfloat16().to(DEV)
+    ref.backward(cot.float())
+    cb = copy.deepcopy(conv).to(torch.bfloat16)
+    xb = node_input.clone().requires_grad_(True)
+    out = cb(xb, node_attr, src, dst, edge_attr, edge_scalars)
+    assert out.dtype == torch.bfloat16
+    # five bf16-stored stages in a row forward (lin1, radial weights, message, lin2 / alpha, mix), as many again backward
+    assert_close(out, ref.detach().cpu().numpy(), **_bf16_tol(ref, 5), what="convolution block, bf16 storage")
+    out.backward(cot)
+    assert_close(xb.grad, xf.grad.cpu().numpy(), **_bf16_tol(xf.grad, 10), what="convolution block d/dx, bf16 storage")
+    for (name, pb), pf in zip(cb.named_parameters(), conv.parameters()):
+        if pf.grad is None or not pf.numel():
+            continue
+        assert pb.grad.dtype == torch.bfloat16, name
+        assert_close(pb.grad, pf.grad.cpu().numpy(), **_bf16_tol(pf.grad, 10), what=f"convolution block d/d{name}, bf16 storage")
