@@ -140,6 +140,14 @@ int get_code_object(const std::string& family, const std::string& source, std::s
   *key_out = key;
   *path_out = base + ".hsaco";
   if (file_exists(*path_out)) return E3X_OK;
+  // a source that the compiler has rejected before (same compiler, same flags) is not compiled again: the log is kept
+  const std::string failed_path = base + ".failed";
+  if (file_exists(failed_path)) {
+    std::ifstream lf(failed_path);
+    std::stringstream ss;
+    ss << lf.rdbuf();
+    return fail(E3X_ERR_COMPILE, "compiling " + base + ".hip failed before (delete " + failed_path + " to try again):\n" + ss.str());
+  }
 
   if (const char* nojit = std::getenv("E3X_NO_JIT"))
     if (nojit[0] == '1')
@@ -188,6 +196,10 @@ int get_code_object(const std::string& family, const std::string& source, std::s
     std::rename(src_path.c_str(), final_src.c_str());  // keep the source that failed next to its key
     std::remove(log_path.c_str());
     std::remove(tmp_path.c_str());
+    if (WIFEXITED(status) && WEXITSTATUS(status) == 1 && !log.empty()) {  // the compiler's verdict, not a killed or missing compiler
+      std::ofstream ff(failed_path);
+      ff << log;
+    }
     return fail(E3X_ERR_COMPILE, "compiling " + final_src + " failed:\n" + log);
   }
   std::rename(src_path.c_str(), final_src.c_str());

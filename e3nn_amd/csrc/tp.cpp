@@ -1156,7 +1156,14 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
     else if (P->family == "uvw_small") rc = build_uvw_small_source(*P, *K, &src);
     else rc = build_uvu_source(*P, *K, &src);
     if (rc) return rc;
-    if ((rc = e3x::get_code_object(P->family, src, &K->key, &K->hsaco))) return rc;
+    rc = e3x::get_code_object(P->family, src, &K->key, &K->hsaco);
+    if (rc == E3X_ERR_COMPILE && P->family == "uvw_mfma" && P->dtype == E3X_BF16 && !env_int("E3X_NO_JIT", 0)) {
+      // The bf16 template hands LDS addresses to its LDS-DMA loads as scalar operands of inline assembly.  Where the
+      // compiler keeps such an address in a vector register the assembly does not build: the same source with every
+      // address forced through readfirstlane (slower by a few per cent) always does.
+      rc = e3x::get_code_object(P->family, "#define E3X_UVW16_SCALAR_ADDR 1\n" + src, &K->key, &K->hsaco);
+    }
+    if (rc) return rc;
     P->key += (P->key.empty() ? "" : "+") + K->key;
     P->subs.push_back(std::move(K));
   }
