@@ -413,3 +413,25 @@ def test_provider_module_refuses_what_the_kernels_do_not_take():
     # triangular modes have no right() in the reference either (_codegen.py:620-623): the provider defers
     tri = o3.TensorProduct("4x1o", "4x1o", "6x0e", [(0, 0, 0, "uvu<v", True)])
     assert provider.hip_provider_right(tri.irreps_in1, tri.irreps_in2, tri.irreps_out, tri.instructions, True, True, True) is None
+
+
+def test_code_object_cache_remembers_rejected_sources_and_honours_no_jit(tmp_path, monkeypatch):
+    # a cache directory of its own: nothing in it, so every plan below has to be compiled (or refused)
+    monkeypatch.setenv("E3X_KERNEL_CACHE", str(tmp_path))
+    tp = o3.FullyConnectedTensorProduct("64x0e", "64x0e", "64x0e")
+    monkeypatch.setenv("E3X_NO_JIT", "1")
+    with pytest.raises(_lib.E3xError, match="is not in the cache"):
+        tp._plan(torch.bfloat16)
+    monkeypatch.delenv("E3X_NO_JIT")
+    # two weight buffers cannot hold a stage that is fetched three stages ahead: the template's static_assert rejects it
+    monkeypatch.setenv("E3X_UVW16_NBUF", "2")
+    with pytest.raises(_lib.E3xError, match="failed:"):
+        tp._plan(torch.bfloat16)
+    marks = sorted(p.name for p in tmp_path.iterdir() if p.name.endswith(".failed"))
+    assert len(marks) == 2, marks  # the template as it is and its always-building form, both rejected for the same reason
+    assert "static assertion failed" in (tmp_path / marks[0]).read_text()
+    with pytest.raises(_lib.E3xError, match="failed before"):  # no compiler run this time
+        tp._plan(torch.bfloat16)
+    monkeypatch.delenv("E3X_UVW16_NBUF")
+    plan = tp._plan(torch.bfloat16)  # the defaults build, into the same directory
+    assert (tmp_path / (plan.key + ".hsaco")).exists() and plan.family == "uvw_mfma"
