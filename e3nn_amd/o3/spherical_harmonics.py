@@ -58,7 +58,7 @@ class _ShBackwardFn(torch.autograd.Function):
         batch = x.shape[:-1]
         xyz = x.reshape(-1, 3).contiguous()
         n = xyz.shape[0]
-        g2 = g.reshape(n, -1).contiguous()
+        g2 = g.reshape(n, sum(2 * l + 1 for l in ls)).contiguous()  # the width spelled out: -1 is ambiguous for n = 0
         gx = torch.empty_like(xyz)
         _launch("e3x_sh_backward", ls, normalize, normalization, n, x.device, xyz, g2, gx)
         ctx.save_for_backward(xyz, g2)

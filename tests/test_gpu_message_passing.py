@@ -92,6 +92,19 @@ def test_out_of_range_indices_raise_and_empty_graph():
     assert a.grad.shape == (N, 32) and not a.grad.any()
     assert b.grad is None or b.grad.shape == (0, 1)
     assert c.grad is None or c.grad.shape == (0, 32)
+    # the same through the harmonics of (no) edge vectors, stored and formed in the kernel
+    tp2 = ks.cfg3(merged=True)
+    nx = seeded(N, tp2.irreps_in1.dim).to(DEV).requires_grad_(True)
+    vec = torch.zeros(0, 3, device=DEV, requires_grad=True)
+    w2 = torch.zeros(0, tp2.weight_numel, device=DEV, requires_grad=True)
+    edges = DstSortedEdges(e, e, N)
+    for out in (tp2.forward_gather_scatter(nx, o3.spherical_harmonics([0, 1, 2], vec, True, "component"), w2, edges=edges),
+                tp2.forward_gather_scatter_sh(nx, vec, w2, edges, True, "component")):
+        assert out.shape == (N, tp2.irreps_out.dim) and not out.any()
+        gn, gv, gw = torch.autograd.grad(out.sum(), (nx, vec, w2), allow_unused=True)
+        assert gn.shape == nx.shape and not gn.any()
+        assert gv is None or gv.shape == (0, 3)
+        assert gw is None or gw.shape == (0, tp2.weight_numel)
     # source nodes without edges get a zero gradient row, the others what autograd of the dense form gives
     src2 = torch.where(src < 3, src + 3, src)  # nodes 0, 1, 2 send nothing
     a, c = node_x.clone().requires_grad_(True), w.clone().requires_grad_(True)

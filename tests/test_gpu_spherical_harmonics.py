@@ -63,6 +63,13 @@ def test_zero_vector_and_empty_input():
     assert torch.equal(z[:, 0].cpu(), torch.ones(3)) and not z[:, 1:].any()
     e = o3.spherical_harmonics([0, 1, 2], torch.zeros(0, 3, device=DEV), True, "component")
     assert e.shape == (0, 9)
+    # ... and its backward and second backward pass: empty gradients of the right shapes
+    x0 = torch.zeros(0, 3, device=DEV, requires_grad=True)
+    y0 = o3.spherical_harmonics([0, 1, 2], x0, True, "component")
+    (g0,) = torch.autograd.grad(y0.sum(), x0, create_graph=True)
+    assert g0.shape == (0, 3)
+    (h0,) = torch.autograd.grad(g0.sum(), x0)
+    assert h0.shape == (0, 3)
     one = o3.spherical_harmonics(0, torch.randn(2, 3, device=DEV), False, normalization="component")
     assert torch.equal(one.cpu(), torch.ones(2, 1))  # reference docstring example
 
