@@ -223,43 +223,69 @@ class Gate(_BlockModule):
         self.mul.register_buffer("weight", torch.Tensor())
         self.mul.register_buffer("output_mask", torch.ones(Irreps(irreps_gated).dim))
         simplified = [g.simplify() for g in groups]
-        if any(len(s) != len(g) for s, g in zip(simplified[:2], groups[:2])):
-            raise NotImplementedError("Gate: give irreps_scalars and irreps_gates in simplified form (one entry per irrep run)")
         self.irreps_scalars, self.irreps_gates, self.irreps_gated = simplified
         cat = sum(simplified, Irreps([]))
         sorted_in, p, _ = cat.sort()
         in_slices = sorted_in.slices()
         self._irreps_in = sorted_in.simplify()
         pos = 0
-        starts = []  # column of every entry of (scalars, gates, gated) in the sorted input rows
+        starts = []  # column of every entry of the simplified (scalars, gates, gated) in the sorted input rows
         for g in simplified:
             starts.append([in_slices[p[pos + i]].start for i in range(len(g))])
             pos += len(g)
 
-        out_scalars = _act_irreps_out(simplified[0], names_s, [a is not None for a in act_scalars])
-        out_gates = _act_irreps_out(simplified[1], names_g, [a is not None for a in act_gates])
+        def columns_as_given(group, simple, simple_starts):
+            # simplify() joins neighbouring entries of one irrep and keeps the order of the columns, so an entry as given
+            # sits inside one simplified entry, behind the entries joined before it
+            cols, si, used = [], 0, 0
+            for mul, ir in group:
+                if mul == 0:
+                    cols.append(0)
+                    continue
+                cols.append(simple_starts[si] + used * ir.dim)
+                used += mul
+                if used == simple[si].mul:
+                    si, used = si + 1, 0
+            return cols
+
+        # the activations act on the irreps as given: neighbouring entries of one irrep may carry different functions
+        out_scalars = _act_irreps_out(irreps_scalars, names_s, [a is not None for a in act_scalars])
+        out_gates = _act_irreps_out(irreps_gates, names_g, [a is not None for a in act_gates])
         acts, col = [], 0
-        for (mul, ir), start, name in zip(simplified[0], starts[0], names_s):
-            acts.append((start, col, mul, _KINDS[name], second_moment_constant(name)))
+        for (mul, ir), start, name in zip(irreps_scalars, columns_as_given(irreps_scalars, simplified[0], starts[0]), names_s):
+            if mul:
+                acts.append((start, col, mul, _KINDS[name], second_moment_constant(name)))
             col += mul
-        # gates and gated irreps are paired copy by copy; runs are split where their multiplicities differ
-        # (ElementwiseTensorProduct, e3nn/o3/_tensor_product/_sub.py:115-142)
-        gates_left = [[mul, ir, start, name] for (mul, ir), start, name in zip(out_gates, starts[1], names_g)]
-        gated_left = [[mul, ir, start] for (mul, ir), start in zip(simplified[2], starts[2])]
-        gate_blocks, out_gated = [], []
-        gi = 0
-        for mul_y, ir_y, start_y in gated_left:
+        # one record per gate scalar: its column, activation and the parity of the activated scalar
+        gate_copies = []
+        for (mul, ir), (_, ir_out), start, name in zip(irreps_gates, out_gates, columns_as_given(irreps_gates, simplified[1], starts[1]), names_g):
+            gate_copies += [(start + u, _KINDS[name], second_moment_constant(name), ir_out.p) for u in range(mul)]
+        # kernel blocks: gates and gated irreps are paired copy by copy; a block is a run of copies of one gated entry
+        # whose gate scalars are neighbours and share an activation
+        gate_blocks, u = [], 0
+        for (mul_y, ir_y), start_y in zip(simplified[2], starts[2]):
+            k = 0
+            while k < mul_y:
+                g_col, kind, cst, _ = gate_copies[u + k]
+                n = 1
+                while k + n < mul_y and gate_copies[u + k + n][:3] == (g_col + n, kind, cst):
+                    n += 1
+                gate_blocks.append((g_col, start_y + k * ir_y.dim, col + k * ir_y.dim, n, ir_y.dim, kind, cst))
+                k += n
+            col += mul_y * ir_y.dim
+            u += mul_y
+        # output irreps of the gated part: the reference's ElementwiseTensorProduct of the simplified gated irreps and the
+        # simplified activated gates, runs split where their multiplicities differ (e3nn/o3/_tensor_product/_sub.py:103-142)
+        left_y = [[mul, ir] for mul, ir in simplified[2]]
+        left_g = [[mul, ir] for mul, ir in out_gates.simplify()]
+        out_gated, gi = [], 0
+        for mul_y, ir_y in left_y:
             while mul_y > 0:
-                mul_g, ir_g, start_g, name = gates_left[gi]
-                n = min(mul_y, mul_g)
-                gate_blocks.append((start_g, start_y, col, n, ir_y.dim, _KINDS[name], second_moment_constant(name)))
-                out_gated.append((n, Irrep(ir_y.l, ir_y.p * ir_g.p)))
-                col += n * ir_y.dim
-                start_y += n * ir_y.dim
+                n = min(mul_y, left_g[gi][0])
+                out_gated.append((n, Irrep(ir_y.l, ir_y.p * left_g[gi][1].p)))
                 mul_y -= n
-                gates_left[gi][0] -= n
-                gates_left[gi][2] += n
-                if gates_left[gi][0] == 0:
+                left_g[gi][0] -= n
+                if left_g[gi][0] == 0:
                     gi += 1
         self._irreps_out = out_scalars + Irreps(out_gated)
         assert col == self._irreps_out.dim

@@ -95,7 +95,8 @@ def activation_forward(irreps_in, acts, x):
 
 def gate_forward(irreps_scalars, act_scalars, irreps_gates, act_gates, irreps_gated, x):
     """Returns (out, irreps_in, irreps_out) with the reference's sorted + simplified input layout."""
-    groups = [ir_.simplify(ir_.parse(g)) for g in (irreps_scalars, irreps_gates, irreps_gated)]
+    given = [ir_.parse(g) for g in (irreps_scalars, irreps_gates, irreps_gated)]
+    groups = [ir_.simplify(g) for g in given]  # _gate.py:14: the cut is made on the simplified groups ...
     cat = [t for g in groups for t in g]
     srt, p, _ = ir_.sort(cat)  # _gate.py:19-22
     sl = ir_.slices(srt)
@@ -105,8 +106,9 @@ def gate_forward(irreps_scalars, act_scalars, irreps_gates, act_gates, irreps_ga
         cols = [x[..., sl[p[pos + i]]] for i in range(len(g))]
         parts.append(np.concatenate(cols, axis=-1) if cols else np.zeros(x.shape[:-1] + (0,)))
         pos += len(g)
-    scalars, out_s = activation_forward(groups[0], act_scalars, parts[0])
-    gates, out_g = activation_forward(groups[1], act_gates, parts[1])
+    # ... and the activations act on the irreps as given (_gate.py:108-112): same columns, possibly more entries
+    scalars, out_s = activation_forward([t for t in given[0] if t[0]], [a for t, a in zip(given[0], act_scalars) if t[0]], parts[0])
+    gates, out_g = activation_forward([t for t in given[1] if t[0]], [a for t, a in zip(given[1], act_gates) if t[0]], parts[1])
     # ElementwiseTensorProduct(gated, gates): copy u of the gated irreps times gate scalar u; component
     # normalisation makes the factor exactly 1 (sqrt(2l+1) * delta / sqrt(2l+1))
     gated_cols, out_gated = [], []

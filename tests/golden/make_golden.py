@@ -332,6 +332,21 @@ def main_nn(ref="/root/reference"):
     meta["conv"] = {"args": ["4x0e+3x1o+2x1e", "2x0e", "0e+1o+2e", "5x0e+2x1o+3x2e", [3, 8], 4.0],
                     "irreps_mid": str(conv.tp.irreps_out), "tp_instructions": [[i.i_in1, i.i_in2, i.i_out] for i in conv.tp.instructions]}  # fmt: skip
 
+    # (the module parameters above are drawn from the global generator, unseeded: a new run of this section writes
+    # other, equally valid values for them; the committed files keep the values of the first run and gained the cases below)
+    # gates whose scalars / gate scalars are not in simplified form: neighbouring entries of one irrep with different
+    # activation functions, gated irreps given in pieces (drawn last, from a generator of their own, so that the cases
+    # above keep their values)
+    g2 = torch.Generator().manual_seed(1234)
+    for name, (sc, a_s, ga, a_g, gd) in {
+        "gate_entries_as_given": ("3x0e+2x0e+2x0o", ["silu", "relu", "tanh"], "2x0o+3x0o+1x0e", ["tanh", "abs", "sigmoid"], "1x2e+1x3o+3x1e+1x2o"),
+        "gate_gated_in_pieces": ("", [], "4x0e+2x0e", ["sigmoid", "tanh"], "3x1e+1x1e+2x2o"),
+    }.items():
+        gate = nn.Gate(sc, [acts[k] for k in a_s], ga, [acts[k] for k in a_g], gd)
+        x = torch.randn(5, gate.irreps_in.dim, generator=g2)
+        arrays[name + "/x"], arrays[name + "/out"] = x.numpy(), gate(x).numpy()
+        meta[name] = {"args": [sc, a_s, ga, a_g, gd], "irreps_in": str(gate.irreps_in), "irreps_out": str(gate.irreps_out)}
+
     np.savez_compressed(os.path.join(HERE, "nn_cases.npz"), **arrays)
     with open(os.path.join(HERE, "nn_cases.json"), "w") as f:
         json.dump(meta, f, separators=(",", ":"))

@@ -96,7 +96,7 @@ def test_activation_and_gate_against_reference_fixtures():
     act = nn.Activation(m["irreps_in"], [acts[a] if a else None for a in m["acts"]])
     assert str(act.irreps_out) == m["irreps_out"]
     assert_close(act(_t(arr["activation/x"])), arr["activation/out"], what="activation")
-    for name in ("gate_plain", "gate_parity", "gate_only_scalars"):
+    for name in ("gate_plain", "gate_parity", "gate_only_scalars", "gate_entries_as_given", "gate_gated_in_pieces"):
         sc, a_s, ga, a_g, gd = meta[name]["args"]
         gate = nn.Gate(sc, [acts[k] for k in a_s], ga, [acts[k] for k in a_g], gd)
         assert str(gate.irreps_in) == meta[name]["irreps_in"], name

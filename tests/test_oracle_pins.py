@@ -429,7 +429,7 @@ def test_activation_constants_and_forward_match_reference():
     np.testing.assert_allclose(out, arr["activation/out"], rtol=1e-12, atol=1e-13)
 
 
-@pytest.mark.parametrize("name", ["gate_plain", "gate_parity", "gate_only_scalars"])
+@pytest.mark.parametrize("name", ["gate_plain", "gate_parity", "gate_only_scalars", "gate_entries_as_given", "gate_gated_in_pieces"])
 def test_gate_matches_reference(name):
     from oracle import irreps as oir
     from oracle import nn as onn
@@ -438,7 +438,7 @@ def test_gate_matches_reference(name):
     m = meta[name]
     out, irreps_in, irreps_out = onn.gate_forward(*m["args"], arr[name + "/x"])
     assert oir.to_str(irreps_in) == m["irreps_in"]
-    assert oir.to_str(oir.simplify(irreps_out)) == str(m["irreps_out"]) or oir.to_str(irreps_out) == m["irreps_out"]
+    assert oir.to_str(irreps_out) == m["irreps_out"] or oir.to_str(oir.simplify(irreps_out)) == oir.to_str(oir.simplify(oir.parse(m["irreps_out"])))
     np.testing.assert_allclose(out, arr[name + "/out"], rtol=1e-12, atol=1e-13)
 
 
