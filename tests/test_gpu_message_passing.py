@@ -210,6 +210,45 @@ def test_fused_matches_oracle(maker, N, E, idx):
     assert (out - unfused).abs().max().item() < 1e-4 * scale
 
 
+# graph shapes a neighbour list can take: no edges, one edge, one node, every edge onto one row (several passes of 64
+# edges over the same accumulators), rows that alternate between empty and full, a heavy-tailed degree distribution, more
+# source nodes than rows, a list that is already sorted
+@pytest.mark.parametrize("shape,N,Ns,E", [
+    ("uniform", 1, 1, 1), ("uniform", 1, 6, 200), ("one_row", 7, 7, 3000), ("half_empty", 60, 60, 2000), ("power", 300, 305, 3000),
+    ("sorted", 60, 65, 5), ("uniform", 300, 300, 0), ("power", 2, 2, 5000),
+])  # fmt: skip
+def test_graph_shapes_through_both_message_entry_points(shape, N, Ns, E):
+    tp = ks.cfg3(True)
+    g = torch.Generator().manual_seed(N * 7919 + E)
+    if shape == "one_row":
+        dst = torch.full((E,), 3, dtype=torch.int64)
+    elif shape == "half_empty":
+        dst = torch.randint(0, N // 2, (E,), generator=g) * 2
+    elif shape == "power":
+        dst = (torch.rand(E, generator=g) ** 4 * N).long().clamp_(0, N - 1)
+    else:
+        dst = torch.randint(0, N, (E,), generator=g)
+    if shape == "sorted":
+        dst = torch.sort(dst).values
+    src = torch.randint(0, Ns, (E,), generator=g)
+    if E > 2:
+        src[1] -= Ns  # a negative source index wraps, as torch indexing does
+    node_x, vec, w = seeded(Ns, tp.irreps_in1.dim, seed=1), seeded(E, 3, seed=2), seeded(E, tp.weight_numel, seed=4)
+    if E > 3:
+        vec[0] = 0  # the zero vector: harmonics (1, 0, ..., 0)
+    idx = torch.int32 if E % 2 else torch.int64
+    edges = DstSortedEdges(src.to(idx).to(DEV), dst.to(idx).to(DEV), N, num_src_nodes=Ns)
+    attr = o3.spherical_harmonics([0, 1, 2], vec.to(DEV), True, "component")
+    ref = tp_gather_scatter(oracle_spec(tp), node_x.numpy(), attr.cpu().numpy(), w.numpy(), (src % Ns).numpy(), dst.numpy(), N) if E else np.zeros((N, tp.irreps_out.dim))
+    scale = max(1.0, float(np.abs(ref).max()))
+    for what, out in (("stored attributes", tp.forward_gather_scatter(node_x.to(DEV), attr, w.to(DEV), edges=edges)),
+                      ("harmonics in the kernel", tp.forward_gather_scatter_sh(node_x.to(DEV), vec.to(DEV), w.to(DEV), edges, True, "component"))):
+        assert_close(out, ref, atol=1e-4 * scale ** 0.5, rtol=1e-5, what=f"{shape} N={N} E={E}, {what}")
+        # rows without edges are exactly zero
+        empty = np.setdiff1d(np.arange(N), dst.numpy())
+        assert not out[torch.from_numpy(empty).to(DEV)].any()
+
+
 @pytest.mark.parametrize("idx", [torch.int32, torch.int64])
 def test_edge_list_held_in_destination_order(idx):
     # per-edge tensors rewritten once in the order the kernels walk the edges, and an edge list the caller already holds
