@@ -575,6 +575,9 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    from e3nn_amd.csrc.build import ensure_built
+
+    ensure_built()  # a tree that was never built: compile the library (kernels are specialised on first use)
 
     if args.no_headline:
         sections = {"copy": lambda: bench_copy(args, dev), "sh": lambda: bench_sh(args, dev), "mace": lambda: bench_mace(args, dev),

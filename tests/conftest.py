@@ -16,6 +16,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    # a checkout that has never been built: compile the library once (kernels are then specialised on first use)
+    from e3nn_amd.csrc.build import ensure_built
+
+    ensure_built()
+
+
 @pytest.fixture(scope="session")
 def golden_w3j():
     return dict(np.load(os.path.join(GOLDEN, "w3j.npz")))
