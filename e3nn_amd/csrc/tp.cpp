@@ -615,7 +615,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
     }
   }
   s << "constexpr int WT = " << wt << ", KMAX = " << kmax << ";\n";  // KMAX: the largest GEMM K extent
-  for (const char* knob : {"E3X_UVW16_OS", "E3X_UVW16_NBUF", "E3X_UVW16_LEAD"})
+  for (const char* knob : {"E3X_UVW16_OS", "E3X_UVW16_NBUF", "E3X_UVW16_LEAD", "E3X_UVW16_RT2", "E3X_UVW16_RT2_ROWS", "E3X_UVW16_SHIFT", "E3X_UVW16_SHIFT1"})
     if (P.dtype == E3X_BF16 && std::getenv(knob)) s << "#define " << knob << " " << env_int(knob, 0) << "\n";
   s << "struct Nz { int s, r, k; float c; };\nconstexpr int N_NZ = " << n_nz << ";\nconstexpr Nz nz[N_NZ] = {\n"
     << nzs.str() << "};\n";

@@ -288,10 +288,10 @@ def test_uvw_weight_gradient_on_the_dense_configuration():
     assert_close(got, ref, atol=1e-4 * max(1.0, float(np.abs(ref).max())), what="cfg5 weight gradient, 300 rows")
 
 
-def _bf16_uvw(seed_w=0):
-    tp = ks.cfg5().to(DEV)
+def _bf16_uvw(seed_w=0, make=ks.cfg5):
+    tp = make().to(DEV)
     w = _fan_in_weights(tp, seed=seed_w)
-    tpb = ks.cfg5().to(DEV).to(torch.bfloat16)
+    tpb = make().to(DEV).to(torch.bfloat16)
     with torch.no_grad():
         tpb.weight.copy_(w.to(torch.bfloat16))
     return tp, tpb, tpb.weight.detach().float().cpu().numpy()
@@ -342,6 +342,42 @@ def test_uvw_bf16_storage_full_size():
     part = tpb(xb[4096 : 4096 + 256], yb[4096 : 4096 + 256]).float()
     assert (part - out[4096 : 4096 + 256].float()).abs().max().item() <= 2.0**-7 * scale
     assert abs(out.float().var().item() * 16384 - 1.0) < 0.1
+
+
+@pytest.mark.parametrize("Z", [16384 + 1, 16384 + 130, 16384 + 256 + 127])
+def test_uvw_bf16_storage_ragged_batches_in_256_row_workgroups(Z):
+    # from 16384 rows on the 0e and 1o outputs are computed by workgroups of 256 rows (two row tiles per wavefront);
+    # the last workgroup here holds 1 row, a full first tile and 2 rows of the second, or a full first tile less one row
+    tp, tpb, wq = _bf16_uvw()
+    g = torch.Generator(device=DEV).manual_seed(Z)
+    xb = torch.randn(Z, 1152, device=DEV, generator=g).to(torch.bfloat16)
+    yb = torch.randn(Z, 1152, device=DEV, generator=g).to(torch.bfloat16)
+    out = tpb(xb, yb)
+    assert out.shape == (Z, 1152) and torch.isfinite(out.float()).all()
+    rows = torch.cat([torch.tensor([0, 127, 128, 255, 256, 8191]), torch.arange(max(16384 - 2, Z - 140), Z)])
+    ref = _oracle_chunks(oracle_spec(tp), xb[rows].float().cpu().numpy(), yb[rows].float().cpu().numpy(), wq)
+    scale = float(np.abs(ref).max())
+    assert_close(out[rows], ref, atol=1e-2 * scale, rtol=1e-2, what=f"bf16 uvw, Z = {Z}")
+    # the same rows as a batch below the switch (workgroups of 128 rows): equal up to the accumulation order
+    part = tpb(xb[-400:], yb[-400:]).float()
+    assert (part - out[-400:].float()).abs().max().item() <= 2.0**-7 * scale
+
+
+def test_uvw_bf16_storage_small_multiplicities_in_256_row_workgroups():
+    # multiplicities 32 and 64 (fewer weight chunks per stage than wavefronts, two and four matrix steps per outer
+    # index), four output irreps of which 0e, 1o and 1e take the 256-row workgroups; ragged last workgroup
+    tp, tpb, wq = _bf16_uvw(make=ks.mfma_small)
+    Z = 16384 + 128 + 77
+    g = torch.Generator(device=DEV).manual_seed(3)
+    xb = torch.randn(Z, tp.irreps_in1.dim, device=DEV, generator=g).to(torch.bfloat16)
+    yb = torch.randn(Z, tp.irreps_in2.dim, device=DEV, generator=g).to(torch.bfloat16)
+    out = tpb(xb, yb)
+    rows = torch.cat([torch.arange(0, 16384, 333), torch.arange(16384 - 2, Z)])
+    ref = _oracle_chunks(oracle_spec(tp), xb[rows].float().cpu().numpy(), yb[rows].float().cpu().numpy(), wq, chunk=512)
+    scale = float(np.abs(ref).max())
+    assert_close(out[rows], ref, atol=1e-2 * scale, rtol=1e-2, what="bf16 uvw, small multiplicities")
+    part = tpb(xb[-300:], yb[-300:]).float()
+    assert (part - out[-300:].float()).abs().max().item() <= 2.0**-7 * scale
 
 
 def test_provider_binding_runs_the_same_kernels():
