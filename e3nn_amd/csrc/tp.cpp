@@ -520,15 +520,15 @@ int build_uvw_small_source(e3x_plan& P, SubKernel& K, std::string* src) {
 // 64-row slice of the K operand in LDS (K * 256 bytes), the bf16 kernel keeps its K operand in registers
 int k_cap(int dtype) { return dtype == E3X_BF16 ? 256 : 512; }
 
-bool uvw_mfma_eligible(const e3x_plan& P) {
+bool uvw_mfma_eligible(const e3x_plan& P, int dtype) {
   if (!P.shared_weights || P.paths.empty()) return false;
   for (const auto& p : P.paths) {
     const int U = P.in1[p.in1].mul, V = P.in2[p.in2].mul, W = P.out[p.out].mul;
     // fp32: 32-channel granularity (a half-filled last tile); bf16: whole 64-channel tiles
-    if (W % (P.dtype == E3X_BF16 ? 64 : 32) || P.out[p.out].l > 3 || U < 1 || V < 1) return false;
-    const int kcap = k_cap(P.dtype);
+    if (W % (dtype == E3X_BF16 ? 64 : 32) || P.out[p.out].l > 3 || U < 1 || V < 1) return false;
+    const int kcap = k_cap(dtype);
     const bool okU = U % 32 == 0 && U <= kcap, okV = V % 32 == 0 && V <= kcap;
-    if (P.dtype == E3X_BF16) {
+    if (dtype == E3X_BF16) {
       // both multiplicities tile: the outer index runs in blocks of 8
       if (!okU || !okV) return false;
       // the bf16 kernel reads 8 consecutive bf16 of a row with one 16-byte load
@@ -541,6 +541,7 @@ bool uvw_mfma_eligible(const e3x_plan& P) {
   }
   return true;
 }
+bool uvw_mfma_eligible(const e3x_plan& P) { return uvw_mfma_eligible(P, P.dtype); }
 
 int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   // Output channels per workgroup.  fp32: 128 (two accumulator tiles per wave, 64 KB of LDS, two workgroups per CU at
@@ -637,7 +638,7 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
 constexpr int kNodeMaxBlocks = 64;
 
 bool uvw_node_eligible(const e3x_plan& P) {
-  if (P.dtype != E3X_F32 || !P.shared_weights || P.paths.empty() || env_int("E3X_UVW_NODE", 1) == 0) return false;
+  if (!P.shared_weights || P.paths.empty() || env_int("E3X_UVW_NODE", 1) == 0) return false;
   if (P.in2_dim < 1 || P.in2_dim > 16 || P.in1_dim % 4) return false;
   for (const auto& r : P.in2) if (r.l != 0) return false;
   std::vector<int> blocks(P.out.size(), 0);
@@ -658,7 +659,8 @@ bool uvw_node_eligible(const e3x_plan& P) {
   for (int n : blocks) if (n > kNodeMaxBlocks) return false;
   // a handful of (u, v) pairs in shapes the other matrix-core kernel does not take: the vector-ALU kernel keeps the
   // weights in registers and needs no padding to 32 channels
-  return pairs > 64 || uvw_mfma_eligible(P);
+  // (the same choice in both storages: the tiling rule asked is the fp32 kernel's)
+  return pairs > env_int("E3X_NODE_MIN_PAIRS", 64) || uvw_mfma_eligible(P, E3X_F32);
 }
 
 int build_uvw_node_source(e3x_plan& P, std::string* src) {
@@ -713,7 +715,8 @@ int build_uvw_node_source(e3x_plan& P, std::string* src) {
     // matrix steps on split operands (see the template) where every input multiplicity is a multiple of 16
     bool split = true;
     for (const auto& p : P.paths) split = split && P.in1[p.in1].mul % 16 == 0;
-    split = split && env_int("E3X_NODE_SPLIT", 1) != 0;
+    // (bf16 storage: the fp32 instruction on the converted values, whose products with the scalar are exact)
+    split = split && P.dtype == E3X_F32 && env_int("E3X_NODE_SPLIT", 1) != 0;
     if (split) s << "#define E3X_NODE_SPLIT 1\n";
     P.arithmetic = split ? "bf16 matrix instruction, six products of three-way split operands" : "fp32 matrix instruction";
   }

@@ -147,15 +147,15 @@ def all_tensor_products():
         ("cfg5", cfg5(), (torch.float32, torch.bfloat16)),
         ("mfma_small", mfma_small(), (torch.float32,)),
         ("mfma_full_tiles", mfma_full_tiles(), (torch.float32,)),
-        ("node_fctp", node_fctp(), (torch.float32,)),
+        ("node_fctp", node_fctp(), (torch.float32, torch.bfloat16)),
         ("radial_layer", radial_layer(), (torch.float32,)),
         ("wide_k", wide_k(), (torch.float32,)),
         ("wide_k_full_tiles", wide_k_full_tiles(), (torch.float32,)),
         ("outer_split", outer_split(), (torch.float32,)),
         ("node_block", node_block(), (torch.float32,)),
-        ("node_wide_out", node_wide_out(), (torch.float32,)),
-        ("node_narrow", node_narrow(), (torch.float32,)),
-        ("node_partial_tile", node_partial_tile(), (torch.float32,)),
+        ("node_wide_out", node_wide_out(), (torch.float32, torch.bfloat16)),
+        ("node_narrow", node_narrow(), (torch.float32, torch.bfloat16)),
+        ("node_partial_tile", node_partial_tile(), (torch.float32, torch.bfloat16)),
         ("unaligned_mfma", unaligned_mfma(), (torch.float32,)),
         ("unaligned_offsets", unaligned_offsets(), (torch.float32,)),
         ("mixed_modes", mixed_modes(), (torch.float32,)),

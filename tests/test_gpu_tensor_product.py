@@ -188,6 +188,26 @@ def test_uvw_matrix_core_kernel_against_oracle(maker, Z, family):
     assert_close(out, ref, what=str(tp))
 
 
+@pytest.mark.parametrize("maker,Z", [(ks.node_fctp, 333), (ks.node_fctp, 1), (ks.node_wide_out, 130), (ks.node_narrow, 301), (ks.node_partial_tile, 257)])
+def test_node_wise_kernel_in_bf16_storage_against_oracle(maker, Z):
+    # rows, scalars and weights stored as bf16 (8-byte pieces; weight rows element by element where the channel
+    # counts are no multiples of 4), fp32 matrix instructions on the converted values, one rounding of the output
+    tp = maker().to(DEV)
+    w = _fan_in_weights(tp)
+    tpb = maker().to(DEV).to(torch.bfloat16)
+    assert tpb._plan(torch.bfloat16).family == "uvw_node"
+    with torch.no_grad():
+        tpb.weight.copy_(w.to(torch.bfloat16))
+    xb = seeded(Z, tp.irreps_in1.dim, seed=41).to(DEV).to(torch.bfloat16)
+    yb = seeded(Z, tp.irreps_in2.dim, seed=42).to(DEV).to(torch.bfloat16)
+    out = tpb(xb, yb)
+    assert out.dtype == torch.bfloat16 and out.shape == (Z, tp.irreps_out.dim)
+    ref = otp.tp_forward(oracle_spec(tp), xb.float().cpu().numpy(), yb.float().cpu().numpy(), tpb.weight.detach().float().cpu().numpy())
+    scale = float(np.abs(ref).max())
+    # bf16 rounds to nearest with 8 significant bits: at most 2^-8 relative; the absolute term covers elements near zero
+    assert_close(out, ref, atol=2.0**-9 * scale, rtol=2.0**-8, what=f"bf16 node-wise {tp}")
+
+
 def test_uvw_full_size_dense_configuration():
     # FCTP(128x0e+128x1o+128x2e x same -> same), batch 65536, weights N(0, 1/fan_in), inputs N(0, 1)
     tp = ks.cfg5().to(DEV)

@@ -278,7 +278,8 @@ def test_state_dict_keys_match_the_reference():
 def test_kernel_family_selection_for_scalar_second_inputs():
     """Shared-weight uvw products whose second input holds scalars only take the node-wise matrix-core kernel when the
     input multiplicities are multiples of 8; a handful of (u, v) pairs stays on the vector-ALU kernel with its weights
-    in registers; anything with a non-scalar second input, per-sample weights or bf16 storage takes the other kernels."""
+    in registers; anything with a non-scalar second input or per-sample weights takes the other kernels.  The choice is
+    the same in fp32 and bf16 storage."""
     fam = lambda tp, dt=torch.float32: tp._plan(dt).family  # noqa: E731
     assert fam(ks.node_fctp()) == fam(ks.node_narrow()) == fam(ks.node_partial_tile()) == fam(ks.node_wide_out()) == "uvw_node"
     assert fam(ks.outer_split()) == fam(ks.mfma_small()) == "uvw_mfma"  # second input with l > 0
@@ -286,6 +287,12 @@ def test_kernel_family_selection_for_scalar_second_inputs():
     assert fam(o3.FullyConnectedTensorProduct("12x0e", "4x0e", "32x0e")) == "uvw_small"  # multiplicity not a multiple of 8
     assert fam(o3.FullyConnectedTensorProduct("64x0e", "4x0e", "64x0e", shared_weights=False, internal_weights=False)) == "uvw_small"
     assert fam(ks.cfg5(), torch.bfloat16) == "uvw_mfma"
+    for tp in (ks.node_fctp(), ks.node_narrow(), ks.node_partial_tile(), ks.node_wide_out()):
+        assert fam(tp, torch.bfloat16) == "uvw_node"
+    # the layers of a radial network 8 -> 64 -> 352 as products with the constant "0e": same family in both storages
+    for h_in, h_out, want in ((8, 64, "uvw_small"), (64, 352, "uvw_node")):
+        layer = o3.TensorProduct(f"{h_in}x0e", "0e", f"{h_out}x0e", [(0, 0, 0, "uvw", True)], internal_weights=False, shared_weights=True)
+        assert fam(layer) == fam(layer, torch.bfloat16) == want
 
 
 def test_radial_message_kernel_is_offered_only_for_what_it_takes():
