@@ -115,7 +115,7 @@ int e3x_wigner_3j(int l1, int l2, int l3, double* out);
 int e3x_tp_plan_create(const e3x_tp_desc* desc, e3x_plan** out);
 int e3x_tp_plan_destroy(e3x_plan* plan);
 /* weight_numel (reference _tensor_product.py:403), in1/in2/out dims, and the kernel family
- * name ("uvu", "uvw_small", "uvw_mfma"); any out pointer may be NULL. */
+ * name ("uvu", "uvw_small", "uvw_mfma", "uvw_node"); any out pointer may be NULL. */
 int e3x_tp_plan_info(const e3x_plan* plan, int64_t* weight_numel, int64_t* in1_dim, int64_t* in2_dim,
                      int64_t* out_dim, const char** family, const char** cache_key);
 
