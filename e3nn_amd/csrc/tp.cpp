@@ -524,8 +524,8 @@ bool uvw_mfma_eligible(const e3x_plan& P, int dtype) {
   if (!P.shared_weights || P.paths.empty()) return false;
   for (const auto& p : P.paths) {
     const int U = P.in1[p.in1].mul, V = P.in2[p.in2].mul, W = P.out[p.out].mul;
-    // fp32: 32-channel granularity (a half-filled last tile); bf16: whole 64-channel tiles
-    if (W % (dtype == E3X_BF16 ? 64 : 32) || P.out[p.out].l > 3 || U < 1 || V < 1) return false;
+    // 32-channel granularity (a half-filled last tile)
+    if (W % 32 || P.out[p.out].l > 3 || U < 1 || V < 1) return false;
     const int kcap = k_cap(dtype);
     const bool okU = U % 32 == 0 && U <= kcap, okV = V % 32 == 0 && V <= kcap;
     if (dtype == E3X_BF16) {

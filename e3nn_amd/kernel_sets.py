@@ -50,6 +50,12 @@ def mfma_full_tiles():
     return o3.FullyConnectedTensorProduct("64x0e+64x1o", "64x0e+64x1o+64x2e", "64x0e+128x1o+64x1e+64x2e")
 
 
+def mfma_half_tiles():
+    # output multiplicities 32 and 96: the matrix-core kernels end an irrep with a tile of 32 channels (bf16 storage:
+    # half of the 64-channel workgroup tile computes on copies and stores nothing)
+    return o3.FullyConnectedTensorProduct("64x0e+32x1o", "32x0e+32x1o", "32x0e+96x1o+32x2e")
+
+
 def node_fctp():
     # node-wise step of a convolution: features x a few scalar node attributes (one-hot species), the GEMM K index is
     # the feature multiplicity and the attribute index is a short outer loop (reference
@@ -147,6 +153,7 @@ def all_tensor_products():
         ("cfg5", cfg5(), (torch.float32, torch.bfloat16)),
         ("mfma_small", mfma_small(), (torch.float32,)),
         ("mfma_full_tiles", mfma_full_tiles(), (torch.float32,)),
+        ("mfma_half_tiles", mfma_half_tiles(), (torch.float32, torch.bfloat16)),
         ("node_fctp", node_fctp(), (torch.float32, torch.bfloat16)),
         ("radial_layer", radial_layer(), (torch.float32,)),
         ("wide_k", wide_k(), (torch.float32,)),

@@ -400,6 +400,22 @@ def test_uvw_bf16_storage_small_multiplicities_in_256_row_workgroups():
     assert (part - out[-300:].float()).abs().max().item() <= 2.0**-7 * scale
 
 
+@pytest.mark.parametrize("Z", [300, 16384 + 77])
+def test_uvw_bf16_storage_tiles_of_32_channels(Z):
+    # irreps of 32 and 96 channels: their last workgroup tile holds 32 channels instead of 64 (both row tilings)
+    tp, tpb, wq = _bf16_uvw(make=ks.mfma_half_tiles)
+    assert tpb._plan(torch.bfloat16).family == "uvw_mfma"
+    g = torch.Generator(device=DEV).manual_seed(Z)
+    xb = torch.randn(Z, tp.irreps_in1.dim, device=DEV, generator=g).to(torch.bfloat16)
+    yb = torch.randn(Z, tp.irreps_in2.dim, device=DEV, generator=g).to(torch.bfloat16)
+    out = tpb(xb, yb)
+    assert torch.isfinite(out.float()).all()
+    rows = torch.cat([torch.arange(0, min(Z, 16384), 97), torch.arange(max(0, Z - 200), Z)])
+    ref = _oracle_chunks(oracle_spec(tp), xb[rows].float().cpu().numpy(), yb[rows].float().cpu().numpy(), wq, chunk=512)
+    scale = float(np.abs(ref).max())
+    assert_close(out[rows], ref, atol=1e-2 * scale, rtol=1e-2, what=f"bf16 uvw, 32-channel tiles, Z = {Z}")
+
+
 def test_provider_binding_runs_the_same_kernels():
     # modules built by the provider from (Irreps, Instruction) data give the product's own results, with e3nn's
     # broadcasting of leading dimensions -- also after the pickle round trip e3nn puts its generated modules through
