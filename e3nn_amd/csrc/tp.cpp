@@ -715,8 +715,7 @@ int build_uvw_node_source(e3x_plan& P, std::string* src) {
     // matrix steps on split operands (see the template) where every input multiplicity is a multiple of 16
     bool split = true;
     for (const auto& p : P.paths) split = split && P.in1[p.in1].mul % 16 == 0;
-    // (bf16 storage: the fp32 instruction on the converted values, whose products with the scalar are exact)
-    split = split && P.dtype == E3X_F32 && env_int("E3X_NODE_SPLIT", 1) != 0;
+    split = split && env_int("E3X_NODE_SPLIT", 1) != 0;
     if (split) s << "#define E3X_NODE_SPLIT 1\n";
     P.arithmetic = split ? "bf16 matrix instruction, six products of three-way split operands" : "fp32 matrix instruction";
   }
