@@ -225,6 +225,10 @@ int build_uvu_source(e3x_plan& P, SubKernel& K, std::string* src, bool bwd_only 
     return u * (accregs + x1regs + wregs) + (int)P.in2_dim <= 200;
   };
   while (upl > 1 && !fits(upl)) upl /= 2;
+  // narrow sets: a group of lanes is at least 8 wide, so fewer indices per lane keep its lanes busy (measured on
+  // 500 000 edges, l <= 2: multiplicity 8 with 4 / 2 / 1 per lane 0.203 / 0.109 / 0.096 ms in fp32 and 0.485 / 0.138 /
+  // 0.085 ms in bf16 storage; multiplicity 16: 0.230 / 0.126 / 0.123 ms and 0.520 / 0.098 / 0.099 ms)
+  while (upl > 1 && max_mul / upl < 8) upl /= 2;
   upl = env_int("E3X_UVU_UPL", upl);
   // the backward kernel also holds the output gradient of its indices: one index per lane keeps it at several waves
   // per SIMD (measured on the 32-channel l <= 2 set: 1.39 ms against 1.85 ms with four)
@@ -538,6 +542,17 @@ bool uvw_mfma_eligible(const e3x_plan& P, int dtype) {
       // any length -- e.g. node features x a few node attributes, or a linear map (second input "0e")
       return false;
     }
+  }
+  if (dtype == E3X_BF16) {
+    // LDS of the bf16 kernel: four weight buffers of one stage (32 KB each up to 128 K indices, 64 KB above) and two
+    // blocks of the R operand for 128 rows
+    int kmax = 32, drmax = 1;
+    for (const auto& p : P.paths) {
+      kmax = std::max(kmax, std::max(P.in1[p.in1].mul, P.in2[p.in2].mul));
+      drmax = std::max(drmax, 2 * std::max(P.in1[p.in1].l, P.in2[p.in2].l) + 1);
+    }
+    const long long stage = (long long)(256 / kmax >= 2 ? 2 : 1) * (kmax / 8) * 64 * 16;
+    if (4 * stage + 2LL * drmax * 128 * 16 > 160 * 1024) return false;
   }
   return true;
 }

@@ -16,7 +16,7 @@ SH2 = str(o3.Irreps.spherical_harmonics(2))
 SH3 = str(o3.Irreps.spherical_harmonics(3))
 
 # backward pass in bf16 storage as well (callers of prebuild may add names): a matrix-core uvw set, per-edge uvu weights
-BACKWARD_BF16_CASES = ["mfma_small", "cfg3_merged"]
+BACKWARD_BF16_CASES = ["mfma_small", "cfg3_merged", "wide_k_l3"]
 
 
 def cfg1():
@@ -54,6 +54,12 @@ def mfma_half_tiles():
     # output multiplicities 32 and 96: the matrix-core kernels end an irrep with a tile of 32 channels (bf16 storage:
     # half of the 64-channel workgroup tile computes on copies and stores nothing)
     return o3.FullyConnectedTensorProduct("64x0e+32x1o", "32x0e+32x1o", "32x0e+96x1o+32x2e")
+
+
+def wide_k_l3():
+    # 256 and 96 copies of l = 2, 3 against 32 vectors: the input gradients contract over 256 indices with an R operand
+    # of 5 and 7 components, the largest LDS footprint of the bf16 matrix-core kernel
+    return o3.FullyConnectedTensorProduct("256x2e+96x3o", "32x1o", "128x1o+64x3o")
 
 
 def node_fctp():
@@ -154,6 +160,7 @@ def all_tensor_products():
         ("mfma_small", mfma_small(), (torch.float32,)),
         ("mfma_full_tiles", mfma_full_tiles(), (torch.float32,)),
         ("mfma_half_tiles", mfma_half_tiles(), (torch.float32, torch.bfloat16)),
+        ("wide_k_l3", wide_k_l3(), (torch.float32, torch.bfloat16)),
         ("node_fctp", node_fctp(), (torch.float32, torch.bfloat16)),
         ("radial_layer", radial_layer(), (torch.float32,)),
         ("wide_k", wide_k(), (torch.float32,)),

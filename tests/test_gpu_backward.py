@@ -276,7 +276,7 @@ def test_spherical_harmonics_gradient_any_l_list(ls, normalize, normalization):
 
 
 @pytest.mark.parametrize("maker,Z,shared", [(ks.mfma_small, 300, True), (lambda: ks.golden_tp("uvu_shared_v2"), 200, True),
-                                            (lambda: ks.cfg3(True), 130, False)])  # fmt: skip
+                                            (lambda: ks.cfg3(True), 130, False), (ks.wide_k_l3, 150, True)])  # fmt: skip
 def test_gradients_in_bf16_storage(maker, Z, shared):
     """bf16 storage, fp32 accumulation: every gradient against float64 autograd of the oracle on the same (bf16-rounded)
     inputs, to the bf16 tolerance rel 1e-2 of the largest entry (inputs, outputs and gradients are rounded to bf16)."""
