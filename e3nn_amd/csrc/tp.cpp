@@ -582,7 +582,12 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
   P.arithmetic = P.dtype != E3X_F32 ? "bf16 matrix instruction" : split ? "bf16 matrix instruction, six products of three-way split operands" : "fp32 matrix instruction";
   if (P.dtype == E3X_F32) s << "#define E3X_UVW_KC " << env_int("E3X_UVW_KC", split ? 16 : 32) << "\n";
   if (env_int("E3X_UVW_KS", 0)) s << "#define E3X_UVW_KS " << env_int("E3X_UVW_KS", 0) << "\n";
-  if (env_int("E3X_UVW_WPE", wt == 128 ? 2 : 0)) s << "#define E3X_UVW_WPE " << env_int("E3X_UVW_WPE", wt == 128 ? 2 : 0) << "\n";
+  // two waves per SIMD (256 registers) for 128-channel tiles and for l = 3 outputs, whose seven accumulator tiles do not
+  // fit the 168 registers of three (64x1o+64x2e squared -> 32x3o: 3122 registers' worth of spills there, none here)
+  bool out_l3 = false;
+  for (const auto& p : P.paths) out_l3 = out_l3 || P.out[p.out].l >= 3;
+  const int wpe = env_int("E3X_UVW_WPE", wt == 128 || out_l3 ? 2 : 0);
+  if (wpe) s << "#define E3X_UVW_WPE " << wpe << "\n";
   int n_nz = 0, n_path = 0, n_target = 0, dka = 1, drmax = 1;
   for (size_t c = 0; c < P.out.size(); ++c) {
     std::ostringstream mine;
@@ -1161,6 +1166,7 @@ extern "C" int e3x_tp_plan_create(const e3x_tp_desc* d, e3x_plan** out) {
     P->family = "uvu";
     parts = split_uvu_paths(*P);
   }
+  if (P->paths.empty()) parts.clear();  // nothing to contract: every entry point fills the outputs with zeros and returns
   for (auto& ids : parts) {
     std::unique_ptr<SubKernel> K(new SubKernel);
     K->path_ids = ids;

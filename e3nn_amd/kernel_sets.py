@@ -56,6 +56,11 @@ def mfma_half_tiles():
     return o3.FullyConnectedTensorProduct("64x0e+32x1o", "32x0e+32x1o", "32x0e+96x1o+32x2e")
 
 
+def mfma_l3_out():
+    # an l = 3 output (seven accumulator tiles per wave) beside a vector output, 32 and 64 channels
+    return o3.FullyConnectedTensorProduct("64x1o+64x2e", "64x1o+64x2e", "32x3o+64x1o")
+
+
 def wide_k_l3():
     # 256 and 96 copies of l = 2, 3 against 32 vectors: the input gradients contract over 256 indices with an R operand
     # of 5 and 7 components, the largest LDS footprint of the bf16 matrix-core kernel
@@ -161,6 +166,7 @@ def all_tensor_products():
         ("mfma_full_tiles", mfma_full_tiles(), (torch.float32,)),
         ("mfma_half_tiles", mfma_half_tiles(), (torch.float32, torch.bfloat16)),
         ("wide_k_l3", wide_k_l3(), (torch.float32, torch.bfloat16)),
+        ("mfma_l3_out", mfma_l3_out(), (torch.float32,)),
         ("node_fctp", node_fctp(), (torch.float32, torch.bfloat16)),
         ("radial_layer", radial_layer(), (torch.float32,)),
         ("wide_k", wide_k(), (torch.float32,)),

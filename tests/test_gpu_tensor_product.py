@@ -106,6 +106,18 @@ def test_batch_broadcasting_weight_lists_and_errors():
     assert shared(torch.zeros(0, 64, device=DEV), torch.zeros(0, 9, device=DEV)).shape == (0, 144)
 
 
+def test_product_without_instructions_gives_zeros():
+    # no path is allowed by parity (e3nn builds such a product without complaint): zeros forward, zero gradients
+    tp = o3.FullyConnectedTensorProduct("8x3o", "64x2e", "16x2e").to(DEV)
+    assert len(tp.instructions) == 0 and tp.weight_numel == 0
+    x1 = seeded(5, tp.irreps_in1.dim).to(DEV).requires_grad_(True)
+    x2 = seeded(5, tp.irreps_in2.dim, seed=1).to(DEV).requires_grad_(True)
+    out = tp(x1, x2)
+    assert out.shape == (5, 80) and not out.any()
+    g1, g2 = torch.autograd.grad(out, (x1, x2), torch.ones_like(out), allow_unused=True)
+    assert (g1 is None or not g1.any()) and (g2 is None or not g2.any())
+
+
 def test_missing_output_paths_are_exact_zeros():
     tp = ks.golden_tp("empty_path_and_missing_output").to(DEV)
     out = tp(seeded(6, tp.irreps_in1.dim).to(DEV), seeded(6, tp.irreps_in2.dim, seed=1).to(DEV))
@@ -170,6 +182,8 @@ def _fan_in_weights(tp, seed=0):
     [(ks.mfma_small, 150, "uvw_mfma"), (ks.cfg5, 70, "uvw_mfma"), (ks.wide_k, 130, "uvw_mfma"), (ks.outer_split, 200, "uvw_mfma"),
      # every multiplicity a multiple of 64: the matrix steps on split operands (also on restaged K blocks)
      (ks.mfma_full_tiles, 150, "uvw_mfma"), (ks.wide_k_full_tiles, 130, "uvw_mfma"),
+     # an l = 3 output: seven accumulator tiles per wave, two waves per SIMD
+     (ks.mfma_l3_out, 210, "uvw_mfma"),
      # scalar second input: the node-wise kernel; batches that end inside a wave's 64 rows, inside a workgroup's 256
      # rows, and below one wave
      (ks.node_fctp, 333, "uvw_node"), (ks.node_fctp, 17, "uvw_node"), (ks.node_fctp, 1280, "uvw_node"),
