@@ -153,6 +153,12 @@ def odd_mul():
     return message_tensor_product("80x0e+24x1o+5x2e", SH2, keep="0e+1o+2e")
 
 
+def narrow_message():
+    # 16 channels per irrep: fewer multiplicity indices per lane than the wider sets, so that a lane group stays busy
+    f = "16x0e+16x1o+16x2e"
+    return message_tensor_product(f, SH2, irreps_out=f)
+
+
 def all_tensor_products():
     """(name, TensorProduct, dtypes) for everything that must be in the kernel cache."""
     out = [
@@ -182,6 +188,7 @@ def all_tensor_products():
         ("scalar_exact", scalar_exact(), (torch.float32,)),
         ("right_small", right_small(), (torch.float32,)),
         ("odd_mul", odd_mul(), (torch.float32,)),
+        ("narrow_message", narrow_message(), (torch.float32, torch.bfloat16)),
     ]
     return out
 
@@ -189,7 +196,7 @@ def all_tensor_products():
 # instruction sets whose backward pass the GPU tests run (transposed plans are separate kernels)
 BACKWARD_CASES = ["cfg1", "cfg3_merged", "cfg3_builder", "cfg4_A", "cfg5", "mfma_small", "mfma_full_tiles", "outer_split", "node_fctp", "node_block",
                   "node_wide_out", "node_narrow", "node_partial_tile", "radial_layer", "odd_mul", "unaligned_mfma", "unaligned_offsets",
-                  "mixed_modes", "scalar_exact"]  # fmt: skip
+                  "mixed_modes", "scalar_exact", "narrow_message"]  # fmt: skip
 
 
 def linear_channels(norm="element"):
@@ -255,7 +262,7 @@ def conv_wide():
 
 # (set, normalize, normalization) of the message kernels that form the spherical harmonics of the edge vectors themselves
 SH_MESSAGE_CASES = [("cfg3_merged", True, "component"), ("cfg3_merged", False, "integral"), ("cfg3_builder", True, "norm"),
-                    ("cfg4_A", True, "component"), ("odd_mul", True, "integral")]  # fmt: skip
+                    ("cfg4_A", True, "component"), ("odd_mul", True, "integral"), ("narrow_message", True, "component")]  # fmt: skip
 
 
 # node-wise blocks that the GPU tests also run in bf16 storage (forward and backward)

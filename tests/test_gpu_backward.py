@@ -48,7 +48,7 @@ def test_uvu_plain_gradients(maker, Z):
                                            (lambda: ks.cfg4("A"), 25, 300, torch.int32),
                                            # multiplicities that leave lane groups partly filled (80, 24, 5): every
                                            # weight-gradient column must still be written (the buffer is not zero-filled)
-                                           (ks.odd_mul, 40, 600, torch.int32)])  # fmt: skip
+                                           (ks.odd_mul, 40, 600, torch.int32), (ks.narrow_message, 60, 900, torch.int64)])  # fmt: skip
 def test_fused_message_gradients(maker, N, E, idx):
     tp = maker()
     spec = oracle_spec(tp)

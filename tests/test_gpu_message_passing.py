@@ -190,6 +190,7 @@ def test_row_processing_order(idx):
     (lambda: ks.cfg4("A"), 60, 1_500, torch.int32),
     (lambda: ks.cfg4("B"), 40, 700, torch.int32),
     (ks.odd_mul, 90, 2_000, torch.int32),
+    (ks.narrow_message, 150, 4_000, torch.int64),  # 16 channels: two multiplicity indices per lane
 ])  # fmt: skip
 def test_fused_matches_oracle(maker, N, E, idx):
     tp = maker()
@@ -304,6 +305,7 @@ def test_edge_list_held_in_destination_order(idx):
     (lambda: ks.cfg3(False), 300, 9_000, torch.int64, True, "norm"),
     (lambda: ks.cfg4("A"), 60, 1_500, torch.int32, True, "component"),
     (ks.odd_mul, 90, 2_000, torch.int32, True, "integral"),
+    (ks.narrow_message, 70, 1_800, torch.int64, True, "component"),
 ])  # fmt: skip
 def test_fused_with_the_harmonics_formed_in_the_kernel(maker, N, E, idx, normalize, normalization):
     # edge_attr = spherical_harmonics(0 .. lmax, edge_vec) evaluated inside the message kernel from the 12-byte vectors:
