@@ -653,9 +653,11 @@ int build_uvw_mfma_source(e3x_plan& P, std::string* src) {
 }
 
 // ---- uvw with a scalar second input (node-wise linear layers) on the matrix cores ------------------
-// A target (one output irrep x 32 channels) keeps the weights of all its paths in LDS: at most kNodeMaxBlocks
-// blocks of 8 x 32 floats (64 KB, two workgroups per CU).
-constexpr int kNodeMaxBlocks = 64;
+// A target (one output irrep x 32 channels) keeps the weights of all its paths in LDS: at most this many blocks of
+// 8 x 32 floats (144 KB, one workgroup per CU; up to 64 KB two or three).  Measured on 128x0e+128x1o+128x2e x S
+// species, 50 000 rows, against the kernels these shapes took with a limit of 64 blocks: S = 6 (96 blocks) 0.78 against
+// 1.10 ms in fp32 and 0.58 against 2.37 ms in bf16 storage, S = 8 (128 blocks) 1.04 against 1.33 and 0.72 against 2.84 ms.
+int node_max_blocks() { return env_int("E3X_NODE_MAX_BLOCKS", 144); }
 
 bool uvw_node_eligible(const e3x_plan& P) {
   if (!P.shared_weights || P.paths.empty() || env_int("E3X_UVW_NODE", 1) == 0) return false;
@@ -676,7 +678,7 @@ bool uvw_node_eligible(const e3x_plan& P) {
     blocks[p.out] += a.mul / 8 * b.mul;
     pairs += (long long)a.mul * b.mul;
   }
-  for (int n : blocks) if (n > kNodeMaxBlocks) return false;
+  for (int n : blocks) if (n > node_max_blocks()) return false;
   // a handful of (u, v) pairs in shapes the other matrix-core kernel does not take: the vector-ALU kernel keeps the
   // weights in registers and needs no padding to 32 channels
   // (the same choice in both storages: the tiling rule asked is the fp32 kernel's)

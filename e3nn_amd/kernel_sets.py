@@ -74,6 +74,11 @@ def node_fctp():
     return o3.FullyConnectedTensorProduct("128x0e+64x1o+32x2e", "4x0e", "128x0e+64x1o+96x2e")
 
 
+def node_many_species():
+    # six species at 128 channels: 96 weight blocks per target, more than half of the LDS (one workgroup per CU)
+    return o3.FullyConnectedTensorProduct("128x0e+64x1o", "6x0e", "64x0e+32x1o")
+
+
 def node_block():
     # a node-wise layer of an interaction block at NequIP-like width: 32 channels out, 4 species (the weight-gradient
     # kernel puts two species side by side in the 64 columns of a tile)
@@ -179,6 +184,7 @@ def all_tensor_products():
         ("wide_k_full_tiles", wide_k_full_tiles(), (torch.float32,)),
         ("outer_split", outer_split(), (torch.float32,)),
         ("node_block", node_block(), (torch.float32,)),
+        ("node_many_species", node_many_species(), (torch.float32, torch.bfloat16)),
         ("node_wide_out", node_wide_out(), (torch.float32, torch.bfloat16)),
         ("node_narrow", node_narrow(), (torch.float32, torch.bfloat16)),
         ("node_partial_tile", node_partial_tile(), (torch.float32, torch.bfloat16)),

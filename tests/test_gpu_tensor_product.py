@@ -188,7 +188,7 @@ def _fan_in_weights(tp, seed=0):
      # rows, and below one wave
      (ks.node_fctp, 333, "uvw_node"), (ks.node_fctp, 17, "uvw_node"), (ks.node_fctp, 1280, "uvw_node"),
      (ks.radial_layer, 1000, "uvw_node"), (ks.node_block, 200, "uvw_node"), (ks.node_wide_out, 77, "uvw_node"), (ks.node_narrow, 301, "uvw_node"),
-     (ks.node_partial_tile, 129, "uvw_node")],
+     (ks.node_partial_tile, 129, "uvw_node"), (ks.node_many_species, 260, "uvw_node")],
 )  # fmt: skip
 def test_uvw_matrix_core_kernel_against_oracle(maker, Z, family):
     tp = maker().to(DEV)
@@ -202,7 +202,8 @@ def test_uvw_matrix_core_kernel_against_oracle(maker, Z, family):
     assert_close(out, ref, what=str(tp))
 
 
-@pytest.mark.parametrize("maker,Z", [(ks.node_fctp, 333), (ks.node_fctp, 1), (ks.node_wide_out, 130), (ks.node_narrow, 301), (ks.node_partial_tile, 257)])
+@pytest.mark.parametrize("maker,Z", [(ks.node_fctp, 333), (ks.node_fctp, 1), (ks.node_wide_out, 130), (ks.node_narrow, 301), (ks.node_partial_tile, 257),
+                                     (ks.node_many_species, 140)])  # fmt: skip
 def test_node_wise_kernel_in_bf16_storage_against_oracle(maker, Z):
     # rows, scalars and weights stored as bf16 (8-byte pieces; weight rows element by element where the channel
     # counts are no multiples of 4), fp32 matrix instructions on the converted values, one rounding of the output
